@@ -1,0 +1,228 @@
+"""TEST INFRASTRUCTURE -- Python face of the CPU oracles.
+
+* plan oracle: ctypes binding of oracle/plan_oracle.cpp (restatement of
+  ROF/reuse_search_ext/src/reuse_search_ext.h); `ref_plan` runs the upstream builder itself
+  when oracle/_ref holds it (built by `make -C oracle ref` from the upstream sources in place).
+* aggregation oracle: float64 closed forms (numpy/scipy) and the fp32 kernel restatements of
+  oracle/agg_oracle.c (ROF/reuse_conv/reuse_conv_kernel.cu:205-286, 396-601, 836-954, 123-196).
+
+Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg may import this module.
+"""
+from __future__ import annotations
+
+import contextlib
+import ctypes as C
+import glob
+import os
+import sys
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = None
+
+PLAN_ARRAYS = (
+    "part_ptr", "part2Node", "num_parts_per_node_acc", "intersect_ptr", "intersect_data", "intersect_count",
+    "index_ordered", "index_picked", "new_indices_src", "part_pointers_cache", "column_index_cache",
+    "part_cache_flagindex", "uniqpart_column_index", "uniqpart_pointers", "part2Node_ptr", "part2Node_col",
+)
+
+
+def lib():
+    global _LIB
+    if _LIB is None:
+        path = os.path.join(_HERE, "liboracle.so")
+        if not os.path.exists(path):
+            raise RuntimeError("oracle/liboracle.so is not built: run `make -C oracle`")
+        L = C.CDLL(path)
+        L.orc_plan_build.restype = C.c_void_p
+        L.orc_plan_build.argtypes = [C.c_void_p] * 4 + [C.c_uint32, C.c_uint32, C.c_int, C.c_int]
+        L.orc_plan_array.restype = C.c_int64
+        L.orc_plan_array.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p]
+        L.orc_plan_free.argtypes = [C.c_void_p]
+        L.orc_transpose_csr.argtypes = [C.c_void_p, C.c_void_p, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]
+        L.orc_rsqrt_rn.restype = C.c_float
+        L.orc_rsqrt_rn.argtypes = [C.c_float]
+        _LIB = L
+    return _LIB
+
+
+def _u32(a):
+    return np.ascontiguousarray(np.asarray(a).astype(np.uint32, copy=False))
+
+
+def _i32(a):
+    return np.ascontiguousarray(np.asarray(a).astype(np.int32, copy=False))
+
+
+def _f32(a):
+    return np.ascontiguousarray(np.asarray(a, dtype=np.float32))
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+# --------------------------------------------------------------------------- plan
+def oracle_plan(indptr_dst, indices_src, part_size, indptr_src=None, indices_dst=None, discard=True):
+    """All plan arrays (dict of uint32 arrays) from the restated algorithm.  For a symmetric graph
+    the out-neighbour CSR equals the in-neighbour CSR (ROF_main.py:62-64) and may be omitted."""
+    ipd, isrc = _u32(indptr_dst), _u32(indices_src)
+    ips = ipd if indptr_src is None else _u32(indptr_src)
+    idst = isrc if indices_dst is None else _u32(indices_dst)
+    L = lib()
+    h = L.orc_plan_build(_p(ipd), _p(isrc), _p(ips), _p(idst), len(ipd) - 1, len(isrc), int(part_size), int(discard))
+    out = {}
+    try:
+        for name in PLAN_ARRAYS:
+            n = L.orc_plan_array(h, name.encode(), None)
+            a = np.empty(n, dtype=np.uint32)
+            L.orc_plan_array(h, name.encode(), _p(a))
+            out[name] = a
+    finally:
+        L.orc_plan_free(h)
+    return out
+
+
+def oracle_transpose_csr(indptr, indices):
+    ip, ix = _u32(indptr), _u32(indices)
+    op = np.empty_like(ip)
+    ox = np.empty_like(ix)
+    lib().orc_transpose_csr(_p(ip), _p(ix), len(ip) - 1, len(ix), _p(op), _p(ox))
+    return op, ox
+
+
+def ref_module():
+    """The upstream pybind module compiled from the upstream sources, or None if not built."""
+    d = os.path.join(_HERE, "_ref")
+    if not glob.glob(os.path.join(d, "reuse_search_ext*.so")):
+        return None
+    if d not in sys.path:
+        sys.path.insert(0, d)
+    import reuse_search_ext  # noqa: the upstream module name
+    return reuse_search_ext
+
+
+@contextlib.contextmanager
+def _quiet():
+    """The upstream builder prints progress to stdout from C++ (h:86-115 and others)."""
+    sys.stdout.flush()
+    old = os.dup(1)
+    null = os.open(os.devnull, os.O_WRONLY)
+    os.dup2(null, 1)
+    try:
+        yield
+    finally:
+        os.dup2(old, 1)
+        os.close(null)
+        os.close(old)
+
+
+def ref_plan(indptr_dst, indices_src, part_size, indptr_src=None, indices_dst=None, discard=True):
+    """Same dict as oracle_plan, produced by the upstream code through the call sequence of
+    ROF_evaluation/ROF_main.py:71-127.  Needs >= 9 nodes: upstream split_part prints
+    indptr_dst[0..9] unconditionally (h:91-94)."""
+    R = ref_module()
+    if R is None:
+        raise RuntimeError("oracle/_ref is not built")
+    ipd, isrc = _u32(indptr_dst), _u32(indices_src)
+    assert len(ipd) >= 10
+    ips = ipd if indptr_src is None else _u32(indptr_src)
+    idst = isrc if indices_dst is None else _u32(indices_dst)
+    e = np.empty(0, dtype=np.uint32)
+    with _quiet():
+        pp, p2n, acc = R.py_split_part(e, e.copy(), ipd, part_size)
+        ilist, cnt = R.py_get_part_intersect(pp, isrc, ips, idst, part_size, bool(discard))
+        ordered, picked = R.py_greedy_max_reuse(cnt, pp, isrc)
+        new_idx, _, cptr, ccol, flag = R.py_reorganize_indices(pp, isrc, ilist, picked, ipd, acc, part_size)
+        ucol, uptr, dptr, dcol = R.py_reorganize_indices_uniquely(pp, isrc, ilist, picked, ipd, acc, part_size)
+    iptr = np.zeros(len(ilist) + 1, dtype=np.uint32)
+    np.cumsum([len(a) for a in ilist], out=iptr[1:])
+    idata = np.concatenate([np.asarray(a, dtype=np.uint32) for a in ilist]) if len(ilist) else e
+    return {
+        "part_ptr": pp, "part2Node": p2n, "num_parts_per_node_acc": acc, "intersect_ptr": iptr,
+        "intersect_data": idata.astype(np.uint32), "intersect_count": np.asarray(cnt[0], dtype=np.uint32),
+        "index_ordered": ordered, "index_picked": picked, "new_indices_src": new_idx,
+        "part_pointers_cache": cptr, "column_index_cache": ccol, "part_cache_flagindex": flag,
+        "uniqpart_column_index": ucol, "uniqpart_pointers": uptr, "part2Node_ptr": dptr, "part2Node_col": dcol,
+    }
+
+
+# --------------------------------------------------------------------------- aggregation
+def rsqrt_rn(deg):
+    """Correctly rounded fp32 1/sqrt, the value of __frsqrt_rn (cu:254)."""
+    return (1.0 / np.sqrt(np.asarray(deg, dtype=np.float64))).astype(np.float32)
+
+
+def closed_form(indptr, indices, x, deg=None, normalized=True):
+    """float64 D^-1/2 A D^-1/2 x (normalized) or A x, A taken row = destination (SURVEY fact F2:
+    out[v] = rs(deg v) * sum_{u in row v} rs(deg u) x[u], cu:254,270,276,282)."""
+    import scipy.sparse as sp
+
+    n = len(indptr) - 1
+    a = sp.csr_matrix((np.ones(len(indices), dtype=np.float64), np.asarray(indices), np.asarray(indptr)), shape=(n, n))
+    x64 = np.asarray(x, dtype=np.float64)
+    if not normalized:
+        return a @ x64
+    d = np.diff(indptr).astype(np.float32) if deg is None else np.asarray(deg, dtype=np.float32)
+    with np.errstate(divide="ignore"):
+        r = 1.0 / np.sqrt(d.astype(np.float64))
+    y = a @ (x64 * np.where(np.isfinite(r), r, 0.0)[:, None])
+    return y * r[:, None]
+
+
+def _agg_sig():
+    L = lib()
+    if getattr(L, "_agg_ready", False):
+        return L
+    vp, i64, i = C.c_void_p, C.c_int64, C.c_int
+    L.orc_agg_parts.argtypes = [vp, i64, vp, vp, vp, vp, i, i, i, vp, i64]
+    L.orc_agg_v1.argtypes = [vp, i64, vp, vp, vp, vp, i, i, vp, vp, vp, vp, i, vp, i64]
+    L.orc_agg_v2.argtypes = [vp, i64, vp, vp, vp, vp, vp, i, i, i, vp, i64]
+    L.orc_spmm_rows.argtypes = [vp, i64, vp, vp, vp, i, i, i, vp, i64]
+    L._agg_ready = True
+    return L
+
+
+def agg_parts(x, deg, column_index, part_pointers, part2node, normalized=True):
+    """fp32 GNNA kernel (cu:205-286) / SAG kernel when normalized=False (cu:123-196)."""
+    x, deg = _f32(x), _f32(deg)
+    col, pp, p2n = _i32(column_index), _i32(part_pointers), _i32(part2node)
+    out = np.zeros_like(x)
+    _agg_sig().orc_agg_parts(_p(x), x.shape[1], _p(deg), _p(col), _p(pp), _p(p2n), len(p2n), x.shape[1],
+                             int(normalized), _p(out), x.shape[1])
+    return out
+
+
+def agg_v1(x, deg, column_index, part_pointers, part2node, flag, cache_ptr, cache_col):
+    """fp32 caching + reusing kernels (cu:396-601).  Returns (out, cache[cache_num, dim+1])."""
+    x, deg = _f32(x), _f32(deg)
+    col, pp, p2n = _i32(column_index), _i32(part_pointers), _i32(part2node)
+    fl, cp, cc = _i32(flag), _i32(cache_ptr), _i32(cache_col)
+    out = np.zeros_like(x)
+    cache = np.zeros((len(cp) - 1, x.shape[1] + 1), dtype=np.float32)
+    _agg_sig().orc_agg_v1(_p(x), x.shape[1], _p(deg), _p(col), _p(pp), _p(p2n), len(p2n), x.shape[1], _p(cache),
+                          _p(fl), _p(cp), _p(cc), len(cp) - 1, _p(out), x.shape[1])
+    return out, cache
+
+
+def agg_v2(x, deg, uniq_col, uniq_ptr, dst_ptr, dst_col, normalized=True):
+    """fp32 fused kernel (cu:836-954)."""
+    x, deg = _f32(x), _f32(deg)
+    uc, up, dp, dc = _i32(uniq_col), _i32(uniq_ptr), _i32(dst_ptr), _i32(dst_col)
+    out = np.zeros_like(x)
+    _agg_sig().orc_agg_v2(_p(x), x.shape[1], _p(deg), _p(uc), _p(up), _p(dp), _p(dc), len(up) - 1, x.shape[1],
+                          int(normalized), _p(out), x.shape[1])
+    return out
+
+
+def spmm_rows(x, deg_rs, indptr, indices, normalized=True, out=None):
+    """Destination-parallel CPU SpMM over all host threads: the cpu_baseline leg."""
+    x = _f32(x)
+    ip, ix = _i32(indptr), _i32(indices)
+    drs = _f32(deg_rs)
+    if out is None:
+        out = np.empty_like(x)
+    _agg_sig().orc_spmm_rows(_p(x), x.shape[1], _p(drs), _p(ip), _p(ix), len(ip) - 1, x.shape[1], int(normalized),
+                             _p(out), x.shape[1])
+    return out
