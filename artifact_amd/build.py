@@ -1,0 +1,56 @@
+"""Compile librof.so (gfx950 kernels + host code) in-tree with hipcc / g++.
+
+    python -m artifact_amd.build
+
+hipcc cross-compiles for gfx950 without a GPU.  The library is loaded with ctypes
+(artifact_amd/_lib.py); nothing here links against PyTorch.
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "librof.so")
+
+HOST_SOURCES = ["plan_builder.cpp", "layout.cpp"]
+HIP_SOURCES = ["agg_kernels.hip"]
+
+# packed fp32 instructions stay off: the compiler must not form v_pk_{add,mul,fma}_f32
+HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang",
+             "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
+HOST_FLAGS = ["-O3", "-std=c++17", "-fPIC", "-fopenmp", "-Wall"]
+
+
+def _run(cmd):
+    print("+", " ".join(cmd), flush=True)
+    subprocess.run(cmd, check=True)
+
+
+def build_library(verbose=True):
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    gxx = shutil.which("g++") or "g++"
+    inc = ["-I" + os.path.join(ROOT, "include"), "-I" + CSRC]
+    objdir = os.path.join(HERE, "build")
+    os.makedirs(objdir, exist_ok=True)
+    objs = []
+    for s in HOST_SOURCES:
+        o = os.path.join(objdir, s + ".o")
+        _run([gxx] + HOST_FLAGS + inc + ["-c", os.path.join(CSRC, s), "-o", o])
+        objs.append(o)
+    for s in HIP_SOURCES:
+        o = os.path.join(objdir, s + ".o")
+        _run([hipcc] + HIP_FLAGS + inc + ["-c", os.path.join(CSRC, s), "-o", o])
+        objs.append(o)
+    _run([hipcc, "-shared", "-fPIC", "-o", LIB] + objs + ["-fopenmp", "-lgomp"])
+    return LIB
+
+
+if __name__ == "__main__":
+    build_library()
+    print("built", LIB)
+    sys.exit(0)

@@ -1,0 +1,488 @@
+// gfx950 (CDNA4, wave64) kernels of the reuse-aware neighbour aggregation and their launchers.
+//
+// One kernel template does all the summing.  A *task* gathers a list of rows and writes their
+// weighted sum to one output row:
+//     out[task_out[t], :] = scale[t] * sum_i w[i] * row(col[i])        i in task_ptr[t] .. task_ptr[t+1]
+// where row(c) is x[c, :] for c < nsplit and the partial-sum row part[c - nsplit, :] otherwise
+// (the first task_nref[t] entries of a task are of the second kind).  Launch 1 fills the
+// partial-sum rows (reuse groups that several destinations share, segments of very long rows),
+// launch 2 produces every destination row.  There are no atomics: each output row has one writer.
+//
+// Mapping to the machine:
+//   * the feature dimension runs across lanes, VEC consecutive elements per lane (one 16-byte
+//     load), LPR lanes per row, so a wavefront gathers G = 64/LPR rows per load instruction and a
+//     row is read as one contiguous 16*LPR-byte burst;
+//   * long tasks get a whole wavefront: its G lane groups take every G-th entry and are combined
+//     at the end by a cross-lane butterfly (__shfl_xor -> DPP / ds_swizzle class instructions);
+//   * short tasks are packed G to a wavefront, one lane group each; they are pre-sorted by length
+//     so the groups of one wavefront finish together;
+//   * column ids and weights are fetched coalesced, one per lane, and handed to the lane groups
+//     with ds_bpermute, so the only per-entry memory instruction is the row gather itself;
+//   * workgroups are renumbered so that each XCD (own L2) works on runs of consecutive tasks.
+// MFMA is not used: there is no dense contraction here, only gather + add, bounded by HBM.
+//
+// Reference semantics: ROF/reuse_conv/reuse_conv_kernel.cu:205-286 (GNNA), 396-601 (v1),
+// 836-954 (v2 fused), 123-196 (SAG).
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <new>
+
+#include "rof.h"
+#include "rof_internal.h"
+
+namespace {
+
+thread_local char g_dev_err[256] = "";
+
+#define HIP_TRY(expr)                                                                  \
+    do {                                                                               \
+        hipError_t e_ = (expr);                                                        \
+        if (e_ != hipSuccess) {                                                        \
+            rof_set_device_error(#expr, hipGetErrorString(e_));                        \
+            return ROF_ERR_DEVICE;                                                     \
+        }                                                                              \
+    } while (0)
+
+struct AggArgs {
+    const void *x;         // feature rows
+    int64_t ldx;
+    const float *part;     // partial-sum rows (ids >= nsplit)
+    int64_t ldp;
+    int32_t nsplit;
+    const int32_t *task_ptr, *task_nref, *task_out;
+    const float *task_scale;   // null: no scaling
+    const int32_t *col;
+    const float *w;            // null: unweighted
+    float *out;
+    int64_t ldo;
+    int32_t feat;
+    int32_t n_wave, n_tasks;
+    int32_t n_blocks;          // logical workgroups
+    int32_t xcd_run;           // consecutive logical workgroups kept on one XCD
+    int32_t vec_store;         // output rows allow aligned 16-byte stores
+};
+
+constexpr int kWavesPerBlock = 4;
+constexpr int kXcds = 8;
+
+template <typename XT, int VEC>
+struct RowLoad;
+
+template <>
+struct RowLoad<float, 4> {
+    static __device__ __forceinline__ void load(const float *p, float (&v)[4]) {
+        float4 t = *reinterpret_cast<const float4 *>(p);
+        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+    }
+};
+template <>
+struct RowLoad<float, 8> {
+    static __device__ __forceinline__ void load(const float *p, float (&v)[8]) {
+        float4 t = *reinterpret_cast<const float4 *>(p);
+        float4 u = *reinterpret_cast<const float4 *>(p + 4);
+        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+        v[4] = u.x; v[5] = u.y; v[6] = u.z; v[7] = u.w;
+    }
+};
+template <>
+struct RowLoad<float, 1> {
+    static __device__ __forceinline__ void load(const float *p, float (&v)[1]) { v[0] = *p; }
+};
+// bf16 is the upper half of an fp32
+template <>
+struct RowLoad<uint16_t, 8> {
+    static __device__ __forceinline__ void load(const uint16_t *p, float (&v)[8]) {
+        uint4 t = *reinterpret_cast<const uint4 *>(p);
+        v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u);
+        v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
+        v[4] = __uint_as_float(t.z << 16); v[5] = __uint_as_float(t.z & 0xffff0000u);
+        v[6] = __uint_as_float(t.w << 16); v[7] = __uint_as_float(t.w & 0xffff0000u);
+    }
+};
+template <>
+struct RowLoad<uint16_t, 1> {
+    static __device__ __forceinline__ void load(const uint16_t *p, float (&v)[1]) {
+        v[0] = __uint_as_float(((uint32_t)*p) << 16);
+    }
+};
+
+// Sum the entries [beg, end) of one task into acc.  WAVE: all lane groups of the wavefront share
+// the task (beg/end wave-uniform) and take every G-th entry; otherwise each lane group owns its
+// task.  ST is the element type of the source rows, `base`/`ld` its address and row stride, `bias`
+// is subtracted from the column id.
+template <typename ST, int VEC, int LPR, bool WAVE>
+__device__ __forceinline__ void gather_sum(const ST *__restrict__ src, int64_t ld, int32_t bias,
+                                           const int32_t *__restrict__ col, const float *__restrict__ w,
+                                           int32_t beg, int32_t end, int lane, int sub, int li, int cbase, bool act,
+                                           float (&acc)[VEC]) {
+    constexpr int G = 64 / LPR;
+    constexpr int U = LPR >= 4 ? 4 : LPR;
+    constexpr int CH = WAVE ? 64 : LPR;     // entries fetched per step by the wave / by the lane group
+    for (int32_t base = beg; __any(base < end); base += CH) {
+        const int32_t mine = base + (WAVE ? lane : li);
+        int32_t mycol = 0;
+        float myw = 1.0f;
+        if (mine < end) {
+            mycol = col[mine];
+            if (w) myw = w[mine];
+        }
+#pragma unroll
+        for (int j0 = 0; j0 < LPR; j0 += U) {
+            const int first = WAVE ? j0 * G + sub : j0;
+            if (!__any(base + first < end)) break;
+            int32_t c[U];
+            float wt[U];
+            bool ok[U];
+            float v[U][VEC];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int slot = WAVE ? (j0 + u) * G + sub : (j0 + u);          // entry of the chunk
+                const int from = WAVE ? slot : sub * LPR + slot;                // lane that fetched it
+                c[u] = __shfl(mycol, from);
+                wt[u] = __shfl(myw, from);
+                ok[u] = act && (base + slot < end);
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (ok[u]) RowLoad<ST, VEC>::load(src + (int64_t)(c[u] - bias) * ld + cbase, v[u]);
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (ok[u]) {
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) acc[k] = fmaf(wt[u], v[u][k], acc[k]);
+                }
+        }
+    }
+}
+
+template <typename XT, int VEC, int LPR>
+__global__ __launch_bounds__(256) void rof_rows_kernel(AggArgs a) {
+    constexpr int G = 64 / LPR;
+    // XCD-aware renumbering: the hardware deals workgroup ids round-robin to the 8 XCDs; give each
+    // XCD runs of `xcd_run` consecutive logical workgroups instead of every 8th one.
+    const int hw = blockIdx.x;
+    const int xcd = hw % kXcds, nth = hw / kXcds;
+    const int run = a.xcd_run;
+    const int logical = ((nth / run) * kXcds + xcd) * run + (nth % run);
+    if (logical >= a.n_blocks) return;
+
+    const int lane = threadIdx.x & 63;
+    const int sub = lane / LPR, li = lane % LPR;
+    const int gw = logical * kWavesPerBlock + (threadIdx.x >> 6);
+    const XT *x = reinterpret_cast<const XT *>(a.x);
+
+    int32_t t, beg = 0, end = 0, mid = 0;
+    bool valid;
+    const bool wave_mode = gw < a.n_wave;
+    if (wave_mode) {
+        t = gw;
+        valid = true;
+    } else {
+        t = a.n_wave + (gw - a.n_wave) * G + sub;
+        valid = t < a.n_tasks;
+    }
+    if (valid) {
+        beg = a.task_ptr[t];
+        end = a.task_ptr[t + 1];
+        mid = beg + a.task_nref[t];
+    }
+
+    for (int c0 = 0; c0 < a.feat; c0 += LPR * VEC) {
+        const int cbase = c0 + li * VEC;
+        const bool act = cbase < a.feat;
+        float acc[VEC];
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) acc[k] = 0.0f;
+
+        if (wave_mode) {
+            if (mid > beg)
+                gather_sum<float, VEC, LPR, true>(a.part, a.ldp, a.nsplit, a.col, a.w, beg, mid, lane, sub, li, cbase,
+                                                  act, acc);
+            gather_sum<XT, VEC, LPR, true>(x, a.ldx, 0, a.col, a.w, mid, end, lane, sub, li, cbase, act, acc);
+#pragma unroll
+            for (int off = LPR; off < 64; off <<= 1) {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) acc[k] += __shfl_xor(acc[k], off);
+            }
+        } else {
+            if (__any(mid > beg))
+                gather_sum<float, VEC, LPR, false>(a.part, a.ldp, a.nsplit, a.col, a.w, beg, mid, lane, sub, li, cbase,
+                                                   act, acc);
+            gather_sum<XT, VEC, LPR, false>(x, a.ldx, 0, a.col, a.w, mid, end, lane, sub, li, cbase, act, acc);
+        }
+
+        const bool writer = valid && act && (!wave_mode || sub == 0);
+        if (writer) {
+            // an empty task writes zeros whatever its scale is (a node without in-edges keeps the
+            // zero-initialised output upstream: reuse_conv_kernel.cu:303)
+            float s = 1.0f;
+            if (a.task_scale && end > beg) s = a.task_scale[t];
+            float *o = a.out + (int64_t)a.task_out[t] * a.ldo + cbase;
+            if (VEC >= 4 && a.vec_store && cbase + VEC <= a.feat) {
+#pragma unroll
+                for (int k = 0; k < VEC; k += 4)
+                    *reinterpret_cast<float4 *>(o + k) =
+                        make_float4(acc[k] * s, acc[k + 1] * s, acc[k + 2] * s, acc[k + 3] * s);
+            } else {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k)
+                    if (cbase + k < a.feat) o[k] = acc[k] * s;
+            }
+        }
+    }
+}
+
+// rsqrt of the in-degree, correctly rounded like __frsqrt_rn (reuse_conv_kernel.cu:254,276)
+__device__ __forceinline__ float rsqrt_rn(float d) { return (float)(1.0 / sqrt((double)d)); }
+
+__global__ void rof_entry_weights_kernel(const int32_t *__restrict__ col, int64_t m, const float *__restrict__ deg,
+                                         int32_t nsplit, float *__restrict__ w) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < m) {
+        int32_t c = col[i];
+        w[i] = c < nsplit ? rsqrt_rn(deg[c]) : 1.0f;
+    }
+}
+
+__global__ void rof_task_scale_kernel(const int32_t *__restrict__ task_out, int32_t T, const float *__restrict__ deg,
+                                      float *__restrict__ scale) {
+    int32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < T) scale[i] = rsqrt_rn(deg[task_out[i]]);
+}
+
+template <typename XT, int VEC>
+int launch_lpr(const AggArgs &a0, int lpr, hipStream_t st) {
+    AggArgs a = a0;
+    const int g = 64 / lpr;
+    const int64_t shorts = (int64_t)a.n_tasks - a.n_wave;
+    const int64_t waves = a.n_wave + (shorts + g - 1) / g;
+    if (waves == 0) return ROF_OK;
+    a.n_blocks = (int32_t)((waves + kWavesPerBlock - 1) / kWavesPerBlock);
+    const int64_t span = (int64_t)kXcds * a.xcd_run;
+    const int64_t grid = (a.n_blocks + span - 1) / span * span;
+    dim3 gr((unsigned)grid), bl(64 * kWavesPerBlock);
+    switch (lpr) {
+        case 4: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 4>), gr, bl, 0, st, a); break;
+        case 8: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 8>), gr, bl, 0, st, a); break;
+        case 16: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 16>), gr, bl, 0, st, a); break;
+        case 32: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 32>), gr, bl, 0, st, a); break;
+        default: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 64>), gr, bl, 0, st, a); break;
+    }
+    HIP_TRY(hipGetLastError());
+    return ROF_OK;
+}
+
+int launch_phase(const AggArgs &a, int dtype, int vec, hipStream_t st) {
+    int need = (a.feat + vec - 1) / vec, lpr = 4;
+    while (lpr < need && lpr < 64) lpr <<= 1;
+    if (dtype == ROF_F32) return vec == 4 ? launch_lpr<float, 4>(a, lpr, st) : launch_lpr<float, 1>(a, lpr, st);
+    return vec == 8 ? launch_lpr<uint16_t, 8>(a, lpr, st) : launch_lpr<uint16_t, 1>(a, lpr, st);
+}
+
+int upload_phase(const rof_phase_host &h, rof_phase_dev &d, bool with_scale, hipStream_t st, int64_t *bytes) {
+    d.n_wave = h.n_wave;
+    d.n_tasks = h.n_tasks;
+    d.n_entries = (int64_t)h.col.size();
+    auto put = [&](int32_t **dst, const std::vector<int32_t> &src) -> int {
+        size_t nb = (src.size() ? src.size() : 1) * sizeof(int32_t);
+        HIP_TRY(hipMalloc((void **)dst, nb));
+        *bytes += (int64_t)nb;
+        if (!src.empty()) HIP_TRY(hipMemcpyAsync(*dst, src.data(), src.size() * sizeof(int32_t), hipMemcpyHostToDevice, st));
+        return ROF_OK;
+    };
+    int rc;
+    if ((rc = put(&d.task_ptr, h.task_ptr))) return rc;
+    if ((rc = put(&d.task_nref, h.task_nref))) return rc;
+    if ((rc = put(&d.task_out, h.task_out))) return rc;
+    if ((rc = put(&d.col, h.col))) return rc;
+    size_t wb = (h.col.size() ? h.col.size() : 1) * sizeof(float);
+    HIP_TRY(hipMalloc((void **)&d.w, wb));
+    *bytes += (int64_t)wb;
+    if (with_scale) {
+        size_t sb = (size_t)(h.n_tasks ? h.n_tasks : 1) * sizeof(float);
+        HIP_TRY(hipMalloc((void **)&d.scale, sb));
+        *bytes += (int64_t)sb;
+    }
+    return ROF_OK;
+}
+
+void free_phase(rof_phase_dev &d) {
+    if (d.task_ptr) (void)hipFree(d.task_ptr);
+    if (d.task_nref) (void)hipFree(d.task_nref);
+    if (d.task_out) (void)hipFree(d.task_out);
+    if (d.col) (void)hipFree(d.col);
+    if (d.w) (void)hipFree(d.w);
+    if (d.scale) (void)hipFree(d.scale);
+    d = rof_phase_dev();
+}
+
+inline int64_t round_up(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
+
+int g_xcd_run_a = 1, g_xcd_run_b = 16;
+
+}  // namespace
+
+void rof_set_device_error(const char *what, const char *text) {
+    snprintf(g_dev_err, sizeof(g_dev_err), "%s: %s", what, text);
+}
+
+extern "C" {
+
+const char *rof_last_device_error(void) { return g_dev_err; }
+
+const char *rof_strerror(int status) {
+    switch (status) {
+        case ROF_OK: return "ok";
+        case ROF_ERR_ARG: return "invalid argument";
+        case ROF_ERR_RANGE: return "index out of range";
+        case ROF_ERR_ALLOC: return "allocation failed";
+        case ROF_ERR_DEVICE: return "HIP call failed";
+        case ROF_ERR_STATE: return "layout is not in the required state";
+        case ROF_ERR_UNSUPPORTED: return "unsupported size or type";
+        case ROF_ERR_WORKSPACE: return "workspace too small";
+        default: return "unknown status";
+    }
+}
+
+int rof_version(void) { return 1; }
+
+// Tuning knob used by the benchmark sweeps: consecutive workgroups per XCD for launch 1 / launch 2.
+int rof_set_xcd_run(int run_a, int run_b) {
+    if (run_a < 1 || run_b < 1 || run_a > 4096 || run_b > 4096) return ROF_ERR_ARG;
+    g_xcd_run_a = run_a;
+    g_xcd_run_b = run_b;
+    return ROF_OK;
+}
+
+int rof_layout_upload(rof_layout *L, void *stream) {
+    if (!L) return ROF_ERR_ARG;
+    if (L->uploaded) return ROF_OK;
+    hipStream_t st = (hipStream_t)stream;
+    HIP_TRY(hipGetDevice(&L->device));
+    int rc;
+    if ((rc = upload_phase(L->a, L->da, false, st, &L->device_bytes))) return rc;
+    if ((rc = upload_phase(L->b, L->db, true, st, &L->device_bytes))) return rc;
+    HIP_TRY(hipStreamSynchronize(st));   // the host vectors may be released after this call
+    L->uploaded = true;
+    return ROF_OK;
+}
+
+int rof_layout_set_degrees(rof_layout *L, const float *deg, void *stream) {
+    if (!L || !deg) return ROF_ERR_ARG;
+    if (!L->uploaded) return ROF_ERR_STATE;
+    hipStream_t st = (hipStream_t)stream;
+    const int tb = 256;
+    if (L->da.n_entries)
+        hipLaunchKernelGGL(rof_entry_weights_kernel, dim3((unsigned)((L->da.n_entries + tb - 1) / tb)), dim3(tb), 0, st,
+                           L->da.col, L->da.n_entries, deg, L->n, L->da.w);
+    if (L->db.n_entries)
+        hipLaunchKernelGGL(rof_entry_weights_kernel, dim3((unsigned)((L->db.n_entries + tb - 1) / tb)), dim3(tb), 0, st,
+                           L->db.col, L->db.n_entries, deg, L->n, L->db.w);
+    if (L->db.n_tasks)
+        hipLaunchKernelGGL(rof_task_scale_kernel, dim3((unsigned)((L->db.n_tasks + tb - 1) / tb)), dim3(tb), 0, st,
+                           L->db.task_out, L->db.n_tasks, deg, L->db.scale);
+    HIP_TRY(hipGetLastError());
+    L->weights_set = true;
+    return ROF_OK;
+}
+
+size_t rof_layout_workspace_bytes(const rof_layout *L, int feat_dim) {
+    if (!L || feat_dim < 1) return 0;
+    return (size_t)L->n_slots * (size_t)round_up(feat_dim, 8) * sizeof(float);
+}
+
+void rof_layout_free(rof_layout *L) {
+    if (!L) return;
+    if (L->uploaded) {
+        free_phase(L->da);
+        free_phase(L->db);
+    }
+    delete L;
+}
+
+int rof_aggregate(const rof_layout *L, const void *x, int x_dtype, int64_t ldx, float *out, int64_t ldo, int feat,
+                  int normalized, void *workspace, size_t workspace_bytes, void *stream) {
+    if (!L || !x || !out || feat < 1 || ldx < feat || ldo < feat) return ROF_ERR_ARG;
+    if (x_dtype != ROF_F32 && x_dtype != ROF_BF16) return ROF_ERR_UNSUPPORTED;
+    if (!L->uploaded || (normalized && !L->weights_set)) return ROF_ERR_STATE;
+    if ((int64_t)L->n * ldx >= ((int64_t)1 << 40) || (int64_t)L->n * ldo >= ((int64_t)1 << 40)) return ROF_ERR_UNSUPPORTED;
+    const size_t need = rof_layout_workspace_bytes(L, feat);
+    if (need && (!workspace || workspace_bytes < need)) return ROF_ERR_WORKSPACE;
+    if (need && ((uintptr_t)workspace & 15)) return ROF_ERR_ARG;
+    hipStream_t st = (hipStream_t)stream;
+
+    const int esz = x_dtype == ROF_F32 ? 4 : 2;
+    const int wide = x_dtype == ROF_F32 ? 4 : 8;
+    const bool aligned = (ldx % wide == 0) && (((uintptr_t)x) % 16 == 0);
+    const int vec = aligned ? wide : 1;
+    (void)esz;
+    const int64_t ldp = round_up(feat, 8);
+
+    AggArgs a;
+    memset(&a, 0, sizeof(a));
+    a.x = x;
+    a.ldx = ldx;
+    a.part = (const float *)workspace;
+    a.ldp = ldp;
+    a.nsplit = L->n;
+    a.feat = feat;
+    int rc;
+    if (L->da.n_tasks) {   // launch 1: partial-sum rows
+        a.task_ptr = L->da.task_ptr;
+        a.task_nref = L->da.task_nref;
+        a.task_out = L->da.task_out;
+        a.task_scale = nullptr;
+        a.col = L->da.col;
+        a.w = normalized ? L->da.w : nullptr;
+        a.out = (float *)workspace;
+        a.ldo = ldp;
+        a.n_wave = L->da.n_wave;
+        a.n_tasks = L->da.n_tasks;
+        a.xcd_run = g_xcd_run_a;
+        a.vec_store = 1;
+        if ((rc = launch_phase(a, x_dtype, vec, st))) return rc;
+    }
+    if (L->db.n_tasks) {   // launch 2: destination rows
+        a.task_ptr = L->db.task_ptr;
+        a.task_nref = L->db.task_nref;
+        a.task_out = L->db.task_out;
+        a.task_scale = normalized ? L->db.scale : nullptr;
+        a.col = L->db.col;
+        a.w = normalized ? L->db.w : nullptr;
+        a.out = out;
+        a.ldo = ldo;
+        a.n_wave = L->db.n_wave;
+        a.n_tasks = L->db.n_tasks;
+        a.xcd_run = g_xcd_run_b;
+        a.vec_store = (ldo % 4 == 0) && (((uintptr_t)out) % 16 == 0);
+        if ((rc = launch_phase(a, x_dtype, vec, st))) return rc;
+    }
+    return ROF_OK;
+}
+
+int rof_aggregate_timed(const rof_layout *L, const void *x, int x_dtype, int64_t ldx, float *out, int64_t ldo,
+                        int feat, int normalized, void *workspace, size_t workspace_bytes, void *stream, int iters,
+                        float *ms_per_call) {
+    if (!ms_per_call || iters < 1) return ROF_ERR_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    hipEvent_t e0, e1;
+    HIP_TRY(hipEventCreate(&e0));
+    HIP_TRY(hipEventCreate(&e1));
+    int rc = ROF_OK;
+    HIP_TRY(hipEventRecord(e0, st));
+    for (int i = 0; i < iters && rc == ROF_OK; ++i)
+        rc = rof_aggregate(L, x, x_dtype, ldx, out, ldo, feat, normalized, workspace, workspace_bytes, st);
+    HIP_TRY(hipEventRecord(e1, st));
+    HIP_TRY(hipEventSynchronize(e1));
+    float ms = 0.f;
+    HIP_TRY(hipEventElapsedTime(&ms, e0, e1));
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    *ms_per_call = ms / iters;
+    return rc;
+}
+
+}  // extern "C"

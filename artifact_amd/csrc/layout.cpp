@@ -1,0 +1,452 @@
+// Host side of the device layout: turns a plan in any of the three upstream tensor formats into
+//   (1) the canonical arrays -- a CSR of reuse groups with their consumers, and a destination-centric
+//       CSR of residual neighbours -- from which the upstream v2 tensors can be rebuilt bit for bit;
+//   (2) the execution schedule for the gfx950 kernels: every destination row becomes one task whose
+//       entries are either feature-row ids or "virtual" ids >= N naming a partial-sum row; groups that
+//       are worth sharing and segments of very long rows become tasks of a first launch that fills those
+//       partial-sum rows.  Tasks are ordered long-to-short, short ones tile by tile, so that the lanes
+//       of a wavefront that share one launch slot do the same amount of work.
+#include <algorithm>
+#include <cstdint>
+#include <cstring>
+#include <new>
+#include <numeric>
+#include <vector>
+#include <omp.h>
+
+#include "rof.h"
+#include "rof_internal.h"
+
+namespace {
+
+typedef std::vector<int32_t> ivec;
+
+const int32_t kShortRow = 32;        // tasks up to this many entries share a wavefront
+const int32_t kHubSplitDefault = 2048;
+const int32_t kSegmentDefault = 512;
+const int32_t kTileRows = 4096;      // short tasks are length-sorted inside tiles of this many rows
+
+bool ptr_ok(const int32_t *p, int64_t n, int64_t *total) {
+    if (!p || p[0] != 0) return false;
+    for (int64_t i = 0; i < n; ++i)
+        if (p[i] > p[i + 1]) return false;
+    *total = p[n];
+    return true;
+}
+
+bool ids_ok(const int32_t *a, int64_t len, int64_t bound) {
+    bool ok = true;
+#pragma omp parallel for schedule(static) reduction(&& : ok)
+    for (int64_t i = 0; i < len; ++i)
+        if (a[i] < 0 || a[i] >= bound) ok = false;
+    return ok;
+}
+
+// Is the multi-consumer-first / node-ascending / part_size-chunked shape of the upstream v2 emitter
+// (reuse_search_ext.h:537-636) present?  Only then does the export reproduce the input exactly.
+bool v2_is_canonical(const int32_t *uptr, const int32_t *dptr, const int32_t *dcol, int64_t U, int ps, int64_t G) {
+    int64_t w = G;
+    while (w < U) {
+        int32_t node = dcol[dptr[w]];
+        if (w > G && dcol[dptr[w - 1]] >= node) return false;   // nodes strictly ascending across runs
+        int64_t run = w;
+        while (run < U && dcol[dptr[run]] == node) ++run;
+        for (int64_t q = w; q < run; ++q) {
+            int32_t len = uptr[q + 1] - uptr[q];
+            if (len < 1 || len > ps || (q + 1 < run && len != ps)) return false;
+        }
+        w = run;
+    }
+    return true;
+}
+
+struct TaskList {   // tasks in natural order, before sorting
+    ivec ptr{0}, nref, out, col;
+    void begin_task(int32_t out_row) { out.push_back(out_row); }
+    void end_task(int32_t refs) {
+        nref.push_back(refs);
+        ptr.push_back((int32_t)col.size());
+    }
+};
+
+// Long tasks first (descending), then short tasks tile by tile, each tile descending.
+void order_tasks(const ivec &ptr, int64_t tile_rows, ivec &order, int32_t &n_wave) {
+    int64_t T = (int64_t)ptr.size() - 1;
+    order.clear();
+    order.reserve(T);
+    ivec longs;
+    for (int64_t t = 0; t < T; ++t)
+        if (ptr[t + 1] - ptr[t] > kShortRow) longs.push_back((int32_t)t);
+    std::stable_sort(longs.begin(), longs.end(),
+                     [&ptr](int32_t x, int32_t y) { return ptr[x + 1] - ptr[x] > ptr[y + 1] - ptr[y]; });
+    n_wave = (int32_t)longs.size();
+    order = longs;
+    std::vector<ivec> bucket(kShortRow + 1);
+    for (int64_t t0 = 0; t0 < T; t0 += tile_rows) {
+        int64_t t1 = std::min(T, t0 + tile_rows);
+        for (auto &b : bucket) b.clear();
+        for (int64_t t = t0; t < t1; ++t) {
+            int32_t len = ptr[t + 1] - ptr[t];
+            if (len <= kShortRow) bucket[len].push_back((int32_t)t);
+        }
+        for (int32_t len = kShortRow; len >= 0; --len) order.insert(order.end(), bucket[len].begin(), bucket[len].end());
+    }
+}
+
+void finalize_phase(const TaskList &tl, int64_t tile_rows, rof_phase_host &ph) {
+    int64_t T = (int64_t)tl.out.size();
+    ivec order;
+    order_tasks(tl.ptr, tile_rows, order, ph.n_wave);
+    ph.n_tasks = (int32_t)T;
+    ph.task_ptr.assign(T + 1, 0);
+    ph.task_nref.resize(T);
+    ph.task_out.resize(T);
+    for (int64_t i = 0; i < T; ++i) {
+        int32_t t = order[i];
+        ph.task_ptr[i + 1] = ph.task_ptr[i] + (tl.ptr[t + 1] - tl.ptr[t]);
+        ph.task_nref[i] = tl.nref[t];
+        ph.task_out[i] = tl.out[t];
+    }
+    ph.col.resize(tl.col.size());
+#pragma omp parallel for schedule(dynamic, 4096)
+    for (int64_t i = 0; i < T; ++i) {
+        int32_t t = order[i];
+        int32_t len = tl.ptr[t + 1] - tl.ptr[t];
+        if (len) memcpy(ph.col.data() + ph.task_ptr[i], tl.col.data() + tl.ptr[t], (size_t)len * sizeof(int32_t));
+    }
+}
+
+int build_schedule(rof_layout *L, const rof_layout_opts *o) {
+    const int32_t n = L->n;
+    const int64_t G = (int64_t)L->group_ptr.size() - 1;
+    const int32_t hub_split = (o && o->hub_split > 0) ? o->hub_split : kHubSplitDefault;
+    const int32_t segment = (o && o->segment > 0) ? o->segment : kSegmentDefault;
+    const bool disable = o && o->disable_reuse;
+    const int32_t min_consumers = o ? o->min_consumers : 0;
+
+    // which groups are computed once and shared
+    std::vector<int32_t> slot_of(G, -1);
+    int64_t slots = 0;
+    for (int64_t g = 0; g < G; ++g) {
+        int64_t len = L->group_ptr[g + 1] - L->group_ptr[g];
+        int64_t cnt = L->group_dst_ptr[g + 1] - L->group_dst_ptr[g];
+        bool share;
+        if (disable) share = false;
+        else if (min_consumers < 0) share = true;   // every group, even one nobody consumes (v1 cache rows)
+        else if (min_consumers > 0) share = cnt >= min_consumers;
+        else share = (cnt - 1) * len > cnt + 1;   // row gathers saved > partial-row reads + the one write
+        if (share && (min_consumers < 0 || (len > 0 && cnt > 0))) slot_of[g] = (int32_t)slots++;
+    }
+    L->n_materialised = slots;
+
+    // node -> groups it consumes (ascending group index)
+    ivec ng_ptr((size_t)n + 1, 0), ng;
+    for (int64_t j = 0; j < (int64_t)L->group_dst.size(); ++j) ng_ptr[L->group_dst[j] + 1]++;
+    for (int32_t v = 0; v < n; ++v) ng_ptr[v + 1] += ng_ptr[v];
+    ng.resize(ng_ptr[n]);
+    {
+        ivec at(ng_ptr.begin(), ng_ptr.end() - 1);
+        for (int64_t g = 0; g < G; ++g)
+            for (int32_t j = L->group_dst_ptr[g]; j < L->group_dst_ptr[g + 1]; ++j) ng[at[L->group_dst[j]]++] = (int32_t)g;
+    }
+
+    TaskList ta, tb;
+    for (int64_t g = 0; g < G; ++g) {
+        if (slot_of[g] < 0) continue;
+        ta.begin_task(slot_of[g]);
+        ta.col.insert(ta.col.end(), L->group_col.begin() + L->group_ptr[g], L->group_col.begin() + L->group_ptr[g + 1]);
+        ta.end_task(0);
+    }
+    tb.ptr.reserve((size_t)n + 1);
+    tb.nref.reserve(n);
+    tb.out.reserve(n);
+    tb.col.reserve(L->res_col.size() + L->group_dst.size());
+    int64_t gathered = (int64_t)ta.col.size(), reads = 0, segments = 0;
+    ivec reals;
+    for (int32_t v = 0; v < n; ++v) {
+        tb.begin_task(v);
+        int32_t refs = 0;
+        reals.clear();
+        for (int32_t j = ng_ptr[v]; j < ng_ptr[v + 1]; ++j) {
+            int32_t g = ng[j];
+            if (slot_of[g] >= 0) {
+                tb.col.push_back(n + slot_of[g]);
+                ++refs;
+            } else {
+                reals.insert(reals.end(), L->group_col.begin() + L->group_ptr[g], L->group_col.begin() + L->group_ptr[g + 1]);
+            }
+        }
+        const int32_t *res = L->res_col.data() + L->res_ptr[v];
+        int64_t nres = L->res_ptr[v + 1] - L->res_ptr[v];
+        int64_t nreal = (int64_t)reals.size() + nres;
+        gathered += nreal;
+        if (nreal > hub_split) {
+            // cut the row's feature-row entries into segments; each becomes a partial-sum task
+            reals.insert(reals.end(), res, res + nres);
+            for (int64_t s0 = 0; s0 < nreal; s0 += segment) {
+                int64_t s1 = std::min<int64_t>(nreal, s0 + segment);
+                int32_t slot = (int32_t)slots++;
+                ta.begin_task(slot);
+                ta.col.insert(ta.col.end(), reals.begin() + s0, reals.begin() + s1);
+                ta.end_task(0);
+                tb.col.push_back(n + slot);
+                ++refs;
+                ++segments;
+            }
+        } else {
+            tb.col.insert(tb.col.end(), reals.begin(), reals.end());
+            tb.col.insert(tb.col.end(), res, res + nres);
+        }
+        reads += refs;
+        tb.end_task(refs);
+    }
+    if (slots + (int64_t)n >= INT32_MAX || tb.col.size() >= (size_t)INT32_MAX) return ROF_ERR_UNSUPPORTED;
+    L->n_slots = slots;
+    L->n_segments = segments;
+    L->gathered_rows = gathered;
+    L->partial_reads = reads;
+    finalize_phase(ta, 1 << 30, L->a);
+    finalize_phase(tb, kTileRows, L->b);
+    return ROF_OK;
+}
+
+rof_layout *new_layout(int32_t n, int ps) {
+    rof_layout *L = new (std::nothrow) rof_layout;
+    if (!L) return nullptr;
+    L->n = n;
+    L->part_size = ps;
+    return L;
+}
+
+// Build the canonical arrays from "unique parts": part w has sources src[sptr[w]..sptr[w+1]) and
+// consumers dcol[dptr[w]..dptr[w+1]).
+void canonical_from_unique(rof_layout *L, const int32_t *src, const int32_t *sptr, const int32_t *dptr,
+                           const int32_t *dcol, int64_t U) {
+    const int32_t n = L->n;
+    L->group_ptr.assign(1, 0);
+    L->group_dst_ptr.assign(1, 0);
+    L->res_ptr.assign((size_t)n + 1, 0);
+    int64_t e = 0;
+    for (int64_t w = 0; w < U; ++w) {
+        int32_t cnt = dptr[w + 1] - dptr[w], len = sptr[w + 1] - sptr[w];
+        e += (int64_t)cnt * len;
+        if (cnt >= 2) {
+            L->group_col.insert(L->group_col.end(), src + sptr[w], src + sptr[w + 1]);
+            L->group_ptr.push_back((int32_t)L->group_col.size());
+            L->group_dst.insert(L->group_dst.end(), dcol + dptr[w], dcol + dptr[w + 1]);
+            L->group_dst_ptr.push_back((int32_t)L->group_dst.size());
+        } else if (cnt == 1) {
+            L->res_ptr[dcol[dptr[w]] + 1] += len;
+        }
+    }
+    L->e_orig = e;
+    for (int32_t v = 0; v < n; ++v) L->res_ptr[v + 1] += L->res_ptr[v];
+    L->res_col.resize(L->res_ptr[n]);
+    ivec at(L->res_ptr.begin(), L->res_ptr.end() - 1);
+    for (int64_t w = 0; w < U; ++w) {
+        if (dptr[w + 1] - dptr[w] != 1) continue;
+        int32_t v = dcol[dptr[w]], len = sptr[w + 1] - sptr[w];
+        if (len) memcpy(L->res_col.data() + at[v], src + sptr[w], (size_t)len * sizeof(int32_t));
+        at[v] += len;
+    }
+}
+
+int finish(rof_layout *L, const rof_layout_opts *opts, rof_layout **out) {
+    int st = build_schedule(L, opts);
+    if (st) {
+        delete L;
+        return st;
+    }
+    *out = L;
+    return ROF_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int rof_layout_from_v2(const int32_t *ucol, const int32_t *uptr, const int32_t *dptr, const int32_t *dcol,
+                       int64_t U, int32_t n, int part_size, const rof_layout_opts *opts, rof_layout **out) {
+    if (!out || !uptr || !dptr || U < 0 || n < 0 || part_size < 1) return ROF_ERR_ARG;
+    int64_t ne = 0, nd = 0;
+    if (!ptr_ok(uptr, U, &ne) || !ptr_ok(dptr, U, &nd)) return ROF_ERR_RANGE;
+    if ((ne && !ucol) || (nd && !dcol)) return ROF_ERR_ARG;
+    if (!ids_ok(ucol, ne, n) || !ids_ok(dcol, nd, n)) return ROF_ERR_RANGE;
+    try {
+        rof_layout *L = new_layout(n, part_size);
+        if (!L) return ROF_ERR_ALLOC;
+        canonical_from_unique(L, ucol, uptr, dptr, dcol, U);
+        int64_t G = (int64_t)L->group_ptr.size() - 1;
+        bool groups_first = true;
+        for (int64_t w = 0; w < U && groups_first; ++w) {
+            int32_t cnt = dptr[w + 1] - dptr[w];
+            if ((w < G) != (cnt >= 2) || cnt == 0) groups_first = false;
+        }
+        L->canonical = groups_first && v2_is_canonical(uptr, dptr, dcol, U, part_size, G);
+        return finish(L, opts, out);
+    } catch (const std::bad_alloc &) {
+        return ROF_ERR_ALLOC;
+    }
+}
+
+int rof_layout_from_v1(const int32_t *col, const int32_t *pptr, const int32_t *p2n, int64_t parts, const int32_t *flag,
+                       const int32_t *cptr, const int32_t *ccol, int64_t cache_num, int32_t n, int part_size,
+                       const rof_layout_opts *opts, rof_layout **out) {
+    if (!out || !pptr || !cptr || parts < 0 || cache_num < 0 || n < 0 || part_size < 1) return ROF_ERR_ARG;
+    if (parts && (!p2n || !flag)) return ROF_ERR_ARG;
+    int64_t ne = 0, nc = 0;
+    if (!ptr_ok(pptr, parts, &ne) || !ptr_ok(cptr, cache_num, &nc)) return ROF_ERR_RANGE;
+    if ((ne && !col) || (nc && !ccol)) return ROF_ERR_ARG;
+    if (!ids_ok(col, ne, n) || !ids_ok(ccol, nc, n) || !ids_ok(p2n, parts, n)) return ROF_ERR_RANGE;
+    if (!ids_ok(flag, parts, cache_num + 1)) return ROF_ERR_RANGE;
+    try {
+        rof_layout *L = new_layout(n, part_size);
+        if (!L) return ROF_ERR_ALLOC;
+        // groups = cache rows (reuse_conv_kernel.cu:431-440); consumers = nodes of the flagged parts
+        // (cu:523-531), which come in ascending node order because part2Node is non-decreasing
+        L->group_ptr.assign(cptr, cptr + cache_num + 1);
+        L->group_col.assign(ccol, ccol + nc);
+        L->group_dst_ptr.assign((size_t)cache_num + 1, 0);
+        L->res_ptr.assign((size_t)n + 1, 0);
+        int64_t e = 0;
+        for (int64_t p = 0; p < parts; ++p) {
+            if (flag[p] > 0) {
+                L->group_dst_ptr[flag[p]]++;
+                e += cptr[flag[p]] - cptr[flag[p] - 1];
+            } else {
+                L->res_ptr[p2n[p] + 1] += pptr[p + 1] - pptr[p];
+                e += pptr[p + 1] - pptr[p];
+            }
+        }
+        L->e_orig = e;
+        for (int64_t g = 0; g < cache_num; ++g) L->group_dst_ptr[g + 1] += L->group_dst_ptr[g];
+        for (int32_t v = 0; v < n; ++v) L->res_ptr[v + 1] += L->res_ptr[v];
+        L->group_dst.resize(L->group_dst_ptr[cache_num]);
+        L->res_col.resize(L->res_ptr[n]);
+        ivec gat(L->group_dst_ptr.begin(), L->group_dst_ptr.end() - 1), rat(L->res_ptr.begin(), L->res_ptr.end() - 1);
+        for (int64_t p = 0; p < parts; ++p) {
+            if (flag[p] > 0) {
+                L->group_dst[gat[flag[p] - 1]++] = p2n[p];
+            } else {
+                int32_t len = pptr[p + 1] - pptr[p];
+                if (len) memcpy(L->res_col.data() + rat[p2n[p]], col + pptr[p], (size_t)len * sizeof(int32_t));
+                rat[p2n[p]] += len;
+            }
+        }
+        bool ok = true;   // canonical iff every cache row has >= 2 consumers
+        for (int64_t g = 0; g < cache_num; ++g)
+            if (L->group_dst_ptr[g + 1] - L->group_dst_ptr[g] < 2) ok = false;
+        L->canonical = ok;
+        return finish(L, opts, out);
+    } catch (const std::bad_alloc &) {
+        return ROF_ERR_ALLOC;
+    }
+}
+
+int rof_layout_from_parts(const int32_t *col, const int32_t *pptr, const int32_t *p2n, int64_t parts, int32_t n,
+                          int part_size, const rof_layout_opts *opts, rof_layout **out) {
+    if (!out || !pptr || parts < 0 || n < 0 || part_size < 1 || (parts && !p2n)) return ROF_ERR_ARG;
+    int64_t ne = 0;
+    if (!ptr_ok(pptr, parts, &ne)) return ROF_ERR_RANGE;
+    if (ne && !col) return ROF_ERR_ARG;
+    if (!ids_ok(col, ne, n) || !ids_ok(p2n, parts, n)) return ROF_ERR_RANGE;
+    try {
+        rof_layout *L = new_layout(n, part_size);
+        if (!L) return ROF_ERR_ALLOC;
+        L->group_ptr.assign(1, 0);
+        L->group_dst_ptr.assign(1, 0);
+        L->res_ptr.assign((size_t)n + 1, 0);
+        for (int64_t p = 0; p < parts; ++p) L->res_ptr[p2n[p] + 1] += pptr[p + 1] - pptr[p];
+        for (int32_t v = 0; v < n; ++v) L->res_ptr[v + 1] += L->res_ptr[v];
+        L->res_col.resize(L->res_ptr[n]);
+        ivec at(L->res_ptr.begin(), L->res_ptr.end() - 1);
+        for (int64_t p = 0; p < parts; ++p) {
+            int32_t len = pptr[p + 1] - pptr[p];
+            if (len) memcpy(L->res_col.data() + at[p2n[p]], col + pptr[p], (size_t)len * sizeof(int32_t));
+            at[p2n[p]] += len;
+        }
+        L->e_orig = ne;
+        L->canonical = true;
+        return finish(L, opts, out);
+    } catch (const std::bad_alloc &) {
+        return ROF_ERR_ALLOC;
+    }
+}
+
+int rof_layout_export(const rof_layout *L, rof_bag **out) {
+    if (!L || !out) return ROF_ERR_ARG;
+    rof_bag *bag = new (std::nothrow) rof_bag;
+    if (!bag) return ROF_ERR_ALLOC;
+    try {
+        auto put = [bag](const char *name, const ivec &v) {
+            auto &d = bag->arr[name];
+            d.resize(v.size());
+            if (!v.empty()) memcpy(d.data(), v.data(), v.size() * sizeof(int32_t));
+        };
+        put("group_ptr", L->group_ptr);
+        put("group_col", L->group_col);
+        put("group_dst_ptr", L->group_dst_ptr);
+        put("group_dst", L->group_dst);
+        put("res_ptr", L->res_ptr);
+        put("res_col", L->res_col);
+        bag->arr["canonical"].assign(1, L->canonical ? 1u : 0u);
+        // v2 tensors: groups first, then every node's residual list re-chunked by part_size
+        // (reuse_search_ext.h:537-636)
+        const int ps = L->part_size;
+        int64_t G = (int64_t)L->group_ptr.size() - 1;
+        auto &ucol = bag->arr["uniqpart_column_index"], &uptr = bag->arr["uniqpart_pointers"];
+        auto &dptr = bag->arr["part2Node_ptr"], &dcol = bag->arr["part2Node_col"];
+        ucol.assign(L->group_col.begin(), L->group_col.end());
+        ucol.insert(ucol.end(), L->res_col.begin(), L->res_col.end());
+        uptr.assign(L->group_ptr.begin(), L->group_ptr.end());
+        dptr.assign(L->group_dst_ptr.begin(), L->group_dst_ptr.end());
+        dcol.assign(L->group_dst.begin(), L->group_dst.end());
+        uint32_t base = (uint32_t)L->group_col.size();
+        for (int32_t v = 0; v < L->n; ++v) {
+            int32_t beg = L->res_ptr[v], end = L->res_ptr[v + 1];
+            for (int32_t q = beg; q < end; q += ps) {
+                uptr.push_back(base + (uint32_t)std::min(q + ps, end));
+                dcol.push_back((uint32_t)v);
+                dptr.push_back((uint32_t)dcol.size());
+            }
+        }
+        (void)G;
+        // schedule, for inspection and host-side tests
+        put("a_task_ptr", L->a.task_ptr);
+        put("a_task_nref", L->a.task_nref);
+        put("a_task_out", L->a.task_out);
+        put("a_col", L->a.col);
+        put("b_task_ptr", L->b.task_ptr);
+        put("b_task_nref", L->b.task_nref);
+        put("b_task_out", L->b.task_out);
+        put("b_col", L->b.col);
+    } catch (const std::bad_alloc &) {
+        delete bag;
+        return ROF_ERR_ALLOC;
+    }
+    *out = bag;
+    return ROF_OK;
+}
+
+int rof_layout_stats(const rof_layout *L, int64_t s[16]) {
+    if (!L || !s) return ROF_ERR_ARG;
+    memset(s, 0, 16 * sizeof(int64_t));
+    s[0] = L->n;
+    s[1] = L->e_orig;
+    s[2] = (int64_t)L->group_ptr.size() - 1;
+    s[3] = L->n_materialised;
+    s[4] = L->gathered_rows;
+    s[5] = L->partial_reads;
+    s[6] = L->n_slots;
+    s[7] = L->n_segments;
+    s[8] = L->a.n_tasks;
+    s[9] = L->b.n_tasks;
+    s[10] = L->device_bytes;
+    s[11] = L->part_size;
+    s[12] = L->a.n_wave;
+    s[13] = L->b.n_wave;
+    s[14] = L->canonical ? 1 : 0;
+    return ROF_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,53 @@
+// Internal types shared by the host-side sources of librof.so.  Not installed.
+#ifndef ROF_INTERNAL_H_
+#define ROF_INTERNAL_H_
+
+#include <cstdint>
+#include <map>
+#include <string>
+#include <vector>
+
+struct rof_bag {
+    std::map<std::string, std::vector<uint32_t>> arr;
+};
+
+// One launch worth of work: tasks in execution order.  Task t gathers the rows named by
+// col[task_ptr[t] .. task_ptr[t+1]) -- the first task_nref[t] of them are partial-sum rows
+// (ids >= the node count, pointing into the workspace), the rest are feature rows -- and writes
+// their weighted sum to output row task_out[t].  Tasks [0, n_wave) are long and get a whole
+// wavefront each; the remaining ones are short and share a wavefront.
+struct rof_phase_host {
+    std::vector<int32_t> task_ptr, task_nref, task_out, col;
+    int32_t n_wave = 0;
+    int32_t n_tasks = 0;
+};
+
+struct rof_phase_dev {
+    int32_t *task_ptr = nullptr, *task_nref = nullptr, *task_out = nullptr, *col = nullptr;
+    float *w = nullptr;       // per entry: rsqrt(deg[col]) for feature rows, 1 for partial rows
+    float *scale = nullptr;   // per task: rsqrt(deg[task_out]) (destination rows only)
+    int32_t n_wave = 0, n_tasks = 0;
+    int64_t n_entries = 0;
+};
+
+struct rof_layout {
+    int32_t n = 0;
+    int32_t part_size = 0;
+    int64_t e_orig = 0;
+    bool canonical = false;   // group/residual arrays reproduce the upstream v2 tensors exactly
+    // canonical arrays: CSR of reuse groups (+ their consumers) and destination-centric residual CSR
+    std::vector<int32_t> group_ptr, group_col, group_dst_ptr, group_dst, res_ptr, res_col;
+    // schedule
+    rof_phase_host a, b;      // a: partial sums (materialised groups, hub segments); b: destination rows
+    int64_t n_slots = 0;      // rows of the partial-sum workspace
+    int64_t n_materialised = 0, n_segments = 0, gathered_rows = 0, partial_reads = 0;
+    // device copies
+    rof_phase_dev da, db;
+    bool uploaded = false, weights_set = false;
+    int device = -1;
+    int64_t device_bytes = 0;
+};
+
+void rof_set_device_error(const char *what, const char *text);
+
+#endif

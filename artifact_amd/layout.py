@@ -1,0 +1,201 @@
+"""Device layout of a reuse plan: host-side handle around `rof_layout` (include/rof.h).
+
+A layout is built from plan arrays in any of the three upstream tensor formats and owns the
+device copy of its execution schedule.  `aggregate` runs the two kernel launches on the current
+PyTorch stream; PyTorch is used only for device memory and the stream handle.
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+
+from . import _lib
+from ._lib import LayoutOpts, RofError, bag_take, check, i32, ptr
+
+ROF_F32, ROF_BF16 = 0, 1
+
+STAT_NAMES = ("nodes", "edges", "groups", "materialised_groups", "gathered_rows", "partial_reads", "partial_rows",
+              "hub_segments", "tasks_a", "tasks_b", "device_bytes", "part_size", "wave_tasks_a", "wave_tasks_b",
+              "canonical")
+
+EXPORT_NAMES = ("group_ptr", "group_col", "group_dst_ptr", "group_dst", "res_ptr", "res_col", "canonical",
+                "uniqpart_column_index", "uniqpart_pointers", "part2Node_ptr", "part2Node_col",
+                "a_task_ptr", "a_task_nref", "a_task_out", "a_col", "b_task_ptr", "b_task_nref", "b_task_out", "b_col")
+
+
+def _opts(min_consumers=0, disable_reuse=False, hub_split=0, segment=0):
+    o = LayoutOpts()
+    o.min_consumers = int(min_consumers)
+    o.disable_reuse = int(bool(disable_reuse))
+    o.hub_split = int(hub_split)
+    o.segment = int(segment)
+    return o
+
+
+class Layout:
+    """Owns one rof_layout.  Build with from_v2 / from_v1 / from_parts (host numpy int32 arrays)."""
+
+    def __init__(self, handle, num_nodes):
+        self._h = handle
+        self.num_nodes = int(num_nodes)
+        self._deg_key = None
+        self._workspace = None
+
+    # ---- construction -------------------------------------------------------------------
+    @classmethod
+    def from_v2(cls, uniqpart_column_index, uniqpart_pointers, part2Node_ptr, part2Node_col, num_nodes, part_size,
+                **opts):
+        uc, up, dp, dc = i32(uniqpart_column_index), i32(uniqpart_pointers), i32(part2Node_ptr), i32(part2Node_col)
+        if len(up) < 1 or len(up) != len(dp):
+            raise ValueError("uniqpart_pointers and part2Node_ptr must both have one entry per unique part plus one")
+        h = C.c_void_p()
+        o = _opts(**opts)
+        check(_lib.lib().rof_layout_from_v2(ptr(uc), up.ctypes.data, dp.ctypes.data, ptr(dc), len(up) - 1,
+                                            int(num_nodes), int(part_size), C.byref(o), C.byref(h)))
+        return cls(h, num_nodes)
+
+    @classmethod
+    def from_v1(cls, column_index, part_pointers, part2Node, part_cache_flagindex, part_pointers_cache,
+                column_index_cache, num_nodes, part_size, **opts):
+        col, pp, p2n = i32(column_index), i32(part_pointers), i32(part2Node)
+        fl, cp, cc = i32(part_cache_flagindex), i32(part_pointers_cache), i32(column_index_cache)
+        if len(pp) != len(p2n) + 1 or len(fl) != len(p2n) or len(cp) < 1:
+            raise ValueError("inconsistent v1 plan array lengths")
+        h = C.c_void_p()
+        o = _opts(**opts)
+        check(_lib.lib().rof_layout_from_v1(ptr(col), pp.ctypes.data, ptr(p2n), len(p2n), ptr(fl), cp.ctypes.data,
+                                            ptr(cc), len(cp) - 1, int(num_nodes), int(part_size), C.byref(o),
+                                            C.byref(h)))
+        return cls(h, num_nodes)
+
+    @classmethod
+    def from_parts(cls, column_index, part_pointers, part2Node, num_nodes, part_size, **opts):
+        col, pp, p2n = i32(column_index), i32(part_pointers), i32(part2Node)
+        if len(pp) != len(p2n) + 1:
+            raise ValueError("part_pointers must have one entry per part plus one")
+        h = C.c_void_p()
+        o = _opts(**opts)
+        check(_lib.lib().rof_layout_from_parts(ptr(col), pp.ctypes.data, ptr(p2n), len(p2n), int(num_nodes),
+                                               int(part_size), C.byref(o), C.byref(h)))
+        return cls(h, num_nodes)
+
+    @classmethod
+    def from_csr(cls, indptr, indices, part_size=1 << 30, **opts):
+        """No reuse: every row of a destination-centric CSR is one part."""
+        ip = i32(indptr)
+        n = len(ip) - 1
+        return cls.from_parts(indices, ip, np.arange(n, dtype=np.int32), n, min(int(part_size), 1 << 30), **opts)
+
+    # ---- host-side inspection ------------------------------------------------------------
+    def export(self):
+        h = C.c_void_p()
+        check(_lib.lib().rof_layout_export(self._h, C.byref(h)))
+        r = bag_take(h, EXPORT_NAMES, dtype=np.int32)
+        r["canonical"] = bool(r["canonical"][0])
+        return r
+
+    def stats(self):
+        s = (C.c_int64 * 16)()
+        check(_lib.lib().rof_layout_stats(self._h, s))
+        return {k: int(s[i]) for i, k in enumerate(STAT_NAMES)}
+
+    def algorithmic_bytes(self, feat_dim, in_bytes=4):
+        """Bytes one aggregation must move at least once per use, as counted for the roofline:
+        every gathered row with its 4-byte column id, every partial-sum row read (fp32) and written,
+        and per node one output row plus row pointer and norm."""
+        s = self.stats()
+        return (s["gathered_rows"] * (4 + feat_dim * in_bytes) + s["partial_reads"] * (4 + feat_dim * 4)
+                + s["partial_rows"] * feat_dim * 4 + s["nodes"] * (feat_dim * 4 + 8) + 4 * (s["partial_rows"] + 1))
+
+    # ---- device side ---------------------------------------------------------------------
+    def upload(self, stream=0):
+        check(_lib.lib().rof_layout_upload(self._h, C.c_void_p(stream)))
+        return self
+
+    def set_degrees(self, degrees, stream=None):
+        """degrees: float32 CUDA tensor [num_nodes] (the in-degree vector of ROF_main.py:138,144)."""
+        import torch
+
+        if degrees.dtype != torch.float32 or not degrees.is_cuda or not degrees.is_contiguous():
+            raise RofError("degrees must be a contiguous float32 CUDA tensor")
+        if degrees.numel() != self.num_nodes:
+            raise RofError("degrees must have one entry per node")
+        key = (degrees.data_ptr(), degrees._version)
+        if key == self._deg_key:
+            return self
+        st = torch.cuda.current_stream().cuda_stream if stream is None else stream
+        self.upload(st)
+        check(_lib.lib().rof_layout_set_degrees(self._h, C.c_void_p(degrees.data_ptr()), C.c_void_p(st)))
+        self._deg_key = key
+        self._deg_ref = degrees   # keep the pointer's owner alive while it is the cache key
+        return self
+
+    def workspace_bytes(self, feat_dim):
+        return int(_lib.lib().rof_layout_workspace_bytes(self._h, int(feat_dim)))
+
+    def _args(self, x, out, feat_dim, workspace):
+        import torch
+
+        if not x.is_cuda or x.dim() != 2 or x.stride(1) != 1:
+            raise RofError("x must be a 2-D CUDA tensor with unit column stride")
+        if x.shape[0] < self.num_nodes:
+            raise RofError("x must have one row per node")
+        if x.dtype == torch.float32:
+            dt = ROF_F32
+        elif x.dtype == torch.bfloat16:
+            dt = ROF_BF16
+        else:
+            raise RofError("x must be float32 or bfloat16")
+        f = x.shape[1] if feat_dim is None else int(feat_dim)
+        if out is None:
+            out = torch.empty((self.num_nodes, f), dtype=torch.float32, device=x.device)
+        if out.dtype != torch.float32 or not out.is_cuda or out.dim() != 2 or out.stride(1) != 1:
+            raise RofError("out must be a 2-D float32 CUDA tensor with unit column stride")
+        if out.shape[0] < self.num_nodes or out.shape[1] < f:
+            raise RofError("out is too small")
+        need = self.workspace_bytes(f)
+        if workspace is None:
+            if self._workspace is None or self._workspace.numel() * 4 < need or self._workspace.device != x.device:
+                self._workspace = torch.empty(max(1, (need + 3) // 4), dtype=torch.float32, device=x.device)
+            workspace = self._workspace
+        return dt, f, out, workspace
+
+    def aggregate(self, x, normalized=True, out=None, feat_dim=None, workspace=None):
+        """out[v] = s(v) * sum_u w(u) x[u] through the plan; x may be a column-padded view."""
+        import torch
+
+        dt, f, out, workspace = self._args(x, out, feat_dim, workspace)
+        st = torch.cuda.current_stream().cuda_stream
+        self.upload(st)
+        check(_lib.lib().rof_aggregate(self._h, C.c_void_p(x.data_ptr()), dt, x.stride(0), C.c_void_p(out.data_ptr()),
+                                       out.stride(0), f, int(bool(normalized)), C.c_void_p(workspace.data_ptr()),
+                                       workspace.numel() * workspace.element_size(), C.c_void_p(st)))
+        return out
+
+    def aggregate_timed(self, x, iters, normalized=True, out=None, feat_dim=None, workspace=None):
+        """Mean milliseconds per aggregation over `iters` back-to-back calls, measured with HIP events
+        recorded on the stream the kernels run on."""
+        import torch
+
+        dt, f, out, workspace = self._args(x, out, feat_dim, workspace)
+        st = torch.cuda.current_stream().cuda_stream
+        self.upload(st)
+        ms = C.c_float()
+        check(_lib.lib().rof_aggregate_timed(self._h, C.c_void_p(x.data_ptr()), dt, x.stride(0),
+                                             C.c_void_p(out.data_ptr()), out.stride(0), f, int(bool(normalized)),
+                                             C.c_void_p(workspace.data_ptr()),
+                                             workspace.numel() * workspace.element_size(), C.c_void_p(st), int(iters),
+                                             C.byref(ms)))
+        return float(ms.value), out
+
+    def close(self):
+        if self._h is not None:
+            _lib.lib().rof_layout_free(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

@@ -1,0 +1,237 @@
+"""Layer API of the reuse-aware GCN convolution: drop-in for ROF/reuse_conv/reuse_conv.py.
+
+`ROF_GCNConvFunc` and `ROF_GCNConv` keep the upstream names, argument meaning, parameter set,
+initialisers and error behaviour (reuse_conv.py:30-150); `ROF_inputInfo` restates the plan container
+whose class is missing from the upstream tree but whose contract is fixed by its call sites
+(ROF_evaluation/ROF_main.py:164-178, reuse_conv.py:34-37,145-146).  `ROF_GINConv` is the sum-aggregation
+layer the GIN workload needs; upstream has only its kernel (ROF.SAG, reuse_conv_kernel.cu:123-196).
+"""
+from __future__ import annotations
+
+import math
+
+import numpy as np
+import torch
+
+from . import ROF
+from . import reuse_search_ext
+from .layout import Layout
+
+__all__ = ["ROF_GCNConvFunc", "ROF_GCNConv", "ROF_GINConv", "ROF_inputInfo", "build_input_info"]
+
+_TENSOR_FIELDS = ("row_pointers", "column_index", "degrees", "part_pointers", "part2Node", "part_cache_flagindex",
+                  "part_pointers_cache", "column_index_cache", "uniqpart_column_index", "uniqpart_pointers",
+                  "part2Node_ptr", "part2Node_col")
+
+
+class ROF_inputInfo:
+    """Plan container: positional constructor of ROF_main.py:164-174, attributes of the same names,
+    `dimWorker` / `part_result_cache` set later by the layer (reuse_conv.py:145-146), in-place `.to`."""
+
+    def __init__(self, row_pointers, column_index, degrees, part_pointers, part2Node, partSize, warpPerBlock,
+                 part_cache_flagindex, part_pointers_cache, column_index_cache, uniqpart_column_index,
+                 uniqpart_pointers, part2Node_ptr, part2Node_col):
+        self.row_pointers = row_pointers
+        self.column_index = column_index
+        self.degrees = degrees
+        self.part_pointers = part_pointers
+        self.part2Node = part2Node
+        self.partSize = partSize
+        self.warpPerBlock = warpPerBlock
+        self.part_cache_flagindex = part_cache_flagindex
+        self.part_pointers_cache = part_pointers_cache
+        self.column_index_cache = column_index_cache
+        self.uniqpart_column_index = uniqpart_column_index
+        self.uniqpart_pointers = uniqpart_pointers
+        self.part2Node_ptr = part2Node_ptr
+        self.part2Node_col = part2Node_col
+        self.dimWorker = 0
+        self.part_result_cache = None
+        self.layouts = {}   # kernel_type -> Layout built from host arrays (skips the device->host round trip)
+
+    def to(self, device):
+        for name in _TENSOR_FIELDS:
+            t = getattr(self, name)
+            if isinstance(t, torch.Tensor):
+                setattr(self, name, t.to(device))
+        if isinstance(self.part_result_cache, torch.Tensor):
+            self.part_result_cache = self.part_result_cache.to(device)
+        return self
+
+    @property
+    def reuse_size(self):
+        return int(self.part_pointers_cache.shape[0]) - 1
+
+    def __getstate__(self):
+        d = dict(self.__dict__)
+        d["layouts"] = {}   # device handles are rebuilt on demand
+        return d
+
+    def __repr__(self):
+        shapes = ", ".join(f"{n}={tuple(getattr(self, n).shape)}" for n in _TENSOR_FIELDS
+                           if isinstance(getattr(self, n), torch.Tensor))
+        return f"ROF_inputInfo(partSize={self.partSize}, warpPerBlock={self.warpPerBlock}, {shapes})"
+
+
+def build_input_info(indptr, indices, part_size=3, device="cuda", warps_per_block=4, plan=None):
+    """CSR (symmetric graph, in-neighbours = out-neighbours) -> ROF_inputInfo, following the glue of
+    ROF_main.py:71-178: plan on the CPU, arrays cast to int32, degrees = diff(indptr) as float32."""
+    indptr = np.asarray(indptr)
+    indices = np.asarray(indices)
+    if plan is None:
+        plan = reuse_search_ext.build_plan(indptr, indices, part_size)
+    n = len(indptr) - 1
+
+    def t(a):
+        return torch.from_numpy(np.ascontiguousarray(np.asarray(a).astype(np.int32))).to(device)
+
+    degree_in = np.diff(indptr.astype(np.int64)).astype(np.float32)
+    info = ROF_inputInfo(t(indptr), t(plan["new_indices_src"]), torch.from_numpy(degree_in).to(device),
+                         t(plan["part_ptr"]), t(plan["part2Node"]), int(part_size), int(warps_per_block),
+                         t(plan["part_cache_flagindex"]), t(plan["part_pointers_cache"]),
+                         t(plan["column_index_cache"]), t(plan["uniqpart_column_index"]), t(plan["uniqpart_pointers"]),
+                         t(plan["part2Node_ptr"]), t(plan["part2Node_col"]))
+    if torch.device(device).type == "cuda":
+        info.layouts["ROF_v2"] = Layout.from_v2(plan["uniqpart_column_index"], plan["uniqpart_pointers"],
+                                                plan["part2Node_ptr"], plan["part2Node_col"], n, part_size)
+    info.plan = plan
+    return info
+
+
+class ROF_GCNConvFunc(torch.autograd.Function):
+    """reuse_conv.py:30-92: dispatch on kernel_type, same plan forward and backward, five gradients."""
+
+    @staticmethod
+    def forward(ctx, x, weight, inputInfo, add_self_loops=False, kernel_type="ROF_v1"):
+        ii = inputInfo
+        ctx.save_for_backward(x, weight, ii.column_index, ii.degrees, ii.part_pointers, ii.part2Node,
+                              ii.part_result_cache, ii.part_cache_flagindex, ii.part_pointers_cache,
+                              ii.column_index_cache, ii.uniqpart_column_index, ii.uniqpart_pointers, ii.part2Node_ptr,
+                              ii.part2Node_col)
+        ctx.partSize = ii.partSize
+        ctx.dimWorker = ii.dimWorker
+        ctx.warpPerBlock = ii.warpPerBlock
+        ctx.kernel_type = kernel_type
+        ctx.layout = getattr(ii, "layouts", {}).get(kernel_type)
+        if add_self_loops:
+            raise NotImplementedError   # reuse_conv.py:72-73
+        if kernel_type == "GNNA":
+            return ROF.GNNA_forward(x, weight, ii.column_index, ii.degrees, ii.part_pointers, ii.part2Node,
+                                    ii.partSize, ii.dimWorker, ii.warpPerBlock)[0]
+        if kernel_type == "ROF_v1":
+            return ROF.reuse_forward_v1(x, weight, ii.column_index, ii.degrees, ii.part_pointers, ii.part2Node,
+                                        ii.partSize, ii.dimWorker, ii.warpPerBlock, ii.part_result_cache,
+                                        ii.part_cache_flagindex, ii.part_pointers_cache, ii.column_index_cache)[0]
+        if kernel_type == "ROF_v2":
+            return ROF.reuse_forward_v2(x, weight, ii.uniqpart_column_index, ii.degrees, ii.uniqpart_pointers,
+                                        ii.part2Node_ptr, ii.part2Node_col, ii.partSize, ii.dimWorker,
+                                        ii.warpPerBlock, layout=ctx.layout)[0]
+        raise NotImplementedError
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        (x, weight, column_index, degrees, part_pointers, part2Node, part_result_cache, part_cache_flagindex,
+         part_pointers_cache, column_index_cache) = ctx.saved_tensors[:-4]
+        uniqpart_column_index, uniqpart_pointers, part2Node_ptr, part2Node_col = ctx.saved_tensors[-4:]
+        ps, dw, wpb = ctx.partSize, ctx.dimWorker, ctx.warpPerBlock
+        grad_output = grad_output.contiguous()
+        if ctx.kernel_type == "GNNA":
+            d_input, d_weight = ROF.GNNA_backward(grad_output, x, weight, column_index, degrees, part_pointers,
+                                                  part2Node, ps, dw, wpb)
+        elif ctx.kernel_type == "ROF_v1":
+            d_input, d_weight = ROF.reuse_backward_v1(grad_output, x, weight, column_index, degrees, part_pointers,
+                                                      part2Node, ps, dw, wpb, part_result_cache, part_cache_flagindex,
+                                                      part_pointers_cache, column_index_cache)
+        elif ctx.kernel_type == "ROF_v2":
+            d_input, d_weight = ROF.reuse_backward_v2(grad_output, x, weight, uniqpart_column_index, degrees,
+                                                      uniqpart_pointers, part2Node_ptr, part2Node_col, ps, dw, wpb,
+                                                      layout=ctx.layout)
+        else:
+            raise NotImplementedError
+        return d_input, d_weight, None, None, None
+
+
+class ROF_GCNConv(torch.nn.Module):
+    """reuse_conv.py:96-150.  Note the upstream default add_self_loops=True raises at call time
+    (reuse_conv.py:102 with :72-73); pass add_self_loops=False as the upstream drivers do."""
+
+    def __init__(self, in_channels, out_channels, bias=True, **kwargs):
+        super().__init__()
+        self.in_channels = in_channels
+        self.out_channels = out_channels
+        self.kwargs = kwargs
+        self.add_self_loops = kwargs.get("add_self_loops", True)
+        self.kernel_type = kwargs.get("kernel_type", "ROF_v1")
+        self.weight = torch.nn.Parameter(torch.empty(in_channels, out_channels))
+        if bias:
+            self.bias = torch.nn.Parameter(torch.empty(out_channels))
+        else:
+            self.register_parameter("bias", None)
+        self.reuse_size = kwargs.get("reuse_size", 0)
+        # scratch of the v1 kernels; a Parameter upstream, so it is kept one here (state_dict parity)
+        self.part_result_cache = torch.nn.Parameter(torch.empty(max(self.reuse_size, 0), out_channels + 1),
+                                                    requires_grad=False)
+        self.dimWorker = kwargs.get("dimWorker", 0)
+        if self.dimWorker == 0:
+            self.dimWorker = 32 if out_channels > 32 else out_channels   # reuse_conv.py:115-120
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        init = self.kwargs.get("weight_initializer", "glorot")
+        if init == "glorot":
+            torch.nn.init.xavier_uniform_(self.weight)
+        elif init == "uniform":
+            bound = 1.0 / math.sqrt(self.in_channels)
+            torch.nn.init.uniform_(self.weight.data, -bound, bound)
+        elif init == "he":
+            bound = math.sqrt(6 / ((1 + 5) * self.in_channels))   # a = sqrt(5): reuse_conv.py:131-136
+            self.weight.data.uniform_(-bound, bound)
+        else:
+            raise NotImplementedError
+        if self.bias is not None:
+            torch.nn.init.zeros_(self.bias)
+        with torch.no_grad():
+            self.part_result_cache.zero_()
+
+    def forward(self, x, inputInfo):
+        inputInfo.part_result_cache = self.part_result_cache
+        inputInfo.dimWorker = self.dimWorker
+        out = ROF_GCNConvFunc.apply(x, self.weight, inputInfo, self.add_self_loops, self.kernel_type)
+        return out if self.bias is None else out + self.bias
+
+
+class _SumAggregate(torch.autograd.Function):
+    """Unnormalised neighbour sum through the reuse plan; the backward pass is the same sum on the
+    gradient because the graphs are symmetric (the assumption upstream makes for GCN as well)."""
+
+    @staticmethod
+    def forward(ctx, x, layout):
+        ctx.layout = layout
+        return layout.aggregate(ROF._padded(x.contiguous()), normalized=False, feat_dim=x.shape[1])
+
+    @staticmethod
+    def backward(ctx, grad):
+        g = grad.contiguous()
+        return ctx.layout.aggregate(ROF._padded(g), normalized=False, feat_dim=g.shape[1]), None
+
+
+class ROF_GINConv(torch.nn.Module):
+    """GIN layer: mlp((1 + eps) * x + sum_{u in N(v)} x_u), the sum evaluated through the reuse plan."""
+
+    def __init__(self, in_channels, out_channels, eps=0.0, kernel_type="ROF_v2"):
+        super().__init__()
+        self.eps = float(eps)
+        self.kernel_type = kernel_type
+        self.mlp = torch.nn.Linear(in_channels, out_channels)
+
+    def forward(self, x, inputInfo):
+        lay = inputInfo.layouts.get(self.kernel_type)
+        if lay is None:
+            ii = inputInfo
+            if self.kernel_type == "GNNA":
+                lay = ROF._layout_parts(ii.column_index, ii.part_pointers, ii.part2Node, x.shape[0], ii.partSize)
+            else:
+                lay = ROF._layout_v2(ii.uniqpart_column_index, ii.uniqpart_pointers, ii.part2Node_ptr,
+                                     ii.part2Node_col, x.shape[0], ii.partSize)
+        agg = _SumAggregate.apply(x, lay)
+        return self.mlp((1.0 + self.eps) * x + agg)

@@ -1,0 +1,182 @@
+/* rof.h -- C ABI of the MI355X reuse-aware neighbour-aggregation library (librof.so).
+ *
+ * Every entry point is extern "C", takes plain pointers and sizes, returns 0 or a negative
+ * rof_status, never throws, never exits the process and keeps no global state besides the
+ * handles it returns.  Host-side functions are safe to call concurrently on different handles;
+ * device-side functions enqueue on the hipStream_t they are given and do not synchronise.
+ *
+ * Citations name the upstream interface each entry point replaces (paths relative to the
+ * upstream tree).
+ */
+#ifndef ROF_H_
+#define ROF_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+    ROF_OK = 0,
+    ROF_ERR_ARG = -1,      /* null pointer, negative size, inconsistent array lengths        */
+    ROF_ERR_RANGE = -2,    /* an index points outside its array (checked on the host)        */
+    ROF_ERR_ALLOC = -3,    /* host or device allocation failed                               */
+    ROF_ERR_DEVICE = -4,   /* a HIP call failed; rof_last_device_error() has the HIP text    */
+    ROF_ERR_STATE = -5,    /* handle not in the state the call needs (e.g. weights not set)  */
+    ROF_ERR_UNSUPPORTED = -6,
+    ROF_ERR_WORKSPACE = -7 /* caller's workspace is smaller than rof_layout_workspace_bytes  */
+} rof_status;
+
+const char *rof_strerror(int status);
+const char *rof_last_device_error(void); /* thread-local text of the last HIP failure */
+int rof_version(void);
+
+/* ------------------------------------------------------------------------------------------
+ * Host side 1: the reuse-plan builder.  Stays on the CPU (OpenMP); every array is bit-exact
+ * with the upstream builder's output for the same input.
+ *
+ * Results come back in a "bag" of named uint32 arrays owned by the library.
+ * ---------------------------------------------------------------------------------------- */
+typedef struct rof_bag rof_bag;
+
+/* Borrowed pointer to a named array (valid until rof_bag_free); returns its length or -1. */
+int64_t rof_bag_get(const rof_bag *bag, const char *name, const uint32_t **data);
+void rof_bag_free(rof_bag *bag);
+
+/* replaces py_split_part -> split_part
+ * (ROF/reuse_search_ext/src/reuse_search_ext.cc:82-103, reuse_search_ext.h:82-148).
+ * bag: "part_ptr"[parts+1], "part2Node"[parts], "num_parts_per_node_acc"[n]. */
+int rof_split_part(const uint32_t *indptr_dst, uint32_t n, int part_size, rof_bag **out);
+
+/* replaces py_get_part_intersect -> get_part_intersect (reuse_search_ext.cc:108-142, h:152-228),
+ * count half: "intersect_count"[parts].  The lists themselves are produced on demand by
+ * rof_part_intersect_lists, because materialising all of them is quadratic in hub degree. */
+int rof_part_intersect_count(const uint32_t *part_ptr, uint64_t num_parts, const uint32_t *indices_src, uint64_t e,
+                             const uint32_t *indptr_src, const uint32_t *indices_dst, uint32_t n, int part_size,
+                             int discard_remainder_part, rof_bag **out);
+
+/* The intersection lists of the parts named in which[0..n_which):
+ * bag: "ptr"[n_which+1], "data"[ptr[n_which]] (each list ascending). */
+int rof_part_intersect_lists(const uint32_t *part_ptr, uint64_t num_parts, const uint32_t *indices_src, uint64_t e,
+                             const uint32_t *indptr_src, const uint32_t *indices_dst, uint32_t n, int part_size,
+                             int discard_remainder_part, const uint32_t *which, uint64_t n_which, rof_bag **out);
+
+/* replaces py_greedy_max_reuse -> greedy_max_reuse (reuse_search_ext.cc:145-160, h:232-303).
+ * bag: "index_ordered"[parts], "index_picked"[P]. */
+int rof_greedy_max_reuse(const uint32_t *intersect_count, uint64_t num_parts, const uint32_t *part_ptr,
+                         const uint32_t *indices_src, uint64_t e, rof_bag **out);
+
+/* replaces py_reorganize_indices -> reorganize_indices (reuse_search_ext.cc:169-211, h:409-505) and
+ * py_reorganize_indices_uniquely -> reorganize_indices_uniquely (cc:214-257, h:507-640).
+ * picked_dst_ptr/picked_dst = the intersection lists of the picked parts, in pick order.
+ * which: 1 = v1 arrays, 2 = v2 arrays, 3 = both.
+ * bag v1: "new_indices_src"[e], "part_pointers_cache"[P+1], "column_index_cache", "part_cache_flagindex"[parts]
+ * bag v2: "uniqpart_column_index", "uniqpart_pointers"[U+1], "part2Node_ptr"[U+1], "part2Node_col". */
+int rof_reorganize(const uint32_t *part_ptr, uint64_t num_parts, const uint32_t *indices_src, uint64_t e,
+                   const uint32_t *index_picked, uint64_t num_picked, const uint32_t *picked_dst_ptr,
+                   const uint32_t *picked_dst, const uint32_t *indptr_dst, uint32_t n,
+                   const uint32_t *num_parts_per_node_acc, int part_size, int which, rof_bag **out);
+
+/* replaces py_inverse_csc_or_csr -> inverse_csc (reuse_search_ext.cc:51-78, h:18-78).
+ * bag: "indptr"[n+1], "indices"[e] (rows ascending). */
+int rof_transpose_csr(const uint32_t *indptr, const uint32_t *indices, uint32_t n, uint64_t e, rof_bag **out);
+
+/* The whole upstream call sequence (ROF_evaluation/ROF_main.py:71-127) in one call.  Pass
+ * indptr_src/indices_dst = NULL for a symmetric graph (ROF_main.py:62-64).
+ * bag: every array above plus "picked_dst_ptr"/"picked_dst". */
+int rof_plan_build(const uint32_t *indptr_dst, const uint32_t *indices_src, const uint32_t *indptr_src,
+                   const uint32_t *indices_dst, uint32_t n, uint64_t e, int part_size, int discard_remainder_part,
+                   rof_bag **out);
+
+/* ------------------------------------------------------------------------------------------
+ * Host side 2: the device layout.  A plan in any of the three upstream tensor formats is
+ * re-laid out into (a) a CSR of reuse groups with their consumers and (b) a destination-centric
+ * CSR of residual neighbours; from those the library derives its execution schedule
+ * (degree-binned row tasks, split hub rows, virtual column ids for group partial sums) and
+ * uploads it.  The layout owns its device memory (hipMalloc) until rof_layout_free.
+ * ---------------------------------------------------------------------------------------- */
+typedef struct rof_layout rof_layout;
+
+typedef struct {
+    int32_t min_consumers;   /* a group is materialised iff it has >= this many consumers; 0 = cost model; -1 = all */
+    int32_t disable_reuse;   /* 1: expand every group back into its consumers' rows (the comparator)      */
+    int32_t hub_split;       /* rows with more entries than this are cut into segments; 0 = default        */
+    int32_t segment;         /* entries per hub segment; 0 = default                                        */
+    int32_t reserved[4];
+} rof_layout_opts;
+
+/* v2 tensors: replaces the plan arguments of reuse_forward_v2 / reuse_backward_v2
+ * (ROF/reuse_conv/reuse_conv.cpp:288-346; kernel contract reuse_conv_kernel.cu:852-954). */
+int rof_layout_from_v2(const int32_t *uniqpart_column_index, const int32_t *uniqpart_pointers,
+                       const int32_t *part2Node_ptr, const int32_t *part2Node_col, int64_t num_uniqparts,
+                       int32_t num_nodes, int part_size, const rof_layout_opts *opts, rof_layout **out);
+
+/* v1 tensors: replaces the plan arguments of reuse_forward_v1 / reuse_backward_v1
+ * (reuse_conv.cpp:199-285; kernel contract reuse_conv_kernel.cu:396-601). */
+int rof_layout_from_v1(const int32_t *column_index, const int32_t *part_pointers, const int32_t *part2Node,
+                       int64_t num_parts, const int32_t *part_cache_flagindex, const int32_t *part_pointers_cache,
+                       const int32_t *column_index_cache, int64_t cache_num, int32_t num_nodes, int part_size,
+                       const rof_layout_opts *opts, rof_layout **out);
+
+/* GNNA tensors (no reuse): replaces the plan arguments of GNNA_forward / GNNA_backward / SAG
+ * (reuse_conv.cpp:132-196; kernel contract reuse_conv_kernel.cu:205-286, 123-196). */
+int rof_layout_from_parts(const int32_t *column_index, const int32_t *part_pointers, const int32_t *part2Node,
+                          int64_t num_parts, int32_t num_nodes, int part_size, const rof_layout_opts *opts,
+                          rof_layout **out);
+
+/* Canonical arrays of the layout (host copies, int32 viewed as uint32):
+ *   "group_ptr"[G+1] "group_col"  "group_dst_ptr"[G+1] "group_dst"  "res_ptr"[N+1] "res_col"
+ * and the v2 tensors reconstructed from them ("uniqpart_column_index", "uniqpart_pointers",
+ * "part2Node_ptr", "part2Node_col"), which equal the input of rof_layout_from_v2 bit for bit
+ * whenever that input has the upstream builder's canonical shape. */
+int rof_layout_export(const rof_layout *layout, rof_bag **out);
+
+/* Counters: [0] nodes [1] original edges [2] groups [3] materialised groups [4] gathered rows per
+ * pass (E_u) [5] partial-row reads (R) [6] partial rows written (incl. hub segments) [7] hub segments
+ * [8] phase-A tasks [9] phase-B tasks [10] device bytes held [11] part_size. */
+int rof_layout_stats(const rof_layout *layout, int64_t stats[16]);
+
+/* Copy the schedule to the current HIP device (idempotent). */
+int rof_layout_upload(rof_layout *layout, void *stream);
+
+/* Per-edge weights rsqrt(deg[src]) and per-row scales rsqrt(deg[dst]) from the float32 in-degree
+ * vector the upstream kernels take (reuse_conv_kernel.cu:254,276,943-944).  degrees: device, [n]. */
+int rof_layout_set_degrees(rof_layout *layout, const float *degrees_dev, void *stream);
+
+size_t rof_layout_workspace_bytes(const rof_layout *layout, int feat_dim);
+
+void rof_layout_free(rof_layout *layout);
+
+/* ------------------------------------------------------------------------------------------
+ * Device side: the aggregation itself (hand-written gfx950 kernels, wave64, no MFMA,
+ * no global atomics).  Computes, for every node v,
+ *     out[v,:] = s(v) * sum over v's neighbour entries u of w(u) * x[u,:]
+ * with w = s = rsqrt(deg) when normalized (GCN: reuse_conv_kernel.cu:205-286, 836-954) and
+ * w = s = 1 otherwise (sum aggregation: reuse_conv_kernel.cu:123-196), evaluated through the
+ * layout's reuse groups.  x: [n, feat_dim] with row stride ldx (elements), out: float32
+ * [n, feat_dim] with row stride ldo; every row of out is overwritten (no zero-fill needed).
+ * The same call serves the backward pass on d_output because upstream runs the un-transposed
+ * plan there (reuse_conv_kernel.cu:1021-1041).
+ * ---------------------------------------------------------------------------------------- */
+enum { ROF_F32 = 0, ROF_BF16 = 1 };
+
+int rof_aggregate(const rof_layout *layout, const void *x, int x_dtype, int64_t ldx, float *out, int64_t ldo,
+                  int feat_dim, int normalized, void *workspace, size_t workspace_bytes, void *stream);
+
+/* Timing helper for benchmarks: runs rof_aggregate `iters` times on `stream` between two HIP
+ * events recorded on that same stream and returns the mean milliseconds per call. */
+int rof_aggregate_timed(const rof_layout *layout, const void *x, int x_dtype, int64_t ldx, float *out, int64_t ldo,
+                        int feat_dim, int normalized, void *workspace, size_t workspace_bytes, void *stream,
+                        int iters, float *ms_per_call);
+
+/* Launch tuning: how many consecutive workgroups of launch 1 / launch 2 stay on one XCD (each XCD
+ * has its own L2, so runs of neighbouring destination rows share gathered rows there).  Process-wide;
+ * no upstream counterpart. */
+int rof_set_xcd_run(int run_launch1, int run_launch2);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ROF_H_ */

@@ -1,0 +1,146 @@
+"""GPU parity of the aggregation kernels, called through the C ABI (librof.so via ctypes).
+
+Bars: fp32 sums rel 1e-5 / abs 1e-6 against the fp32 restatement of the upstream kernels
+(oracle/agg_oracle.c), and against the float64 closed form with the tolerance widened by the
+row length (fp32 accumulation error grows with the number of summands); bf16 inputs rel 1e-2.
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+from artifact_amd import reuse_search_ext as R            # noqa: E402
+from artifact_amd.graphgen import features, make_workload  # noqa: E402
+from artifact_amd.layout import Layout                     # noqa: E402
+
+
+def _case(name, scale_down, ps):
+    indptr, indices = make_workload(name, scale_down)
+    plan = R.build_plan(indptr, indices, ps)
+    return indptr, indices, plan
+
+
+def _layout(plan, n, ps, **opts):
+    return Layout.from_v2(plan["uniqpart_column_index"], plan["uniqpart_pointers"], plan["part2Node_ptr"],
+                          plan["part2Node_col"], n, ps, **opts)
+
+
+def _close(got, want64, x_abs_rowsum=None, rtol=1e-5, atol=1e-6):
+    """|got - want| <= atol + rtol*|want| + rtol*(sum of |terms|): the last term is the standard fp32
+    summation bound and matters only where cancellation makes |want| tiny."""
+    tol = atol + rtol * np.abs(want64)
+    if x_abs_rowsum is not None:
+        tol = tol + rtol * x_abs_rowsum
+    bad = np.abs(got - want64) > tol
+    assert not bad.any(), f"{bad.sum()} elements off, max err {np.abs(got - want64).max():.3e}"
+
+
+@pytest.mark.parametrize("feat", [1, 3, 4, 32, 40, 47, 64, 100, 256, 300])
+def test_gcn_widths_match_oracle(oracle, feat):
+    indptr, indices, plan = _case("c1", 2, 3)
+    n = len(indptr) - 1
+    x = features(n, feat, seed=7)
+    deg = np.diff(indptr).astype(np.float32)
+    lay = _layout(plan, n, 3)
+    xt = torch.from_numpy(x).cuda()
+    lay.set_degrees(torch.from_numpy(deg).cuda())
+    got = lay.aggregate(xt, normalized=True).cpu().numpy()
+    ref32 = oracle.agg_v2(x, deg, plan["uniqpart_column_index"], plan["uniqpart_pointers"], plan["part2Node_ptr"],
+                          plan["part2Node_col"])
+    want = oracle.closed_form(indptr, indices, x, deg)
+    mag = oracle.closed_form(indptr, indices, np.abs(x), deg)
+    _close(got, want, mag)
+    _close(got, ref32.astype(np.float64), mag)
+
+
+@pytest.mark.parametrize("name,sd,ps", [("c1", 0, 3), ("c1", 0, 2), ("c1", 1, 5), ("c2", 3, 3), ("c3", 5, 2),
+                                        ("c4", 6, 3)])
+def test_reuse_equals_no_reuse_and_closed_form(oracle, name, sd, ps):
+    indptr, indices, plan = _case(name, sd, ps)
+    n = len(indptr) - 1
+    feat = 47
+    x = features(n, 48, seed=11)[:, :feat]                  # strided view: row stride 48, width 47
+    deg = np.diff(indptr).astype(np.float32)
+    degt = torch.from_numpy(deg).cuda()
+    xt = torch.from_numpy(np.ascontiguousarray(features(n, 48, seed=11))).cuda()[:, :feat]
+    want = oracle.closed_form(indptr, indices, x, deg)
+    mag = oracle.closed_form(indptr, indices, np.abs(x), deg)
+    outs = []
+    for opts in (dict(), dict(disable_reuse=True), dict(min_consumers=2), dict(hub_split=64, segment=16)):
+        lay = _layout(plan, n, ps, **opts)
+        lay.set_degrees(degt)
+        out = torch.full((n, feat), float("nan"), device="cuda")   # every element must be overwritten
+        lay.aggregate(xt, normalized=True, out=out, feat_dim=feat)
+        got = out.cpu().numpy()
+        assert np.isfinite(got).all()
+        _close(got, want, mag)
+        outs.append(got)
+        lay.close()
+    assert np.allclose(outs[0], outs[1], rtol=1e-5, atol=1e-6)
+
+
+def test_sum_aggregation_unnormalised(oracle):
+    indptr, indices, plan = _case("c3", 5, 2)
+    n = len(indptr) - 1
+    x = features(n, 64, seed=5)
+    lay = _layout(plan, n, 2)
+    got = lay.aggregate(torch.from_numpy(x).cuda(), normalized=False).cpu().numpy()
+    want = oracle.closed_form(indptr, indices, x, normalized=False)
+    _close(got, want, oracle.closed_form(indptr, indices, np.abs(x), normalized=False))
+
+
+def test_unaligned_rows_take_scalar_path(oracle):
+    indptr, indices, plan = _case("c1", 3, 3)
+    n = len(indptr) - 1
+    x = features(n, 47, seed=3)                              # packed rows of 188 bytes: not 16-byte aligned
+    deg = np.diff(indptr).astype(np.float32)
+    lay = _layout(plan, n, 3)
+    lay.set_degrees(torch.from_numpy(deg).cuda())
+    got = lay.aggregate(torch.from_numpy(x).cuda(), normalized=True).cpu().numpy()
+    _close(got, oracle.closed_form(indptr, indices, x, deg), oracle.closed_form(indptr, indices, np.abs(x), deg))
+
+
+@pytest.mark.parametrize("feat", [256, 40])
+def test_bf16_inputs_fp32_accumulate(oracle, feat):
+    indptr, indices, plan = _case("c1", 1, 3)
+    n = len(indptr) - 1
+    xb = torch.from_numpy(features(n, feat, seed=9, kind="uniform")).to(torch.bfloat16)
+    x = xb.to(torch.float32).numpy()                         # the oracle sees the bf16-rounded values
+    deg = np.diff(indptr).astype(np.float32)
+    lay = _layout(plan, n, 3)
+    lay.set_degrees(torch.from_numpy(deg).cuda())
+    got = lay.aggregate(xb.cuda(), normalized=True).cpu().numpy()
+    want = oracle.closed_form(indptr, indices, x, deg)
+    mag = oracle.closed_form(indptr, indices, np.abs(x), deg)
+    _close(got, want, mag, rtol=1e-2, atol=1e-6)             # stated bar for bf16-in / fp32-accumulate
+    _close(got, want, mag, rtol=1e-5, atol=1e-6)             # and in fact as tight as fp32: inputs are exact
+
+
+def test_deterministic_run_to_run():
+    indptr, indices, plan = _case("c1", 1, 3)
+    n = len(indptr) - 1
+    lay = _layout(plan, n, 3)
+    lay.set_degrees(torch.from_numpy(np.diff(indptr).astype(np.float32)).cuda())
+    xt = torch.from_numpy(features(n, 64, seed=1)).cuda()
+    a = lay.aggregate(xt).clone()
+    b = lay.aggregate(xt).clone()
+    assert torch.equal(a, b)                                 # no atomics: bitwise repeatable
+
+
+def test_empty_rows_and_isolated_nodes(oracle):
+    indptr = np.array([0, 0, 2, 2, 3, 3, 3, 3, 3, 3, 3], dtype=np.int32)   # nodes 0,2,4.. have no in-edges
+    indices = np.array([3, 1, 1], dtype=np.int32)
+    n = 10
+    lay = Layout.from_csr(indptr, indices)
+    deg = np.maximum(np.diff(indptr), 0).astype(np.float32)
+    lay.set_degrees(torch.from_numpy(deg).cuda())
+    x = features(n, 8, seed=2)
+    got = lay.aggregate(torch.from_numpy(x).cuda()).cpu().numpy()
+    want = np.zeros_like(x, dtype=np.float64)
+    r = oracle.rsqrt_rn(np.array([2.0, 1.0]))
+    want[1] = r[0] * (r[1] * x[3] + r[0] * x[1])
+    want[3] = r[1] * (r[0] * x[1])
+    assert np.allclose(got, want, rtol=1e-5, atol=1e-6)
+    assert (got[[0, 2, 4, 5, 6, 7, 8, 9]] == 0).all()
