@@ -19,7 +19,7 @@ SYMBOLS = (
     "rof_part_intersect_count", "rof_part_intersect_lists", "rof_greedy_max_reuse", "rof_reorganize",
     "rof_transpose_csr", "rof_plan_build", "rof_layout_from_v2", "rof_layout_from_v1", "rof_layout_from_parts",
     "rof_layout_export", "rof_layout_stats", "rof_layout_upload", "rof_layout_set_degrees",
-    "rof_layout_workspace_bytes", "rof_layout_free", "rof_aggregate", "rof_aggregate_timed", "rof_set_xcd_run",
+    "rof_layout_workspace_bytes", "rof_layout_free", "rof_aggregate", "rof_aggregate_timed", "rof_set_xcd_run", "rof_aggregate_launch_times", "rof_device_copy",
 )
 
 
@@ -69,6 +69,9 @@ def lib():
     L.rof_aggregate.argtypes = [vp, vp, ci, i64, vp, i64, ci, ci, vp, C.c_size_t, vp]
     L.rof_aggregate_timed.argtypes = [vp, vp, ci, i64, vp, i64, ci, ci, vp, C.c_size_t, vp, ci, C.POINTER(C.c_float)]
     L.rof_set_xcd_run.argtypes = [ci, ci]
+    L.rof_device_copy.argtypes = [vp, vp, C.c_size_t, vp]
+    L.rof_aggregate_launch_times.argtypes = [vp, vp, ci, i64, vp, i64, ci, ci, vp, C.c_size_t, vp, ci,
+                                             C.POINTER(C.c_float * 2)]
     _lib = L
     return L
 

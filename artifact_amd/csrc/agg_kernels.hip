@@ -4,9 +4,10 @@
 // weighted sum to one output row:
 //     out[task_out[t], :] = scale[t] * sum_i w[i] * row(col[i])        i in task_ptr[t] .. task_ptr[t+1]
 // where row(c) is x[c, :] for c < nsplit and the partial-sum row part[c - nsplit, :] otherwise
-// (the first task_nref[t] entries of a task are of the second kind).  Launch 1 fills the
-// partial-sum rows (reuse groups that several destinations share, segments of very long rows),
-// launch 2 produces every destination row.  There are no atomics: each output row has one writer.
+// (the first task_nref[t] entries of a task are of the second kind).  Up to three launches in stream
+// order: reuse groups that several destinations share -> partial-sum rows; segments of very long rows
+// (which may read group rows) -> partial-sum rows; every destination row -> out.  There are no
+// atomics: each output row has one writer.
 //
 // Mapping to the machine:
 //   * the feature dimension runs across lanes, VEC consecutive elements per lane (one 16-byte
@@ -111,10 +112,12 @@ struct RowLoad<uint16_t, 1> {
 
 // Sum the entries [beg, end) of one task into acc.  WAVE: all lane groups of the wavefront share
 // the task (beg/end wave-uniform) and take every G-th entry; otherwise each lane group owns its
-// task.  ST is the element type of the source rows, `base`/`ld` its address and row stride, `bias`
-// is subtracted from the column id.
-template <typename ST, int VEC, int LPR, bool WAVE>
-__device__ __forceinline__ void gather_sum(const ST *__restrict__ src, int64_t ld, int32_t bias,
+// task.  ST is the element type of the source rows.  With DUAL (fp32 features only) ids >= nsplit
+// are taken from the partial-sum rows instead, chosen per entry by a pointer select, so a task
+// that mixes both kinds still runs one loop with one fetch of ids and weights per chunk.
+template <typename ST, int VEC, int LPR, bool WAVE, bool DUAL>
+__device__ __forceinline__ void gather_sum(const ST *__restrict__ src, int64_t ld, const float *__restrict__ part,
+                                           int64_t ldp, int32_t nsplit, int32_t bias,
                                            const int32_t *__restrict__ col, const float *__restrict__ w,
                                            int32_t beg, int32_t end, int lane, int sub, int li, int cbase, bool act,
                                            float (&acc)[VEC]) {
@@ -147,7 +150,16 @@ __device__ __forceinline__ void gather_sum(const ST *__restrict__ src, int64_t l
             }
 #pragma unroll
             for (int u = 0; u < U; ++u)
-                if (ok[u]) RowLoad<ST, VEC>::load(src + (int64_t)(c[u] - bias) * ld + cbase, v[u]);
+                if (ok[u]) {
+                    if (DUAL) {
+                        const bool p = c[u] >= nsplit;
+                        const ST *row = p ? reinterpret_cast<const ST *>(part) + (int64_t)(c[u] - nsplit) * ldp
+                                          : src + (int64_t)c[u] * ld;
+                        RowLoad<ST, VEC>::load(row + cbase, v[u]);
+                    } else {
+                        RowLoad<ST, VEC>::load(src + (int64_t)(c[u] - bias) * ld + cbase, v[u]);
+                    }
+                }
 #pragma unroll
             for (int u = 0; u < U; ++u)
                 if (ok[u]) {
@@ -158,7 +170,9 @@ __device__ __forceinline__ void gather_sum(const ST *__restrict__ src, int64_t l
     }
 }
 
-template <typename XT, int VEC, int LPR>
+// PHASE 0: the partial-sum launches (no scaling); PHASE 1: the destination-row launch.  Same code; the
+// parameter only gives them distinct kernel names in profiles.
+template <typename XT, int VEC, int LPR, int PHASE>
 __global__ __launch_bounds__(256) void rof_rows_kernel(AggArgs a) {
     constexpr int G = 64 / LPR;
     // XCD-aware renumbering: the hardware deals workgroup ids round-robin to the 8 XCDs; give each
@@ -197,21 +211,35 @@ __global__ __launch_bounds__(256) void rof_rows_kernel(AggArgs a) {
 #pragma unroll
         for (int k = 0; k < VEC; ++k) acc[k] = 0.0f;
 
+        constexpr bool kF32 = sizeof(XT) == 4;   // fp32 features: partial rows have the same element type
+        constexpr bool kRefs = true;   // segments of long rows may reference group rows too
         if (wave_mode) {
-            if (mid > beg)
-                gather_sum<float, VEC, LPR, true>(a.part, a.ldp, a.nsplit, a.col, a.w, beg, mid, lane, sub, li, cbase,
-                                                  act, acc);
-            gather_sum<XT, VEC, LPR, true>(x, a.ldx, 0, a.col, a.w, mid, end, lane, sub, li, cbase, act, acc);
+            if (kF32 || !kRefs) {
+                gather_sum<XT, VEC, LPR, true, kRefs>(x, a.ldx, a.part, a.ldp, a.nsplit, 0, a.col, a.w, beg, end, lane,
+                                                      sub, li, cbase, act, acc);
+            } else {
+                if (mid > beg)
+                    gather_sum<float, VEC, LPR, true, false>(a.part, a.ldp, nullptr, 0, 0, a.nsplit, a.col, a.w, beg,
+                                                             mid, lane, sub, li, cbase, act, acc);
+                gather_sum<XT, VEC, LPR, true, false>(x, a.ldx, nullptr, 0, 0, 0, a.col, a.w, mid, end, lane, sub, li,
+                                                      cbase, act, acc);
+            }
 #pragma unroll
             for (int off = LPR; off < 64; off <<= 1) {
 #pragma unroll
                 for (int k = 0; k < VEC; ++k) acc[k] += __shfl_xor(acc[k], off);
             }
         } else {
-            if (__any(mid > beg))
-                gather_sum<float, VEC, LPR, false>(a.part, a.ldp, a.nsplit, a.col, a.w, beg, mid, lane, sub, li, cbase,
-                                                   act, acc);
-            gather_sum<XT, VEC, LPR, false>(x, a.ldx, 0, a.col, a.w, mid, end, lane, sub, li, cbase, act, acc);
+            if (kF32 || !kRefs) {
+                gather_sum<XT, VEC, LPR, false, kRefs>(x, a.ldx, a.part, a.ldp, a.nsplit, 0, a.col, a.w, beg, end, lane,
+                                                       sub, li, cbase, act, acc);
+            } else {
+                if (__any(mid > beg))
+                    gather_sum<float, VEC, LPR, false, false>(a.part, a.ldp, nullptr, 0, 0, a.nsplit, a.col, a.w, beg,
+                                                              mid, lane, sub, li, cbase, act, acc);
+                gather_sum<XT, VEC, LPR, false, false>(x, a.ldx, nullptr, 0, 0, 0, a.col, a.w, mid, end, lane, sub, li,
+                                                       cbase, act, acc);
+            }
         }
 
         const bool writer = valid && act && (!wave_mode || sub == 0);
@@ -253,7 +281,14 @@ __global__ void rof_task_scale_kernel(const int32_t *__restrict__ task_out, int3
     if (i < T) scale[i] = rsqrt_rn(deg[task_out[i]]);
 }
 
-template <typename XT, int VEC>
+// plain streaming copy, used only to calibrate profiler byte counters against a known size
+__global__ void rof_copy_kernel(const float4 *__restrict__ src, float4 *__restrict__ dst, int64_t n16) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n16; i += stride) dst[i] = src[i];
+}
+
+template <typename XT, int VEC, int PHASE>
 int launch_lpr(const AggArgs &a0, int lpr, hipStream_t st) {
     AggArgs a = a0;
     const int g = 64 / lpr;
@@ -265,21 +300,23 @@ int launch_lpr(const AggArgs &a0, int lpr, hipStream_t st) {
     const int64_t grid = (a.n_blocks + span - 1) / span * span;
     dim3 gr((unsigned)grid), bl(64 * kWavesPerBlock);
     switch (lpr) {
-        case 4: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 4>), gr, bl, 0, st, a); break;
-        case 8: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 8>), gr, bl, 0, st, a); break;
-        case 16: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 16>), gr, bl, 0, st, a); break;
-        case 32: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 32>), gr, bl, 0, st, a); break;
-        default: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 64>), gr, bl, 0, st, a); break;
+        case 4: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 4, PHASE>), gr, bl, 0, st, a); break;
+        case 8: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 8, PHASE>), gr, bl, 0, st, a); break;
+        case 16: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 16, PHASE>), gr, bl, 0, st, a); break;
+        case 32: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 32, PHASE>), gr, bl, 0, st, a); break;
+        default: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 64, PHASE>), gr, bl, 0, st, a); break;
     }
     HIP_TRY(hipGetLastError());
     return ROF_OK;
 }
 
+template <int PHASE>
 int launch_phase(const AggArgs &a, int dtype, int vec, hipStream_t st) {
     int need = (a.feat + vec - 1) / vec, lpr = 4;
     while (lpr < need && lpr < 64) lpr <<= 1;
-    if (dtype == ROF_F32) return vec == 4 ? launch_lpr<float, 4>(a, lpr, st) : launch_lpr<float, 1>(a, lpr, st);
-    return vec == 8 ? launch_lpr<uint16_t, 8>(a, lpr, st) : launch_lpr<uint16_t, 1>(a, lpr, st);
+    if (dtype == ROF_F32)
+        return vec == 4 ? launch_lpr<float, 4, PHASE>(a, lpr, st) : launch_lpr<float, 1, PHASE>(a, lpr, st);
+    return vec == 8 ? launch_lpr<uint16_t, 8, PHASE>(a, lpr, st) : launch_lpr<uint16_t, 1, PHASE>(a, lpr, st);
 }
 
 int upload_phase(const rof_phase_host &h, rof_phase_dev &d, bool with_scale, hipStream_t st, int64_t *bytes) {
@@ -357,13 +394,23 @@ int rof_set_xcd_run(int run_a, int run_b) {
     return ROF_OK;
 }
 
+int rof_device_copy(void *dst, const void *src, size_t nbytes, void *stream) {
+    if (!dst || !src || (nbytes & 15) || (((uintptr_t)dst | (uintptr_t)src) & 15)) return ROF_ERR_ARG;
+    if (nbytes == 0) return ROF_OK;
+    hipLaunchKernelGGL(rof_copy_kernel, dim3(256 * 32), dim3(256), 0, (hipStream_t)stream, (const float4 *)src,
+                       (float4 *)dst, (int64_t)(nbytes / 16));
+    HIP_TRY(hipGetLastError());
+    return ROF_OK;
+}
+
 int rof_layout_upload(rof_layout *L, void *stream) {
     if (!L) return ROF_ERR_ARG;
     if (L->uploaded) return ROF_OK;
     hipStream_t st = (hipStream_t)stream;
     HIP_TRY(hipGetDevice(&L->device));
     int rc;
-    if ((rc = upload_phase(L->a, L->da, false, st, &L->device_bytes))) return rc;
+    if ((rc = upload_phase(L->g, L->dg, false, st, &L->device_bytes))) return rc;
+    if ((rc = upload_phase(L->s, L->ds, false, st, &L->device_bytes))) return rc;
     if ((rc = upload_phase(L->b, L->db, true, st, &L->device_bytes))) return rc;
     HIP_TRY(hipStreamSynchronize(st));   // the host vectors may be released after this call
     L->uploaded = true;
@@ -375,9 +422,10 @@ int rof_layout_set_degrees(rof_layout *L, const float *deg, void *stream) {
     if (!L->uploaded) return ROF_ERR_STATE;
     hipStream_t st = (hipStream_t)stream;
     const int tb = 256;
-    if (L->da.n_entries)
-        hipLaunchKernelGGL(rof_entry_weights_kernel, dim3((unsigned)((L->da.n_entries + tb - 1) / tb)), dim3(tb), 0, st,
-                           L->da.col, L->da.n_entries, deg, L->n, L->da.w);
+    for (rof_phase_dev *d : {&L->dg, &L->ds})
+        if (d->n_entries)
+            hipLaunchKernelGGL(rof_entry_weights_kernel, dim3((unsigned)((d->n_entries + tb - 1) / tb)), dim3(tb), 0,
+                               st, d->col, d->n_entries, deg, L->n, d->w);
     if (L->db.n_entries)
         hipLaunchKernelGGL(rof_entry_weights_kernel, dim3((unsigned)((L->db.n_entries + tb - 1) / tb)), dim3(tb), 0, st,
                            L->db.col, L->db.n_entries, deg, L->n, L->db.w);
@@ -397,14 +445,16 @@ size_t rof_layout_workspace_bytes(const rof_layout *L, int feat_dim) {
 void rof_layout_free(rof_layout *L) {
     if (!L) return;
     if (L->uploaded) {
-        free_phase(L->da);
+        free_phase(L->dg);
+        free_phase(L->ds);
         free_phase(L->db);
     }
     delete L;
 }
 
-int rof_aggregate(const rof_layout *L, const void *x, int x_dtype, int64_t ldx, float *out, int64_t ldo, int feat,
-                  int normalized, void *workspace, size_t workspace_bytes, void *stream) {
+static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64_t ldx, float *out, int64_t ldo,
+                          int feat, int normalized, void *workspace, size_t workspace_bytes, void *stream,
+                          int launches) {
     if (!L || !x || !out || feat < 1 || ldx < feat || ldo < feat) return ROF_ERR_ARG;
     if (x_dtype != ROF_F32 && x_dtype != ROF_BF16) return ROF_ERR_UNSUPPORTED;
     if (!L->uploaded || (normalized && !L->weights_set)) return ROF_ERR_STATE;
@@ -430,22 +480,26 @@ int rof_aggregate(const rof_layout *L, const void *x, int x_dtype, int64_t ldx, 
     a.nsplit = L->n;
     a.feat = feat;
     int rc;
-    if (L->da.n_tasks) {   // launch 1: partial-sum rows
-        a.task_ptr = L->da.task_ptr;
-        a.task_nref = L->da.task_nref;
-        a.task_out = L->da.task_out;
+    // launches 1 and 2: partial-sum rows (shared groups, then segments of long rows)
+    const rof_phase_dev *partial[2] = {&L->dg, &L->ds};
+    for (int i = 0; i < 2 && (launches & 1); ++i) {
+        const rof_phase_dev &d = *partial[i];
+        if (!d.n_tasks) continue;
+        a.task_ptr = d.task_ptr;
+        a.task_nref = d.task_nref;
+        a.task_out = d.task_out;
         a.task_scale = nullptr;
-        a.col = L->da.col;
-        a.w = normalized ? L->da.w : nullptr;
+        a.col = d.col;
+        a.w = normalized ? d.w : nullptr;
         a.out = (float *)workspace;
         a.ldo = ldp;
-        a.n_wave = L->da.n_wave;
-        a.n_tasks = L->da.n_tasks;
+        a.n_wave = d.n_wave;
+        a.n_tasks = d.n_tasks;
         a.xcd_run = g_xcd_run_a;
         a.vec_store = 1;
-        if ((rc = launch_phase(a, x_dtype, vec, st))) return rc;
+        if ((rc = launch_phase<0>(a, x_dtype, vec, st))) return rc;
     }
-    if (L->db.n_tasks) {   // launch 2: destination rows
+    if (L->db.n_tasks && (launches & 2)) {   // last launch: destination rows
         a.task_ptr = L->db.task_ptr;
         a.task_nref = L->db.task_nref;
         a.task_out = L->db.task_out;
@@ -458,9 +512,14 @@ int rof_aggregate(const rof_layout *L, const void *x, int x_dtype, int64_t ldx, 
         a.n_tasks = L->db.n_tasks;
         a.xcd_run = g_xcd_run_b;
         a.vec_store = (ldo % 4 == 0) && (((uintptr_t)out) % 16 == 0);
-        if ((rc = launch_phase(a, x_dtype, vec, st))) return rc;
+        if ((rc = launch_phase<1>(a, x_dtype, vec, st))) return rc;
     }
     return ROF_OK;
+}
+
+int rof_aggregate(const rof_layout *L, const void *x, int x_dtype, int64_t ldx, float *out, int64_t ldo, int feat,
+                  int normalized, void *workspace, size_t workspace_bytes, void *stream) {
+    return aggregate_impl(L, x, x_dtype, ldx, out, ldo, feat, normalized, workspace, workspace_bytes, stream, 3);
 }
 
 int rof_aggregate_timed(const rof_layout *L, const void *x, int x_dtype, int64_t ldx, float *out, int64_t ldo,
@@ -482,6 +541,41 @@ int rof_aggregate_timed(const rof_layout *L, const void *x, int x_dtype, int64_t
     (void)hipEventDestroy(e0);
     (void)hipEventDestroy(e1);
     *ms_per_call = ms / iters;
+    return rc;
+}
+
+int rof_aggregate_launch_times(const rof_layout *L, const void *x, int x_dtype, int64_t ldx, float *out, int64_t ldo,
+                               int feat, int normalized, void *workspace, size_t workspace_bytes, void *stream,
+                               int iters, float ms_launch[2]) {
+    if (!ms_launch || iters < 1 || !L) return ROF_ERR_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    // each iteration times [launch 1 + launch 2] and then [launch 2 alone]; launch 2 alone is a
+    // complete run because launch 1's rows are still in the workspace
+    hipEvent_t e0, e1, e2;
+    HIP_TRY(hipEventCreate(&e0));
+    HIP_TRY(hipEventCreate(&e1));
+    HIP_TRY(hipEventCreate(&e2));
+    double both = 0.0, second = 0.0;
+    int rc = rof_aggregate(L, x, x_dtype, ldx, out, ldo, feat, normalized, workspace, workspace_bytes, st);
+    for (int i = 0; i < iters && rc == ROF_OK; ++i) {
+        HIP_TRY(hipEventRecord(e0, st));
+        rc = rof_aggregate(L, x, x_dtype, ldx, out, ldo, feat, normalized, workspace, workspace_bytes, st);
+        HIP_TRY(hipEventRecord(e1, st));
+        if (rc == ROF_OK)
+            rc = aggregate_impl(L, x, x_dtype, ldx, out, ldo, feat, normalized, workspace, workspace_bytes, st, 2);
+        HIP_TRY(hipEventRecord(e2, st));
+        HIP_TRY(hipEventSynchronize(e2));
+        float a = 0.f, b = 0.f;
+        HIP_TRY(hipEventElapsedTime(&a, e0, e1));
+        HIP_TRY(hipEventElapsedTime(&b, e1, e2));
+        both += a;
+        second += b;
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    (void)hipEventDestroy(e2);
+    ms_launch[1] = (float)(second / iters);
+    ms_launch[0] = (float)((both - second) / iters);
     return rc;
 }
 

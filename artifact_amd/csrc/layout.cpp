@@ -3,8 +3,8 @@
 //       CSR of residual neighbours -- from which the upstream v2 tensors can be rebuilt bit for bit;
 //   (2) the execution schedule for the gfx950 kernels: every destination row becomes one task whose
 //       entries are either feature-row ids or "virtual" ids >= N naming a partial-sum row; groups that
-//       are worth sharing and segments of very long rows become tasks of a first launch that fills those
-//       partial-sum rows.  Tasks are ordered long-to-short, short ones tile by tile, so that the lanes
+//       are worth sharing become tasks of a first launch and segments of very long rows tasks of a second
+//       launch, both filling partial-sum rows that the last launch (one task per destination) reads.  Tasks are ordered long-to-short, short ones tile by tile, so that the lanes
 //       of a wavefront that share one launch slot do the same amount of work.
 #include <algorithm>
 #include <cstdint>
@@ -124,21 +124,6 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     const bool disable = o && o->disable_reuse;
     const int32_t min_consumers = o ? o->min_consumers : 0;
 
-    // which groups are computed once and shared
-    std::vector<int32_t> slot_of(G, -1);
-    int64_t slots = 0;
-    for (int64_t g = 0; g < G; ++g) {
-        int64_t len = L->group_ptr[g + 1] - L->group_ptr[g];
-        int64_t cnt = L->group_dst_ptr[g + 1] - L->group_dst_ptr[g];
-        bool share;
-        if (disable) share = false;
-        else if (min_consumers < 0) share = true;   // every group, even one nobody consumes (v1 cache rows)
-        else if (min_consumers > 0) share = cnt >= min_consumers;
-        else share = (cnt - 1) * len > cnt + 1;   // row gathers saved > partial-row reads + the one write
-        if (share && (min_consumers < 0 || (len > 0 && cnt > 0))) slot_of[g] = (int32_t)slots++;
-    }
-    L->n_materialised = slots;
-
     // node -> groups it consumes (ascending group index)
     ivec ng_ptr((size_t)n + 1, 0), ng;
     for (int64_t j = 0; j < (int64_t)L->group_dst.size(); ++j) ng_ptr[L->group_dst[j] + 1]++;
@@ -150,63 +135,82 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
             for (int32_t j = L->group_dst_ptr[g]; j < L->group_dst_ptr[g + 1]; ++j) ng[at[L->group_dst[j]]++] = (int32_t)g;
     }
 
-    TaskList ta, tb;
+    // Which groups are computed once and shared.  A group is worth a partial-sum row when the row
+    // gathers it saves exceed the partial-row reads plus the one write it adds.
+    auto worth = [&](int64_t cnt, int64_t len) {
+        if (disable) return false;
+        if (min_consumers < 0) return true;   // every group, even one nobody consumes (v1 cache rows)
+        if (len <= 0 || cnt <= 0) return false;
+        if (min_consumers > 0) return cnt >= min_consumers;
+        return (cnt - 1) * len > cnt + 1;
+    };
+    std::vector<int32_t> slot_of(G, -1);
+    int64_t slots = 0;
+    TaskList tg, ts, tb;
     for (int64_t g = 0; g < G; ++g) {
-        if (slot_of[g] < 0) continue;
-        ta.begin_task(slot_of[g]);
-        ta.col.insert(ta.col.end(), L->group_col.begin() + L->group_ptr[g], L->group_col.begin() + L->group_ptr[g + 1]);
-        ta.end_task(0);
+        if (!worth(L->group_dst_ptr[g + 1] - L->group_dst_ptr[g], L->group_ptr[g + 1] - L->group_ptr[g])) continue;
+        slot_of[g] = (int32_t)slots++;
+        tg.begin_task(slot_of[g]);
+        tg.col.insert(tg.col.end(), L->group_col.begin() + L->group_ptr[g], L->group_col.begin() + L->group_ptr[g + 1]);
+        tg.end_task(0);
     }
+    L->n_materialised = slots;
+
     tb.ptr.reserve((size_t)n + 1);
     tb.nref.reserve(n);
     tb.out.reserve(n);
     tb.col.reserve(L->res_col.size() + L->group_dst.size());
-    int64_t gathered = (int64_t)ta.col.size(), reads = 0, segments = 0;
-    ivec reals;
+    int64_t gathered = (int64_t)tg.col.size(), reads = 0, segments = 0;
+    ivec row;   // one destination's entries: references first, then feature rows
     for (int32_t v = 0; v < n; ++v) {
-        tb.begin_task(v);
+        row.clear();
         int32_t refs = 0;
-        reals.clear();
+        for (int32_t j = ng_ptr[v]; j < ng_ptr[v + 1]; ++j)
+            if (slot_of[ng[j]] >= 0) {
+                row.push_back(n + slot_of[ng[j]]);
+                ++refs;
+            }
         for (int32_t j = ng_ptr[v]; j < ng_ptr[v + 1]; ++j) {
             int32_t g = ng[j];
-            if (slot_of[g] >= 0) {
-                tb.col.push_back(n + slot_of[g]);
-                ++refs;
-            } else {
-                reals.insert(reals.end(), L->group_col.begin() + L->group_ptr[g], L->group_col.begin() + L->group_ptr[g + 1]);
-            }
+            if (slot_of[g] < 0)
+                row.insert(row.end(), L->group_col.begin() + L->group_ptr[g], L->group_col.begin() + L->group_ptr[g + 1]);
         }
-        const int32_t *res = L->res_col.data() + L->res_ptr[v];
-        int64_t nres = L->res_ptr[v + 1] - L->res_ptr[v];
-        int64_t nreal = (int64_t)reals.size() + nres;
-        gathered += nreal;
-        if (nreal > hub_split) {
-            // cut the row's feature-row entries into segments; each becomes a partial-sum task
-            reals.insert(reals.end(), res, res + nres);
-            for (int64_t s0 = 0; s0 < nreal; s0 += segment) {
-                int64_t s1 = std::min<int64_t>(nreal, s0 + segment);
-                int32_t slot = (int32_t)slots++;
-                ta.begin_task(slot);
-                ta.col.insert(ta.col.end(), reals.begin() + s0, reals.begin() + s1);
-                ta.end_task(0);
-                tb.col.push_back(n + slot);
-                ++refs;
-                ++segments;
-            }
-        } else {
-            tb.col.insert(tb.col.end(), reals.begin(), reals.end());
-            tb.col.insert(tb.col.end(), res, res + nres);
-        }
+        row.insert(row.end(), L->res_col.begin() + L->res_ptr[v], L->res_col.begin() + L->res_ptr[v + 1]);
+        const int64_t len = (int64_t)row.size();
+        gathered += len - refs;
         reads += refs;
-        tb.end_task(refs);
+        tb.begin_task(v);
+        if (len > hub_split) {
+            // A long row is cut into segments; each becomes a partial-sum task of the middle launch
+            // (after the groups it may reference, before the rows), and the row itself just adds them up.
+            int32_t nseg = 0;
+            for (int64_t s0 = 0; s0 < len; s0 += segment) {
+                int64_t s1 = std::min<int64_t>(len, s0 + segment);
+                int32_t slot = (int32_t)slots++;
+                ts.begin_task(slot);
+                ts.col.insert(ts.col.end(), row.begin() + s0, row.begin() + s1);
+                ts.end_task((int32_t)std::max<int64_t>(0, std::min<int64_t>(refs, s1) - s0));
+                tb.col.push_back(n + slot);
+                ++nseg;
+            }
+            segments += nseg;
+            reads += nseg;
+            tb.end_task(nseg);
+        } else {
+            tb.col.insert(tb.col.end(), row.begin(), row.end());
+            tb.end_task(refs);
+        }
     }
     if (slots + (int64_t)n >= INT32_MAX || tb.col.size() >= (size_t)INT32_MAX) return ROF_ERR_UNSUPPORTED;
     L->n_slots = slots;
     L->n_segments = segments;
     L->gathered_rows = gathered;
     L->partial_reads = reads;
-    finalize_phase(ta, 1 << 30, L->a);
+    finalize_phase(tg, 1 << 30, L->g);
+    finalize_phase(ts, 1 << 30, L->s);
     finalize_phase(tb, kTileRows, L->b);
+    L->gathered_before_rows = (int64_t)tg.col.size();
+    for (size_t t = 0; t < ts.out.size(); ++t) L->gathered_before_rows += (ts.ptr[t + 1] - ts.ptr[t]) - ts.nref[t];
     return ROF_OK;
 }
 
@@ -412,10 +416,14 @@ int rof_layout_export(const rof_layout *L, rof_bag **out) {
         }
         (void)G;
         // schedule, for inspection and host-side tests
-        put("a_task_ptr", L->a.task_ptr);
-        put("a_task_nref", L->a.task_nref);
-        put("a_task_out", L->a.task_out);
-        put("a_col", L->a.col);
+        put("g_task_ptr", L->g.task_ptr);
+        put("g_task_nref", L->g.task_nref);
+        put("g_task_out", L->g.task_out);
+        put("g_col", L->g.col);
+        put("s_task_ptr", L->s.task_ptr);
+        put("s_task_nref", L->s.task_nref);
+        put("s_task_out", L->s.task_out);
+        put("s_col", L->s.col);
         put("b_task_ptr", L->b.task_ptr);
         put("b_task_nref", L->b.task_nref);
         put("b_task_out", L->b.task_out);
@@ -439,13 +447,14 @@ int rof_layout_stats(const rof_layout *L, int64_t s[16]) {
     s[5] = L->partial_reads;
     s[6] = L->n_slots;
     s[7] = L->n_segments;
-    s[8] = L->a.n_tasks;
+    s[8] = L->g.n_tasks + L->s.n_tasks;
     s[9] = L->b.n_tasks;
     s[10] = L->device_bytes;
     s[11] = L->part_size;
-    s[12] = L->a.n_wave;
+    s[12] = L->g.n_wave + L->s.n_wave;
     s[13] = L->b.n_wave;
     s[14] = L->canonical ? 1 : 0;
+    s[15] = L->gathered_before_rows;
     return ROF_OK;
 }
 

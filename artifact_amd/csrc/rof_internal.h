@@ -38,11 +38,11 @@ struct rof_layout {
     // canonical arrays: CSR of reuse groups (+ their consumers) and destination-centric residual CSR
     std::vector<int32_t> group_ptr, group_col, group_dst_ptr, group_dst, res_ptr, res_col;
     // schedule
-    rof_phase_host a, b;      // a: partial sums (materialised groups, hub segments); b: destination rows
+    rof_phase_host g, s, b;   // g: shared groups; s: segments of long rows (may read g's rows); b: destination rows
     int64_t n_slots = 0;      // rows of the partial-sum workspace
-    int64_t n_materialised = 0, n_segments = 0, gathered_rows = 0, partial_reads = 0;
+    int64_t n_materialised = 0, n_segments = 0, gathered_rows = 0, partial_reads = 0, gathered_before_rows = 0;
     // device copies
-    rof_phase_dev da, db;
+    rof_phase_dev dg, ds, db;
     bool uploaded = false, weights_set = false;
     int device = -1;
     int64_t device_bytes = 0;

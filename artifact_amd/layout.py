@@ -17,11 +17,12 @@ ROF_F32, ROF_BF16 = 0, 1
 
 STAT_NAMES = ("nodes", "edges", "groups", "materialised_groups", "gathered_rows", "partial_reads", "partial_rows",
               "hub_segments", "tasks_a", "tasks_b", "device_bytes", "part_size", "wave_tasks_a", "wave_tasks_b",
-              "canonical")
+              "canonical", "gathered_rows_a")
 
 EXPORT_NAMES = ("group_ptr", "group_col", "group_dst_ptr", "group_dst", "res_ptr", "res_col", "canonical",
                 "uniqpart_column_index", "uniqpart_pointers", "part2Node_ptr", "part2Node_col",
-                "a_task_ptr", "a_task_nref", "a_task_out", "a_col", "b_task_ptr", "b_task_nref", "b_task_out", "b_col")
+                "g_task_ptr", "g_task_nref", "g_task_out", "g_col", "s_task_ptr", "s_task_nref", "s_task_out", "s_col",
+                "b_task_ptr", "b_task_nref", "b_task_out", "b_col")
 
 
 def _opts(min_consumers=0, disable_reuse=False, hub_split=0, segment=0):
@@ -188,6 +189,27 @@ class Layout:
                                              workspace.numel() * workspace.element_size(), C.c_void_p(st), int(iters),
                                              C.byref(ms)))
         return float(ms.value), out
+
+    def launch_times(self, x, iters, normalized=True, out=None, feat_dim=None, workspace=None):
+        """(ms of the partial-sum launch, ms of the destination-row launch), HIP-event means over `iters`."""
+        import torch
+
+        dt, f, out, workspace = self._args(x, out, feat_dim, workspace)
+        st = torch.cuda.current_stream().cuda_stream
+        self.upload(st)
+        ms = (C.c_float * 2)()
+        check(_lib.lib().rof_aggregate_launch_times(self._h, C.c_void_p(x.data_ptr()), dt, x.stride(0),
+                                                    C.c_void_p(out.data_ptr()), out.stride(0), f,
+                                                    int(bool(normalized)), C.c_void_p(workspace.data_ptr()),
+                                                    workspace.numel() * workspace.element_size(), C.c_void_p(st),
+                                                    int(iters), C.byref(ms)))
+        return float(ms[0]), float(ms[1])
+
+    def launch_bytes(self, feat_dim, in_bytes=4):
+        """Algorithmic bytes of (launch 1, launch 2): the split of `algorithmic_bytes`."""
+        s = self.stats()
+        a = s["gathered_rows_a"] * (4 + feat_dim * in_bytes) + s["partial_rows"] * feat_dim * 4 + 4 * (s["partial_rows"] + 1)
+        return a, self.algorithmic_bytes(feat_dim, in_bytes) - a
 
     def close(self):
         if self._h is not None:

@@ -1,0 +1,281 @@
+#!/usr/bin/env python3
+"""Benchmark of the reuse-aware aggregation layer on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4] [--part-size 3]
+
+A step is one aggregation layer: out = D^-1/2 A D^-1/2 (XW) evaluated through the reuse plan on a
+feature matrix that is already resident in HBM (the dense update X*W is not part of the step).
+The default workload is the 2.4M-node R-MAT graph with aggregated width 47.  Prints one JSON line:
+GEdges/s (original edge count / time), the HBM roofline of the destination-row launch measured with
+HIP events on the launch stream, the same kernels with reuse disabled, and a CPU baseline (the
+oracle's destination-parallel SpMM) timed on this machine's host cores.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+DESCR = {
+    "c1": "c1: R-MAT 2^14 nodes, avg deg 16, self loops, GCN sym-norm, F=32, fp32",
+    "c2": "c2: R-MAT 2^18 nodes, avg deg 14, self loops, GCN sym-norm, F=256, fp32",
+    "c3": "c3: SBM 2^20 nodes (256 blocks), deg 24+2, GIN sum aggregation, F=64, fp32",
+    "c4": "c4: R-MAT 2.4M nodes, ~60M directed edges, GCN sym-norm, aggregated width 47, fp32",
+    "c5": "c5: R-MAT 2^22 nodes, avg deg 32, self loops, GCN sym-norm, F=256, bf16 in / fp32 accumulate",
+}
+FEAT = {"c1": 32, "c2": 256, "c3": 64, "c4": 47, "c5": 256}
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def load_or_build(name, part_size, cache_dir):
+    """Graph + plan, cached on local disk so repeated runs on one machine skip the CPU preprocessing."""
+    from artifact_amd import reuse_search_ext as R
+    from artifact_amd.graphgen import make_workload
+
+    path = os.path.join(cache_dir, f"rof_{name}_ps{part_size}.npz") if cache_dir else None
+    if path and os.path.exists(path):
+        z = np.load(path)
+        log(f"[bench] loaded cached graph+plan {path}")
+        return {k: z[k] for k in z.files}, 0.0, 0.0
+    t0 = time.time()
+    indptr, indices = make_workload(name)
+    t_gen = time.time() - t0
+    log(f"[bench] generated {name}: N={len(indptr) - 1} E={len(indices)} in {t_gen:.1f}s")
+    t0 = time.time()
+    plan = R.build_plan(indptr, indices, part_size)
+    t_plan = time.time() - t0
+    log(f"[bench] reuse plan (CPU, {os.cpu_count()} cores visible): {t_plan:.1f}s, picked {len(plan['index_picked'])}")
+    d = {"indptr": indptr, "indices": indices}
+    for k in ("uniqpart_column_index", "uniqpart_pointers", "part2Node_ptr", "part2Node_col", "intersect_count",
+              "index_picked"):
+        d[k] = plan[k]
+    if path:
+        try:
+            os.makedirs(cache_dir, exist_ok=True)
+            np.savez(path, **d)
+        except OSError:
+            pass
+    return d, t_gen, t_plan
+
+
+def cpu_baseline(indptr, indices, x32, normalized, budget_s=20.0):
+    """Oracle port, destination-parallel over the host threads, on the same graph and features."""
+    from oracle import oracle as O
+
+    deg = np.diff(indptr).astype(np.float32)
+    with np.errstate(divide="ignore"):
+        rs = O.rsqrt_rn(deg)
+    rs[~np.isfinite(rs)] = 0.0
+    out = np.empty_like(x32)
+    O.spmm_rows(x32, rs, indptr, indices, normalized, out=out)          # warm-up
+    times = []
+    t_all = time.time()
+    while len(times) < 5 and (time.time() - t_all < budget_s or len(times) < 2):
+        t0 = time.time()
+        O.spmm_rows(x32, rs, indptr, indices, normalized, out=out)
+        times.append(time.time() - t0)
+    threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    return float(np.median(times)), len(times), threads, out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="c4", choices=sorted(DESCR))
+    ap.add_argument("--part-size", type=int, default=3)
+    ap.add_argument("--feat", type=int, default=0, help="override the aggregated width")
+    ap.add_argument("--cache-dir", default="/tmp/rof_bench_cache")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--xcd-run", type=int, default=0)
+    ap.add_argument("--hub-split", type=int, default=0, help="layout tuning: rows longer than this are segmented")
+    ap.add_argument("--segment", type=int, default=0, help="layout tuning: entries per segment")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one 1 GiB rof_copy_kernel launch (reference transfer for profiler byte counters)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: every machine of this build has a single MI355X and the aggregation "
+                 "path has no multi-GPU part (sharding is described in DESIGN.md); run with --gpus 1")
+
+    import torch
+
+    from artifact_amd import _lib
+    from artifact_amd.graphgen import features
+    from artifact_amd.layout import Layout
+
+    L = _lib.lib()   # raises if the HIP library is missing
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    if args.xcd_run:
+        _lib.check(L.rof_set_xcd_run(1, args.xcd_run))
+    dev = torch.device("cuda:0")
+    name, ps = args.workload, args.part_size
+    feat = args.feat or FEAT[name]
+    normalized = name != "c3"
+    bf16 = name == "c5"
+
+    d, t_gen, t_plan = load_or_build(name, ps, args.cache_dir)
+    indptr, indices = d["indptr"], d["indices"]
+    n, e = len(indptr) - 1, len(indices)
+    deg = torch.from_numpy(np.diff(indptr).astype(np.float32)).to(dev)
+
+    # features: N(0,1) fp32 (uniform(-1,1) -> bf16 for c5), rows padded to a multiple of 4 (8) elements
+    mult = 8 if bf16 else 4
+    ld = (feat + mult - 1) // mult * mult
+    x32 = features(n, feat, seed=2000 + int(name[1]), kind="uniform" if bf16 else "normal")
+    xbuf = torch.zeros((n, ld), dtype=torch.bfloat16 if bf16 else torch.float32, device=dev)
+    xbuf[:, :feat] = torch.from_numpy(x32).to(dev)
+    x = xbuf[:, :feat]
+    if bf16:
+        x32 = x.to(torch.float32).cpu().numpy()
+    in_bytes = 2 if bf16 else 4
+
+    t0 = time.time()
+    reuse = Layout.from_v2(d["uniqpart_column_index"], d["uniqpart_pointers"], d["part2Node_ptr"], d["part2Node_col"],
+                           n, ps, hub_split=args.hub_split, segment=args.segment)
+    plain = Layout.from_v2(d["uniqpart_column_index"], d["uniqpart_pointers"], d["part2Node_ptr"], d["part2Node_col"],
+                           n, ps, disable_reuse=True, hub_split=args.hub_split, segment=args.segment)
+    t_layout = time.time() - t0
+    for lay in (reuse, plain):
+        lay.upload()
+        if normalized:
+            lay.set_degrees(deg)
+    out = torch.empty((n, feat), dtype=torch.float32, device=dev)
+    out_plain = torch.empty_like(out)
+
+    # ---- warm-up: W steps, and at least ~0.3 s of work so the clocks have settled
+    t0 = time.perf_counter()
+    done = 0
+    while done < args.warmup or time.perf_counter() - t0 < 0.3:
+        reuse.aggregate(x, normalized, out=out, feat_dim=feat)
+        plain.aggregate(x, normalized, out=out_plain, feat_dim=feat)
+        done += 1
+        if done % 8 == 0:
+            torch.cuda.synchronize()
+    torch.cuda.synchronize()
+
+    # ---- timed region: exactly K steps between synchronisations
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        reuse.aggregate(x, normalized, out=out, feat_dim=feat)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # ---- HIP-event timings on the launch stream; reuse and reuse-disabled alternate so that drift
+    # of clocks or temperature hits both alike
+    per = max(5, args.steps // 4)
+    ev_r, ev_p = [], []
+    for _ in range(4):
+        ev_r.append(reuse.aggregate_timed(x, per, normalized, out=out, feat_dim=feat)[0])
+        ev_p.append(plain.aggregate_timed(x, per, normalized, out=out_plain, feat_dim=feat)[0])
+    ev_ms, plain_ms = float(np.median(ev_r)), float(np.median(ev_p))
+    ms_a, ms_b = reuse.launch_times(x, max(5, args.steps // 2), normalized, out=out, feat_dim=feat)
+    pms_a, pms_b = plain.launch_times(x, max(5, args.steps // 2), normalized, out=out_plain, feat_dim=feat)
+    torch.cuda.synchronize()
+    max_diff = float((out - out_plain).abs().max())
+
+    if args.calibrate_copy:
+        import ctypes
+        a = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        b = torch.empty_like(a)
+        torch.cuda.synchronize()
+        _lib.check(L.rof_device_copy(ctypes.c_void_p(b.data_ptr()), ctypes.c_void_p(a.data_ptr()), a.numel() * 4,
+                                     ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+        torch.cuda.synchronize()
+        del a, b
+
+    st = reuse.stats()
+    bytes_a, bytes_b = reuse.launch_bytes(feat, in_bytes)
+    b_alg = reuse.algorithmic_bytes(feat, in_bytes)
+    b_alg_plain = plain.algorithmic_bytes(feat, in_bytes)
+    b_noreuse_model = e * (4 + feat * in_bytes) + n * (feat * 4 + 8)
+    achieved_b = bytes_b / (ms_b * 1e-3) / 1e9
+
+    result = {
+        "metric": "GEdges/s per aggregation layer (reuse plan), 1 MI355X",
+        "value": e / (wall_ms * 1e-3) / 1e9,
+        "unit": "GEdges/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": wall_ms,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16->f32" if bf16 else "f32",
+        "data": "synthetic",
+        "config": {"workload": DESCR[name], "nodes": n, "edges": e, "feat": feat, "row_stride": ld,
+                   "part_size": ps, "normalized": normalized},
+        "roofline": {
+            "bound": "hbm", "kernel": "rof_rows_kernel (destination-row launch)",
+            "achieved": achieved_b, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved_b / HBM_PEAK_GBS,
+            "traffic": None, "bytes_per_launch": bytes_b, "ms_per_launch": ms_b,
+        },
+        "layer": {
+            "event_ms": ev_ms, "event_ms_runs": ev_r, "launch1_ms": ms_a, "launch2_ms": ms_b,
+            "algorithmic_bytes": b_alg, "achieved_GBs": b_alg / (ev_ms * 1e-3) / 1e9,
+            "frac_of_hbm_peak": b_alg / (ev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "no_reuse_model_bytes": b_noreuse_model,
+        },
+        "reuse_disabled": {
+            "event_ms": plain_ms, "launch1_ms": pms_a, "launch2_ms": pms_b, "GEdges_per_s": e / (plain_ms * 1e-3) / 1e9,
+            "achieved_GBs": b_alg_plain / (plain_ms * 1e-3) / 1e9, "speedup_of_reuse": plain_ms / ev_ms,
+            "max_abs_diff_vs_reuse": max_diff,
+        },
+        "plan": {"groups": st["groups"], "materialised_groups": st["materialised_groups"],
+                 "gathered_rows": st["gathered_rows"], "partial_reads": st["partial_reads"],
+                 "partial_rows": st["partial_rows"], "hub_segments": st["hub_segments"],
+                 "saved_gathers_frac": 1.0 - st["gathered_rows"] / max(1, e),
+                 "cpu_graph_s": t_gen, "cpu_plan_s": t_plan, "cpu_layout_s": t_layout},
+    }
+
+    if not args.no_cpu_baseline:
+        from oracle import oracle as O  # checker + CPU baseline leg only
+
+        cpu_s, runs, threads, cpu_out = cpu_baseline(indptr, indices, np.ascontiguousarray(x32), normalized)
+        got = out.cpu().numpy()
+        err = float(np.abs(got - cpu_out).max())
+        result["cpu_baseline"] = {
+            "value": e / cpu_s / 1e9, "unit": "GEdges/s", "cores": threads, "kind": "port",
+            "sample": f"the full {name} layer (same graph and features), median of {runs} passes of the oracle's "
+                      f"destination-parallel SpMM (oracle/agg_oracle.c) after one warm-up",
+            "ms_per_layer": cpu_s * 1e3, "max_abs_diff_gpu_vs_cpu": err,
+        }
+        try:
+            torch.set_num_threads(threads)
+            rs = O.rsqrt_rn(np.diff(indptr).astype(np.float32))
+            rs[~np.isfinite(rs)] = 0.0
+            vals = torch.from_numpy((rs[np.repeat(np.arange(n), np.diff(indptr))] * rs[indices]).astype(np.float32)
+                                    if normalized else np.ones(e, dtype=np.float32))
+            a = torch.sparse_csr_tensor(torch.from_numpy(indptr.astype(np.int64)),
+                                        torch.from_numpy(indices.astype(np.int64)), vals, size=(n, n))
+            xt = torch.from_numpy(np.ascontiguousarray(x32))
+            torch.sparse.mm(a, xt)
+            ts = []
+            for _ in range(3):
+                t0 = time.time()
+                torch.sparse.mm(a, xt)
+                ts.append(time.time() - t0)
+            result["cpu_baseline"]["torch_sparse_mm_GEdges_per_s"] = e / float(np.median(ts)) / 1e9
+        except Exception as ex:  # the library leg is informative only
+            result["cpu_baseline"]["torch_sparse_mm_error"] = str(ex)[:200]
+
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -135,7 +135,8 @@ int rof_layout_export(const rof_layout *layout, rof_bag **out);
 
 /* Counters: [0] nodes [1] original edges [2] groups [3] materialised groups [4] gathered rows per
  * pass (E_u) [5] partial-row reads (R) [6] partial rows written (incl. hub segments) [7] hub segments
- * [8] phase-A tasks [9] phase-B tasks [10] device bytes held [11] part_size. */
+ * [8] phase-A tasks [9] phase-B tasks [10] device bytes held [11] part_size [12] long tasks of launch 1 [13] of launch 2
+ * [14] canonical flag [15] rows gathered by launch 1. */
 int rof_layout_stats(const rof_layout *layout, int64_t stats[16]);
 
 /* Copy the schedule to the current HIP device (idempotent). */
@@ -170,6 +171,18 @@ int rof_aggregate(const rof_layout *layout, const void *x, int x_dtype, int64_t 
 int rof_aggregate_timed(const rof_layout *layout, const void *x, int x_dtype, int64_t ldx, float *out, int64_t ldo,
                         int feat_dim, int normalized, void *workspace, size_t workspace_bytes, void *stream,
                         int iters, float *ms_per_call);
+
+/* Per-launch timing for the roofline report: ms_launch[1] = mean duration of the destination-row
+ * launch alone (HIP events on `stream` around it), ms_launch[0] = mean duration of the whole call minus
+ * that, i.e. the partial-sum launch.  No upstream counterpart. */
+int rof_aggregate_launch_times(const rof_layout *layout, const void *x, int x_dtype, int64_t ldx, float *out,
+                               int64_t ldo, int feat_dim, int normalized, void *workspace, size_t workspace_bytes,
+                               void *stream, int iters, float ms_launch[2]);
+
+/* Plain device-to-device streaming copy (nbytes a multiple of 16, pointers 16-byte aligned).  Exists so
+ * that a profiler's FETCH_SIZE / WRITE_SIZE counters can be calibrated against a transfer of known size.
+ * No upstream counterpart. */
+int rof_device_copy(void *dst, const void *src, size_t nbytes, void *stream);
 
 /* Launch tuning: how many consecutive workgroups of launch 1 / launch 2 stay on one XCD (each XCD
  * has its own L2, so runs of neighbouring destination rows share gathered rows there).  Process-wide;
