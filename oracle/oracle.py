@@ -118,10 +118,12 @@ def _quiet():
         os.close(old)
 
 
-def ref_plan(indptr_dst, indices_src, part_size, indptr_src=None, indices_dst=None, discard=True):
+def ref_plan(indptr_dst, indices_src, part_size, indptr_src=None, indices_dst=None, discard=True, reorganize=True):
     """Same dict as oracle_plan, produced by the upstream code through the call sequence of
     ROF_evaluation/ROF_main.py:71-127.  Needs >= 9 nodes: upstream split_part prints
-    indptr_dst[0..9] unconditionally (h:91-94)."""
+    indptr_dst[0..9] unconditionally (h:91-94).  With discard=False upstream may pick a remainder
+    part, and its reorganisers then write out of bounds (heap corruption was observed); pass
+    reorganize=False to stop after the greedy step in that setting."""
     R = ref_module()
     if R is None:
         raise RuntimeError("oracle/_ref is not built")
@@ -134,18 +136,25 @@ def ref_plan(indptr_dst, indices_src, part_size, indptr_src=None, indices_dst=No
         pp, p2n, acc = R.py_split_part(e, e.copy(), ipd, part_size)
         ilist, cnt = R.py_get_part_intersect(pp, isrc, ips, idst, part_size, bool(discard))
         ordered, picked = R.py_greedy_max_reuse(cnt, pp, isrc)
-        new_idx, _, cptr, ccol, flag = R.py_reorganize_indices(pp, isrc, ilist, picked, ipd, acc, part_size)
-        ucol, uptr, dptr, dcol = R.py_reorganize_indices_uniquely(pp, isrc, ilist, picked, ipd, acc, part_size)
+        if reorganize:
+            new_idx, _, cptr, ccol, flag = R.py_reorganize_indices(pp, isrc, ilist, picked, ipd, acc, part_size)
+            ucol, uptr, dptr, dcol = R.py_reorganize_indices_uniquely(pp, isrc, ilist, picked, ipd, acc, part_size)
     iptr = np.zeros(len(ilist) + 1, dtype=np.uint32)
     np.cumsum([len(a) for a in ilist], out=iptr[1:])
     idata = np.concatenate([np.asarray(a, dtype=np.uint32) for a in ilist]) if len(ilist) else e
-    return {
+    out = {
         "part_ptr": pp, "part2Node": p2n, "num_parts_per_node_acc": acc, "intersect_ptr": iptr,
         "intersect_data": idata.astype(np.uint32), "intersect_count": np.asarray(cnt[0], dtype=np.uint32),
-        "index_ordered": ordered, "index_picked": picked, "new_indices_src": new_idx,
+        "index_ordered": ordered, "index_picked": picked,
+    }
+    if not reorganize:
+        return out
+    out.update({
+        "new_indices_src": new_idx,
         "part_pointers_cache": cptr, "column_index_cache": ccol, "part_cache_flagindex": flag,
         "uniqpart_column_index": ucol, "uniqpart_pointers": uptr, "part2Node_ptr": dptr, "part2Node_col": dcol,
-    }
+    })
+    return out
 
 
 # --------------------------------------------------------------------------- aggregation
@@ -167,7 +176,8 @@ def closed_form(indptr, indices, x, deg=None, normalized=True):
     d = np.diff(indptr).astype(np.float32) if deg is None else np.asarray(deg, dtype=np.float32)
     with np.errstate(divide="ignore"):
         r = 1.0 / np.sqrt(d.astype(np.float64))
-    y = a @ (x64 * np.where(np.isfinite(r), r, 0.0)[:, None])
+    r = np.where(np.isfinite(r), r, 0.0)     # a node without in-edges keeps a zero row (cu:303)
+    y = a @ (x64 * r[:, None])
     return y * r[:, None]
 
 

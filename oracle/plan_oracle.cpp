@@ -128,7 +128,9 @@ static void permute_rows(const vec &part_ptr, const vec &orig, const vec &ipp, c
             }
             cur_pos[d] = at;
             size_t prev = (d + n - 1) % n;
-            if (flags) (*flags)[acc[prev]] = (u32)i + 1;
+            // with discard off a remainder chunk can be picked and this slot can run past the array
+            // (upstream writes out of bounds there: undefined); the oracle drops such writes
+            if (flags && acc[prev] < flags->size()) (*flags)[acc[prev]] = (u32)i + 1;
             acc[prev] += 1;
         }
     }

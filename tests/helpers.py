@@ -1,0 +1,137 @@
+"""Shared helpers of the test-suite (inputs, golden fixtures, a numpy emulation of the schedule)."""
+import hashlib
+import json
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+GOLDEN = os.path.join(HERE, "golden")
+
+V1_KEYS = ("new_indices_src", "part_pointers_cache", "column_index_cache", "part_cache_flagindex")
+V2_KEYS = ("uniqpart_column_index", "uniqpart_pointers", "part2Node_ptr", "part2Node_col")
+STEP_KEYS = ("part_ptr", "part2Node", "num_parts_per_node_acc", "intersect_count", "index_ordered", "index_picked")
+
+TOY_ADJ = {0: [3, 4, 5], 1: [3, 4, 5], 2: [3, 4, 5, 6], 3: [0, 1, 2, 7], 4: [0, 1, 2, 8], 5: [0, 1, 2, 9], 6: [2, 7],
+           7: [3, 6], 8: [4], 9: [5]}
+
+
+def toy_csr():
+    indptr = np.zeros(11, dtype=np.int32)
+    idx = []
+    for v in range(10):
+        idx += TOY_ADJ[v]
+        indptr[v + 1] = len(idx)
+    return indptr, np.array(idx, dtype=np.int32)
+
+
+def golden_small():
+    """{case: {"in": {...}, "out": {...}}} from tests/golden/plans_small.npz (written by the upstream builder)."""
+    z = np.load(os.path.join(GOLDEN, "plans_small.npz"))
+    cases = {}
+    for key in z.files:
+        name, kind, arr = key.split("/")
+        cases.setdefault(name, {"in": {}, "out": {}})[kind][arr] = z[key]
+    return cases
+
+
+def golden_digests():
+    with open(os.path.join(GOLDEN, "plans_digest.json")) as f:
+        return json.load(f)
+
+
+def sha(a):
+    return hashlib.sha256(np.ascontiguousarray(np.asarray(a, dtype=np.uint32)).tobytes()).hexdigest()
+
+
+def case_inputs(c):
+    i = c["in"]
+    ps, discard = int(i["ps_discard"][0]), bool(i["ps_discard"][1])
+    return i["indptr_dst"], i["indices_src"], i.get("indptr_src"), i.get("indices_dst"), ps, discard
+
+
+def emulate_schedule(ex, n, x, w_of, s_of, n_slots):
+    """Run the exported schedule (groups, segments, rows) in float64 numpy, checking its structure."""
+    feat = x.shape[1]
+    part = np.zeros((n_slots, feat))
+    written = np.zeros(n_slots, dtype=bool)
+    out = np.zeros((n, feat))
+    for ph in ("g", "s", "b"):
+        tp, nr, to, col = ex[ph + "_task_ptr"], ex[ph + "_task_nref"], ex[ph + "_task_out"], ex[ph + "_col"]
+        seen = set()
+        for t in range(len(to)):
+            acc = np.zeros(feat)
+            for i in range(tp[t], tp[t + 1]):
+                c = col[i]
+                if i < tp[t] + nr[t]:
+                    assert c >= n and written[c - n], "reference to a partial row that is not ready"
+                    acc += part[c - n]
+                else:
+                    assert 0 <= c < n
+                    acc += w_of(c) * x[c]
+            assert to[t] not in seen, "two writers for one output row"
+            seen.add(int(to[t]))
+            if ph == "b":
+                out[to[t]] = acc * (s_of(to[t]) if tp[t + 1] > tp[t] else 1.0)
+            else:
+                part[to[t]] = acc
+        if ph != "b":
+            for t in to:
+                written[t] = True
+        else:
+            assert seen == set(range(n)), "every destination row must be written exactly once"
+    return out
+
+
+def check_plan_invariants(ipd, isrc, ps, plan, discard=True):
+    """Structural facts every valid plan satisfies (independent of tie-breaking)."""
+    ipd = np.asarray(ipd).astype(np.int64)
+    isrc = np.asarray(isrc).astype(np.int64)
+    n, e = len(ipd) - 1, len(isrc)
+    pp, p2n = plan["part_ptr"].astype(np.int64), plan["part2Node"].astype(np.int64)
+    # P1: chunks tile every row in order, at most ps long, never crossing a row
+    assert pp[0] == 0 and pp[-1] == e and (np.diff(pp) >= 1).all() and (np.diff(pp) <= ps).all()
+    assert (np.diff(p2n) >= 0).all()
+    assert (ipd[p2n] <= pp[:-1]).all() and (pp[1:] <= ipd[p2n + 1]).all()
+    acc = plan["num_parts_per_node_acc"].astype(np.int64)
+    assert np.array_equal(acc, np.cumsum((np.diff(ipd) + ps - 1) // ps))
+    cnt = plan["intersect_count"].astype(np.int64)
+    picked = plan["index_picked"].astype(np.int64)
+    # P3: picked chunks are full, disjoint in sources, cnt >= 2 and non-increasing in pick order
+    used = set()
+    for p in picked:
+        srcs = isrc[pp[p]:pp[p + 1]]
+        if discard:
+            assert len(srcs) == ps
+        assert cnt[p] >= 2
+        assert used.isdisjoint(srcs.tolist())
+        used.update(srcs.tolist())
+    assert (np.diff(cnt[picked]) <= 0).all()
+    order = plan["index_ordered"].astype(np.int64)
+    assert np.array_equal(np.sort(order), np.arange(len(cnt))) and (np.diff(cnt[order]) <= 0).all()
+    if "uniqpart_pointers" not in plan:
+        return
+    # P5: expanding the v2 plan reproduces the edge multiset
+    uc, up = plan["uniqpart_column_index"].astype(np.int64), plan["uniqpart_pointers"].astype(np.int64)
+    dp, dc = plan["part2Node_ptr"].astype(np.int64), plan["part2Node_col"].astype(np.int64)
+    assert len(up) == len(dp)
+    src_l, dst_l = [], []
+    for w in range(len(up) - 1):
+        s = uc[up[w]:up[w + 1]]
+        d = dc[dp[w]:dp[w + 1]]
+        src_l.append(np.repeat(s, len(d)))
+        dst_l.append(np.tile(d, len(s)))
+    got = np.sort(np.concatenate(dst_l) * n + np.concatenate(src_l)) if src_l else np.empty(0, dtype=np.int64)
+    want = np.sort(np.repeat(np.arange(n), np.diff(ipd)) * n + isrc)
+    assert np.array_equal(got, want)
+    # P6: saved gathers
+    assert e - len(uc) == int(((cnt[picked] - 1) * np.diff(pp)[picked]).sum())
+    # P4: v1 rows are permutations; flagged chunks equal their cache rows
+    new = plan["new_indices_src"].astype(np.int64)
+    for v in range(n):
+        assert np.array_equal(np.sort(new[ipd[v]:ipd[v + 1]]), np.sort(isrc[ipd[v]:ipd[v + 1]]))
+    flag = plan["part_cache_flagindex"].astype(np.int64)
+    cp, cc = plan["part_pointers_cache"].astype(np.int64), plan["column_index_cache"].astype(np.int64)
+    for p in np.nonzero(flag)[0]:
+        k = flag[p] - 1
+        assert np.array_equal(new[pp[p]:pp[p + 1]], cc[cp[k]:cp[k + 1]])

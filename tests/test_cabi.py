@@ -1,0 +1,60 @@
+"""The C ABI: the library loads, exports every symbol include/rof.h declares, reports errors by code.
+No compute call is made here (no GPU)."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from artifact_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "rof.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(rof_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_is_built_in_tree_and_loads():
+    assert os.path.exists(_lib.LIB_PATH), "run `python -m artifact_amd.build`"
+    assert _lib.lib().rof_version() >= 1
+
+
+def test_every_declared_symbol_is_exported():
+    L = _lib.lib()
+    names = _declared()
+    assert len(names) >= 25
+    for name in names:
+        assert hasattr(L, name), f"{name} is declared in include/rof.h but not exported"
+    assert set(_lib.SYMBOLS) == set(names)
+
+
+def test_no_torch_types_in_signatures():
+    text = open(os.path.join(ROOT, "include", "rof.h")).read()
+    assert "torch" not in text.lower() and "at::" not in text and "#include <hip" not in text
+
+
+def test_error_codes_and_messages():
+    L = _lib.lib()
+    assert L.rof_strerror(0) == b"ok"
+    for code, word in ((-1, b"argument"), (-2, b"range"), (-3, b"alloc"), (-4, b"HIP"), (-5, b"state"),
+                       (-7, b"workspace")):
+        assert word in L.rof_strerror(code)
+    h = C.c_void_p()
+    assert L.rof_split_part(None, 0, 3, C.byref(h)) == -1
+    assert L.rof_plan_build(None, None, None, None, 0, 0, 3, 1, C.byref(h)) == -1
+    assert L.rof_layout_from_v2(None, None, None, None, 0, 0, 3, None, C.byref(h)) == -1
+    assert L.rof_aggregate(None, None, 0, 0, None, 0, 1, 1, None, 0, None) == -1
+    assert L.rof_layout_workspace_bytes(None, 4) == 0
+    assert L.rof_set_xcd_run(0, 1) == -1
+    with pytest.raises(_lib.RofError, match="invalid argument"):
+        _lib.check(-1)
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/librof.so")
+    with pytest.raises(_lib.RofError, match="no fallback"):
+        _lib.lib()

@@ -1,0 +1,64 @@
+"""The large workload (2.4M nodes, ~60M directed edges) at full size, checked through properties that
+do not need an oracle run of that size: exact integer sums, a float64 checksum of checksums, linearity,
+and agreement of the reuse path with the reuse-disabled path."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+from artifact_amd import reuse_search_ext as R            # noqa: E402
+from artifact_amd.graphgen import make_workload            # noqa: E402
+from artifact_amd.layout import Layout                     # noqa: E402
+
+
+@pytest.fixture(scope="module")
+def big():
+    ip, ix = make_workload("c4")
+    plan = R.build_plan(ip, ix, 3)
+    n = len(ip) - 1
+    args = (plan["uniqpart_column_index"], plan["uniqpart_pointers"], plan["part2Node_ptr"], plan["part2Node_col"], n, 3)
+    return ip, ix, n, Layout.from_v2(*args), Layout.from_v2(*args, disable_reuse=True)
+
+
+def test_full_size_properties(big):
+    ip, ix, n, reuse, plain = big
+    deg = np.diff(ip).astype(np.float32)
+    dev = "cuda"
+    # (1) unnormalised sum of all-ones features = in-degree, exactly (integers below 2^24)
+    ones = torch.ones((n, 4), device=dev)
+    got = reuse.aggregate(ones, normalized=False).cpu().numpy()
+    assert np.array_equal(got, np.repeat(deg[:, None], 4, axis=1))
+    # (2) checksum of checksums: sum_v out[v] = sum_u outdeg(u) * x[u]  (symmetric graph: outdeg = deg)
+    g = torch.Generator(device=dev).manual_seed(5)
+    xbuf = torch.randn((n, 48), device=dev, generator=g)
+    x = xbuf[:, :47]
+    out = reuse.aggregate(x, normalized=False, feat_dim=47)
+    lhs = out.double().sum(0).cpu().numpy()
+    rhs = (x.double() * torch.from_numpy(deg).to(dev).double()[:, None]).sum(0).cpu().numpy()
+    assert np.allclose(lhs, rhs, rtol=1e-6, atol=1e-2)
+    # (3) reuse path == reuse-disabled path (same kernels) on the normalised layer
+    degt = torch.from_numpy(deg).to(dev)
+    reuse.set_degrees(degt)
+    plain.set_degrees(degt)
+    a = reuse.aggregate(x, feat_dim=47)
+    b = plain.aggregate(x, feat_dim=47)
+    assert torch.allclose(a, b, rtol=1e-5, atol=2e-6)
+    # (4) linearity: agg(2x + 3y) = 2 agg(x) + 3 agg(y)
+    ybuf = torch.randn((n, 48), device=dev, generator=g)
+    y = ybuf[:, :47]
+    zbuf = 2 * xbuf + 3 * ybuf
+    lhs = reuse.aggregate(zbuf[:, :47], feat_dim=47)
+    rhs = 2 * a + 3 * reuse.aggregate(y, feat_dim=47)
+    assert torch.allclose(lhs, rhs, rtol=1e-4, atol=1e-5)
+    # (5) a random sample of rows against a float64 host evaluation
+    rows = np.random.default_rng(1).integers(0, n, 200)
+    xh = x.cpu().numpy().astype(np.float64)
+    r = 1.0 / np.sqrt(deg.astype(np.float64))
+    ah = a.cpu().numpy()
+    for v in rows:
+        nb = ix[ip[v]:ip[v + 1]]
+        want = r[v] * (xh[nb] * r[nb, None]).sum(0) if len(nb) else np.zeros(47)
+        mag = r[v] * (np.abs(xh[nb]) * r[nb, None]).sum(0) if len(nb) else np.zeros(47)
+        assert (np.abs(ah[v] - want) <= 1e-6 + 1e-5 * np.abs(want) + 1e-5 * mag).all(), v

@@ -1,0 +1,149 @@
+"""Host side of the device layout: lossless round trip to the upstream v2 tensors, agreement of the
+three input formats, and a numpy emulation of the execution schedule against the closed form."""
+import numpy as np
+import pytest
+
+from helpers import V2_KEYS, emulate_schedule, toy_csr
+
+from artifact_amd import reuse_search_ext as R
+from artifact_amd._lib import RofError
+from artifact_amd.graphgen import make_workload, rmat_csr
+from artifact_amd.layout import Layout
+
+
+def _v2(plan, n, ps, **o):
+    return Layout.from_v2(plan["uniqpart_column_index"], plan["uniqpart_pointers"], plan["part2Node_ptr"],
+                          plan["part2Node_col"], n, ps, **o)
+
+
+def _v1(plan, n, ps, **o):
+    return Layout.from_v1(plan["new_indices_src"], plan["part_ptr"], plan["part2Node"], plan["part_cache_flagindex"],
+                          plan["part_pointers_cache"], plan["column_index_cache"], n, ps, **o)
+
+
+@pytest.mark.parametrize("wl,sd,ps", [("c1", 3, 3), ("c1", 2, 2), ("c1", 3, 5), ("c3", 6, 2), ("c2", 6, 4)])
+def test_layout_round_trips_to_the_upstream_v2_plan_bit_exactly(wl, sd, ps):
+    ip, ix = make_workload(wl, sd)
+    n = len(ip) - 1
+    plan = R.build_plan(ip, ix, ps)
+    ex = _v2(plan, n, ps).export()
+    assert ex["canonical"]
+    for k in V2_KEYS:
+        assert np.array_equal(ex[k].view(np.uint32), plan[k]), k
+    # the canonical arrays: groups = picked parts with their consumers, residual = what is left per node
+    P = len(plan["index_picked"])
+    assert np.array_equal(ex["group_ptr"], plan["uniqpart_pointers"][:P + 1].view(np.int32))
+    assert np.array_equal(ex["group_dst"], plan["picked_dst"].view(np.int32))
+    assert ex["res_ptr"][-1] + ex["group_ptr"][-1] == len(plan["uniqpart_column_index"])
+    # v1 tensors describe the same plan and must give the same canonical arrays
+    ex1 = _v1(plan, n, ps).export()
+    for k in ("group_ptr", "group_col", "group_dst_ptr", "group_dst", "res_ptr", "res_col"):
+        assert np.array_equal(ex[k], ex1[k]), k
+
+
+def test_toy_layout_literal():
+    ip, ix = toy_csr()
+    plan = R.build_plan(ip, ix, 3)
+    ex = _v2(plan, 10, 3, min_consumers=2).export()
+    assert ex["group_ptr"].tolist() == [0, 3, 6] and ex["group_col"].tolist() == [3, 4, 5, 0, 1, 2]
+    assert ex["group_dst"].tolist() == [0, 1, 2, 3, 4, 5]
+    assert ex["res_ptr"].tolist() == [0, 0, 0, 1, 2, 3, 4, 6, 8, 9, 10]
+    assert ex["res_col"].tolist() == [6, 7, 8, 9, 2, 7, 3, 6, 4, 5]
+    # two partial-sum tasks, ten destination rows; rows 0..2 read partial row 0, rows 3..5 partial row 1
+    assert sorted(ex["g_task_out"].tolist()) == [0, 1]
+    rows = {int(o): ex["b_col"][ex["b_task_ptr"][t]:ex["b_task_ptr"][t + 1]].tolist()
+            for t, o in enumerate(ex["b_task_out"])}
+    assert rows[0] == [10] and rows[2] == [10, 6] and rows[3] == [11, 7] and rows[6] == [2, 7] and rows[9] == [5]
+
+
+OPTS = [dict(), dict(disable_reuse=True), dict(min_consumers=2), dict(min_consumers=-1), dict(hub_split=24, segment=8),
+        dict(hub_split=33, segment=32, min_consumers=2)]
+
+
+@pytest.mark.parametrize("opts", OPTS, ids=[str(o) for o in OPTS])
+def test_schedule_computes_the_closed_form(oracle, opts):
+    ip, ix = rmat_csr(400, 10, seed=77, self_loops=True)
+    n = len(ip) - 1
+    for ps in (2, 3):
+        plan = R.build_plan(ip, ix, ps)
+        lay = _v2(plan, n, ps, **opts)
+        ex, st = lay.export(), lay.stats()
+        x = np.random.default_rng(0).standard_normal((n, 3))
+        r = 1.0 / np.sqrt(np.diff(ip).astype(np.float64))
+        got = emulate_schedule(ex, n, x, lambda c: r[c], lambda v: r[v], st["partial_rows"])
+        assert np.allclose(got, oracle.closed_form(ip, ix, x), rtol=1e-12, atol=1e-12)
+        # bookkeeping used by the roofline report
+        nref = int(ex["g_task_nref"].sum() + ex["s_task_nref"].sum() + ex["b_task_nref"].sum())
+        total = len(ex["g_col"]) + len(ex["s_col"]) + len(ex["b_col"])
+        assert st["partial_reads"] == nref and st["gathered_rows"] == total - nref
+        assert st["edges"] == len(ix) and st["tasks_b"] == n
+        assert st["partial_rows"] == st["materialised_groups"] + st["hub_segments"]
+        if opts.get("disable_reuse"):
+            assert st["gathered_rows"] == len(ix) and st["materialised_groups"] == 0
+        if opts.get("min_consumers") == 2:                   # every group shared: the upstream saving (h:537-605)
+            cnt = plan["intersect_count"][plan["index_picked"]].astype(np.int64)
+            assert len(ix) - st["gathered_rows"] == ps * int((cnt - 1).sum())
+
+
+def test_long_tasks_come_first_and_short_tasks_are_sorted_inside_tiles():
+    ip, ix = make_workload("c1", 1)
+    n = len(ip) - 1
+    lay = Layout.from_csr(ip, ix)
+    ex, st = lay.export(), lay.stats()
+    lens = np.diff(ex["b_task_ptr"])
+    nw = st["wave_tasks_b"]
+    assert (lens[:nw] > 32).all() and (lens[nw:] <= 32).all() and (np.diff(lens[:nw]) <= 0).all()
+    assert sorted(ex["b_task_out"].tolist()) == list(range(n))
+    assert lens.max() <= 2048                                # longer rows were segmented
+
+
+def test_non_canonical_v2_input_is_still_executed_correctly(oracle):
+    ip, ix = rmat_csr(200, 8, seed=5)
+    n = len(ip) - 1
+    plan = R.build_plan(ip, ix, 3)
+    up, dp = plan["uniqpart_pointers"].astype(np.int64), plan["part2Node_ptr"].astype(np.int64)
+    uc, dc = plan["uniqpart_column_index"], plan["part2Node_col"]
+    perm = np.random.default_rng(1).permutation(len(up) - 1)                 # shuffle the unique parts
+    uc2 = np.concatenate([uc[up[w]:up[w + 1]] for w in perm])
+    dc2 = np.concatenate([dc[dp[w]:dp[w + 1]] for w in perm])
+    up2 = np.concatenate([[0], np.cumsum(np.diff(up)[perm])])
+    dp2 = np.concatenate([[0], np.cumsum(np.diff(dp)[perm])])
+    lay = Layout.from_v2(uc2, up2, dp2, dc2, n, 3)
+    ex, st = lay.export(), lay.stats()
+    assert not ex["canonical"]
+    x = np.random.default_rng(2).standard_normal((n, 2))
+    got = emulate_schedule(ex, n, x, lambda c: 1.0, lambda v: 1.0, st["partial_rows"])
+    assert np.allclose(got, oracle.closed_form(ip, ix, x, normalized=False), rtol=1e-12, atol=1e-12)
+
+
+def test_invalid_plan_tensors_are_rejected_on_the_host():
+    ip, ix = toy_csr()
+    plan = R.build_plan(ip, ix, 3)
+    bad = plan["uniqpart_column_index"].copy()
+    bad[0] = 10                                               # node id == N
+    with pytest.raises(RofError, match="out of range"):
+        Layout.from_v2(bad, plan["uniqpart_pointers"], plan["part2Node_ptr"], plan["part2Node_col"], 10, 3)
+    with pytest.raises(RofError, match="out of range"):
+        Layout.from_v2(plan["uniqpart_column_index"], plan["uniqpart_pointers"][::-1].copy(), plan["part2Node_ptr"],
+                       plan["part2Node_col"], 10, 3)
+    with pytest.raises(ValueError):
+        Layout.from_v2(plan["uniqpart_column_index"], plan["uniqpart_pointers"], plan["part2Node_ptr"][:-1],
+                       plan["part2Node_col"], 10, 3)
+    flag = plan["part_cache_flagindex"].copy()
+    flag[0] = 7                                               # only 2 cache rows exist
+    with pytest.raises(RofError, match="out of range"):
+        Layout.from_v1(plan["new_indices_src"], plan["part_ptr"], plan["part2Node"], flag,
+                       plan["part_pointers_cache"], plan["column_index_cache"], 10, 3)
+
+
+def test_algorithmic_bytes_formula():
+    ip, ix = toy_csr()
+    plan = R.build_plan(ip, ix, 3)
+    lay = _v2(plan, 10, 3, min_consumers=2)
+    f = 8
+    # 16 gathered rows, 6 partial reads, 2 partial rows, 10 nodes
+    assert lay.algorithmic_bytes(f) == 16 * (4 + 4 * f) + 6 * (4 + 4 * f) + 2 * 4 * f + 10 * (4 * f + 8) + 4 * 3
+    a, b = lay.launch_bytes(f)
+    assert a + b == lay.algorithmic_bytes(f) and a == 6 * (4 + 4 * f) + 2 * 4 * f + 4 * 3
+    plain = _v2(plan, 10, 3, disable_reuse=True)
+    assert plain.algorithmic_bytes(f) == 28 * (4 + 4 * f) + 10 * (4 * f + 8) + 4
