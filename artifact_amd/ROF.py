@@ -17,12 +17,12 @@ from collections import OrderedDict
 
 import torch
 
-from .layout import Layout
+from .layout import Layout, LayoutFamily
 
 __all__ = ["SAG", "GNNA_forward", "GNNA_backward", "reuse_forward_v1", "reuse_backward_v1", "reuse_forward_v2",
            "reuse_backward_v2", "clear_layout_cache"]
 
-_CACHE: "OrderedDict[tuple, Layout]" = OrderedDict()
+_CACHE: "OrderedDict[tuple, LayoutFamily]" = OrderedDict()
 _CACHE_MAX = 32
 
 
@@ -58,31 +58,43 @@ def _cached(key, build, keep):
     return lay
 
 
-def _host(t):
-    if t.dtype != torch.int32:
-        raise RuntimeError("plan tensors must be int32")
-    return t.detach().cpu().numpy()
+def _host(*tensors):
+    for t in tensors:
+        if t.dtype != torch.int32:
+            raise RuntimeError("plan tensors must be int32")
+    return [t.detach().cpu().numpy() for t in tensors]
 
 
 def _layout_parts(column_index, part_pointers, part2Node, num_nodes, part_size):
     key = _key("parts", part_size, column_index, part_pointers, part2Node)
-    return _cached(key, lambda: Layout.from_parts(_host(column_index), _host(part_pointers), _host(part2Node),
-                                                  num_nodes, part_size), (column_index, part_pointers, part2Node))
+
+    def build():
+        host = _host(column_index, part_pointers, part2Node)
+        return LayoutFamily(lambda lpr: Layout.from_parts(*host, num_nodes, part_size, lanes_per_row=lpr))
+
+    return _cached(key, build, (column_index, part_pointers, part2Node))
 
 
 def _layout_v1(column_index, part_pointers, part2Node, flag, cache_ptr, cache_col, num_nodes, part_size):
     key = _key("v1", part_size, column_index, part_pointers, part2Node, flag, cache_ptr, cache_col)
-    # every cache row is materialised (min_consumers=-1) so that slot g of the workspace is cache row g
-    return _cached(key, lambda: Layout.from_v1(_host(column_index), _host(part_pointers), _host(part2Node),
-                                               _host(flag), _host(cache_ptr), _host(cache_col), num_nodes, part_size,
-                                               min_consumers=-1),
-                   (column_index, part_pointers, part2Node, flag, cache_ptr, cache_col))
+
+    def build():
+        host = _host(column_index, part_pointers, part2Node, flag, cache_ptr, cache_col)
+        # every cache row is materialised (min_consumers=-1) so that slot g of the workspace is cache row g
+        return LayoutFamily(lambda lpr: Layout.from_v1(*host, num_nodes, part_size, min_consumers=-1,
+                                                       lanes_per_row=lpr))
+
+    return _cached(key, build, (column_index, part_pointers, part2Node, flag, cache_ptr, cache_col))
 
 
 def _layout_v2(ucol, uptr, dptr, dcol, num_nodes, part_size):
     key = _key("v2", part_size, ucol, uptr, dptr, dcol)
-    return _cached(key, lambda: Layout.from_v2(_host(ucol), _host(uptr), _host(dptr), _host(dcol), num_nodes,
-                                               part_size), (ucol, uptr, dptr, dcol))
+
+    def build():
+        host = _host(ucol, uptr, dptr, dcol)
+        return LayoutFamily(lambda lpr: Layout.from_v2(*host, num_nodes, part_size, lanes_per_row=lpr))
+
+    return _cached(key, build, (ucol, uptr, dptr, dcol))
 
 
 def _update(x, weight):
@@ -108,45 +120,47 @@ def _padded(t):
     return buf
 
 
-def _forward(layout, x, weight, degrees):
-    layout.set_degrees(degrees)
+def _forward(family, x, weight, degrees):
     tmp, f = _update(x, weight)
-    return layout.aggregate(tmp, normalized=True, feat_dim=f)
+    layout = family.get(f)
+    layout.set_degrees(degrees)
+    return layout.aggregate(tmp, normalized=True, feat_dim=f), layout
 
 
-def _backward(layout, d_output, X, W, degrees):
+def _backward(family, d_output, X, W, degrees):
     # upstream aggregates d_output with the same un-transposed plan (reuse_conv_kernel.cu:353-373,
     # 743-808, 1021-1041), then the two GEMMs (cu:382-383)
-    layout.set_degrees(degrees)
     f = d_output.shape[1]
+    layout = family.get(f)
+    layout.set_degrees(degrees)
     d_input_prime = layout.aggregate(_padded(d_output), normalized=True, feat_dim=f)
     d_input = torch.mm(d_input_prime, W.transpose(0, 1))
     d_weight = torch.mm(X.transpose(0, 1), d_input_prime)
-    return [d_input, d_weight]
+    return [d_input, d_weight], layout
 
 
 def SAG(input, row_pointers, column_index, degrees, part_pointers, part2Node, partSize, dimWorker, warpPerBlock):
     """Unnormalised sum aggregation of `input` itself (reuse_conv.cpp:132-155, kernel cu:123-196)."""
     _check(input=input, row_pointers=row_pointers, column_index=column_index, degrees=degrees,
            part_pointers=part_pointers, part2Node=part2Node)
-    lay = _layout_parts(column_index, part_pointers, part2Node, input.shape[0], partSize)
-    return lay.aggregate(_padded(input), normalized=False, feat_dim=input.shape[1])
+    fam = _layout_parts(column_index, part_pointers, part2Node, input.shape[0], partSize)
+    return fam.get(input.shape[1]).aggregate(_padded(input), normalized=False, feat_dim=input.shape[1])
 
 
 def GNNA_forward(input, weight, column_index, degrees, part_pointers, part2Node, partSize, dimWorker, warpPerBlock):
     """reuse_conv.cpp:158-176 -> [output]."""
     _check(input=input, weight=weight, column_index=column_index, degrees=degrees, part_pointers=part_pointers,
            part2Node=part2Node)
-    lay = _layout_parts(column_index, part_pointers, part2Node, input.shape[0], partSize)
-    return [_forward(lay, input, weight, degrees)]
+    fam = _layout_parts(column_index, part_pointers, part2Node, input.shape[0], partSize)
+    return [_forward(fam, input, weight, degrees)[0]]
 
 
 def GNNA_backward(d_output, X, W, column_index, degrees, part_pointers, part2Node, partSize, dimWorker, warpPerBlock):
     """reuse_conv.cpp:179-196 -> [d_input, d_weight]."""
     _check(d_output=d_output, X=X, W=W, column_index=column_index, degrees=degrees, part_pointers=part_pointers,
            part2Node=part2Node)
-    lay = _layout_parts(column_index, part_pointers, part2Node, X.shape[0], partSize)
-    return _backward(lay, d_output, X, W, degrees)
+    fam = _layout_parts(column_index, part_pointers, part2Node, X.shape[0], partSize)
+    return _backward(fam, d_output, X, W, degrees)[0]
 
 
 def _fill_cache(lay, part_result_cache, f):
@@ -168,9 +182,9 @@ def reuse_forward_v1(input, weight, column_index, degrees, part_pointers, part2N
     _check(input=input, weight=weight, column_index=column_index, degrees=degrees, part_pointers=part_pointers,
            part2Node=part2Node, part_result_cache=part_result_cache, part_cache_flagindex=part_cache_flagindex,
            part_pointers_cache=part_pointers_cache, column_index_cache=column_index_cache)
-    lay = _layout_v1(column_index, part_pointers, part2Node, part_cache_flagindex, part_pointers_cache,
+    fam = _layout_v1(column_index, part_pointers, part2Node, part_cache_flagindex, part_pointers_cache,
                      column_index_cache, input.shape[0], partSize)
-    out = _forward(lay, input, weight, degrees)
+    out, lay = _forward(fam, input, weight, degrees)
     _fill_cache(lay, part_result_cache, weight.shape[1])
     return [out]
 
@@ -181,21 +195,22 @@ def reuse_backward_v1(d_output, X, W, column_index, degrees, part_pointers, part
     _check(d_output=d_output, X=X, W=W, column_index=column_index, degrees=degrees, part_pointers=part_pointers,
            part2Node=part2Node, part_result_cache=part_result_cache, part_cache_flagindex=part_cache_flagindex,
            part_pointers_cache=part_pointers_cache, column_index_cache=column_index_cache)
-    lay = _layout_v1(column_index, part_pointers, part2Node, part_cache_flagindex, part_pointers_cache,
+    fam = _layout_v1(column_index, part_pointers, part2Node, part_cache_flagindex, part_pointers_cache,
                      column_index_cache, X.shape[0], partSize)
-    res = _backward(lay, d_output, X, W, degrees)
+    res, lay = _backward(fam, d_output, X, W, degrees)
     _fill_cache(lay, part_result_cache, d_output.shape[1])
     return res
 
 
 def reuse_forward_v2(input, weight, uniqpart_column_index, degrees, uniqpart_pointers, part2Node_ptr, part2Node_col,
                      partSize, dimWorker, warpPerBlock, layout=None):
-    """reuse_conv.cpp:288-314 -> [output].  `layout` (optional, not upstream) skips the cache lookup."""
+    """reuse_conv.cpp:288-314 -> [output].  `layout` (optional, not upstream): a LayoutFamily built from
+    host arrays, which skips the cache lookup and the device-to-host copy of the plan tensors."""
     _check(input=input, weight=weight, uniqpart_column_index=uniqpart_column_index, degrees=degrees,
            uniqpart_pointers=uniqpart_pointers, part2Node_ptr=part2Node_ptr, part2Node_col=part2Node_col)
-    lay = layout or _layout_v2(uniqpart_column_index, uniqpart_pointers, part2Node_ptr, part2Node_col, input.shape[0],
+    fam = layout or _layout_v2(uniqpart_column_index, uniqpart_pointers, part2Node_ptr, part2Node_col, input.shape[0],
                                partSize)
-    return [_forward(lay, input, weight, degrees)]
+    return [_forward(fam, input, weight, degrees)[0]]
 
 
 def reuse_backward_v2(d_output, X, W, uniqpart_column_index, degrees, uniqpart_pointers, part2Node_ptr, part2Node_col,
@@ -203,6 +218,6 @@ def reuse_backward_v2(d_output, X, W, uniqpart_column_index, degrees, uniqpart_p
     """reuse_conv.cpp:317-346 -> [d_input, d_weight]."""
     _check(d_output=d_output, X=X, W=W, uniqpart_column_index=uniqpart_column_index, degrees=degrees,
            uniqpart_pointers=uniqpart_pointers, part2Node_ptr=part2Node_ptr, part2Node_col=part2Node_col)
-    lay = layout or _layout_v2(uniqpart_column_index, uniqpart_pointers, part2Node_ptr, part2Node_col, X.shape[0],
+    fam = layout or _layout_v2(uniqpart_column_index, uniqpart_pointers, part2Node_ptr, part2Node_col, X.shape[0],
                                partSize)
-    return _backward(lay, d_output, X, W, degrees)
+    return _backward(fam, d_output, X, W, degrees)[0]

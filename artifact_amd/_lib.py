@@ -10,7 +10,7 @@ import os
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "librof.so")
+LIB_PATH = os.environ.get("ROF_LIBRARY") or os.path.join(_HERE, "librof.so")   # override: experiments only
 _lib = None
 
 # every symbol include/rof.h declares (checked by the CPU test-suite against the header text)
@@ -19,7 +19,7 @@ SYMBOLS = (
     "rof_part_intersect_count", "rof_part_intersect_lists", "rof_greedy_max_reuse", "rof_reorganize",
     "rof_transpose_csr", "rof_plan_build", "rof_layout_from_v2", "rof_layout_from_v1", "rof_layout_from_parts",
     "rof_layout_export", "rof_layout_stats", "rof_layout_upload", "rof_layout_set_degrees",
-    "rof_layout_workspace_bytes", "rof_layout_free", "rof_aggregate", "rof_aggregate_timed", "rof_set_xcd_run", "rof_aggregate_launch_times", "rof_device_copy",
+    "rof_layout_workspace_bytes", "rof_layout_free", "rof_aggregate", "rof_aggregate_timed", "rof_set_xcd_run", "rof_aggregate_launch_times", "rof_device_copy", "rof_set_lds_pad",
 )
 
 
@@ -29,7 +29,7 @@ class RofError(RuntimeError):
 
 class LayoutOpts(C.Structure):
     _fields_ = [("min_consumers", C.c_int32), ("disable_reuse", C.c_int32), ("hub_split", C.c_int32),
-                ("segment", C.c_int32), ("reserved", C.c_int32 * 4)]
+                ("segment", C.c_int32), ("lanes_per_row", C.c_int32), ("reserved", C.c_int32 * 3)]
 
 
 def lib():
@@ -69,6 +69,7 @@ def lib():
     L.rof_aggregate.argtypes = [vp, vp, ci, i64, vp, i64, ci, ci, vp, C.c_size_t, vp]
     L.rof_aggregate_timed.argtypes = [vp, vp, ci, i64, vp, i64, ci, ci, vp, C.c_size_t, vp, ci, C.POINTER(C.c_float)]
     L.rof_set_xcd_run.argtypes = [ci, ci]
+    L.rof_set_lds_pad.argtypes = [ci]
     L.rof_device_copy.argtypes = [vp, vp, C.c_size_t, vp]
     L.rof_aggregate_launch_times.argtypes = [vp, vp, ci, i64, vp, i64, ci, ci, vp, C.c_size_t, vp, ci,
                                              C.POINTER(C.c_float * 2)]

@@ -38,6 +38,10 @@ namespace {
 
 thread_local char g_dev_err[256] = "";
 
+// process-wide launch tuning (rof_set_xcd_run, rof_set_lds_pad)
+int g_xcd_run_a = 1, g_xcd_run_b = 16;
+int g_lds_pad = 0;   // bytes of unused LDS requested per workgroup: caps the workgroups resident per CU
+
 #define HIP_TRY(expr)                                                                  \
     do {                                                                               \
         hipError_t e_ = (expr);                                                        \
@@ -66,24 +70,41 @@ struct AggArgs {
     int32_t vec_store;         // output rows allow aligned 16-byte stores
 };
 
+// Row gathers a lane group keeps in flight.  Measured on MI355X with all eight wave slots per SIMD
+// occupied: 2 beats 4 by ~10 % on the miss-dominated workloads (more outstanding gathers per CU slow the
+// L1/L2 miss path down) and loses ~2 % where gathers hit in L2; 8 loses everywhere.
+#ifndef ROF_UNROLL
+#define ROF_UNROLL 2
+#endif
+#ifndef ROF_MIN_BLOCKS
+#define ROF_MIN_BLOCKS 1
+#endif
 constexpr int kWavesPerBlock = 4;
 constexpr int kXcds = 8;
 
 template <typename XT, int VEC>
 struct RowLoad;
 
+#ifdef ROF_NT_LOADS
+#define ROF_LD16(T, p) __builtin_nontemporal_load(reinterpret_cast<const T *>(p))
+#else
+#define ROF_LD16(T, p) (*reinterpret_cast<const T *>(p))
+#endif
+typedef float rof_f4 __attribute__((ext_vector_type(4)));
+typedef unsigned int rof_u4 __attribute__((ext_vector_type(4)));
+
 template <>
 struct RowLoad<float, 4> {
     static __device__ __forceinline__ void load(const float *p, float (&v)[4]) {
-        float4 t = *reinterpret_cast<const float4 *>(p);
+        rof_f4 t = ROF_LD16(rof_f4, p);
         v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
     }
 };
 template <>
 struct RowLoad<float, 8> {
     static __device__ __forceinline__ void load(const float *p, float (&v)[8]) {
-        float4 t = *reinterpret_cast<const float4 *>(p);
-        float4 u = *reinterpret_cast<const float4 *>(p + 4);
+        rof_f4 t = ROF_LD16(rof_f4, p);
+        rof_f4 u = ROF_LD16(rof_f4, p + 4);
         v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
         v[4] = u.x; v[5] = u.y; v[6] = u.z; v[7] = u.w;
     }
@@ -96,7 +117,7 @@ struct RowLoad<float, 1> {
 template <>
 struct RowLoad<uint16_t, 8> {
     static __device__ __forceinline__ void load(const uint16_t *p, float (&v)[8]) {
-        uint4 t = *reinterpret_cast<const uint4 *>(p);
+        rof_u4 t = ROF_LD16(rof_u4, p);
         v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u);
         v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
         v[4] = __uint_as_float(t.z << 16); v[5] = __uint_as_float(t.z & 0xffff0000u);
@@ -110,27 +131,44 @@ struct RowLoad<uint16_t, 1> {
     }
 };
 
+// Address of this lane's slice of gathered row `c`.  xb / pb already include the lane's column
+// offset; ld in bytes.  With DUAL ids >= nsplit name partial-sum rows (pb), chosen by selects, not
+// branches.  OFF32: all byte offsets fit 32 bits and row ids fit 24 (checked on the host), so one
+// 24-bit multiply and a 32-bit add replace the 64-bit multiply.
+template <bool DUAL, bool OFF32>
+__device__ __forceinline__ const char *row_ptr(int32_t c, const char *xb, uint32_t xld, const char *pb, uint32_t pld,
+                                               int32_t nsplit, int32_t bias) {
+    uint32_t r = (uint32_t)(c - bias), l = xld;
+    const char *b = xb;
+    if (DUAL) {
+        const bool p = c >= nsplit;
+        r = p ? (uint32_t)(c - nsplit) : r;
+        l = p ? pld : xld;
+        b = p ? pb : xb;
+    }
+    if (OFF32) return b + __umul24(r, l);
+    return b + (uint64_t)r * l;
+}
+
 // Sum the entries [beg, end) of one task into acc.  WAVE: all lane groups of the wavefront share
 // the task (beg/end wave-uniform) and take every G-th entry; otherwise each lane group owns its
-// task.  ST is the element type of the source rows.  With DUAL (fp32 features only) ids >= nsplit
-// are taken from the partial-sum rows instead, chosen per entry by a pointer select, so a task
-// that mixes both kinds still runs one loop with one fetch of ids and weights per chunk.
-template <typename ST, int VEC, int LPR, bool WAVE, bool DUAL>
-__device__ __forceinline__ void gather_sum(const ST *__restrict__ src, int64_t ld, const float *__restrict__ part,
-                                           int64_t ldp, int32_t nsplit, int32_t bias,
-                                           const int32_t *__restrict__ col, const float *__restrict__ w,
-                                           int32_t beg, int32_t end, int lane, int sub, int li, int cbase, bool act,
-                                           float (&acc)[VEC]) {
+// task.  ST is the element type of the source rows.  Blocks of U entries that are complete for every
+// lane group run without any per-entry predicate; ragged ends are predicated entry by entry.
+template <typename ST, int VEC, int LPR, bool WAVE, bool DUAL, bool OFF32>
+__device__ __forceinline__ void gather_sum(const char *xb, uint32_t xld, const char *pb, uint32_t pld, int32_t nsplit,
+                                           int32_t bias, const int32_t *__restrict__ col,
+                                           const float *__restrict__ w, int32_t beg, int32_t end, int lane, int sub,
+                                           int li, bool act, float (&acc)[VEC]) {
     constexpr int G = 64 / LPR;
-    constexpr int U = LPR >= 4 ? 4 : LPR;
+    constexpr int U = LPR >= ROF_UNROLL ? ROF_UNROLL : LPR;   // row gathers in flight per lane group
     constexpr int CH = WAVE ? 64 : LPR;     // entries fetched per step by the wave / by the lane group
     for (int32_t base = beg; __any(base < end); base += CH) {
         const int32_t mine = base + (WAVE ? lane : li);
-        int32_t mycol = 0;
-        float myw = 1.0f;
+        int32_t mycol = bias;               // past the end: row 0 of the source, weight 0
+        float myw = 0.0f;
         if (mine < end) {
             mycol = col[mine];
-            if (w) myw = w[mine];
+            myw = w ? w[mine] : 1.0f;
         }
 #pragma unroll
         for (int j0 = 0; j0 < LPR; j0 += U) {
@@ -138,42 +176,56 @@ __device__ __forceinline__ void gather_sum(const ST *__restrict__ src, int64_t l
             if (!__any(base + first < end)) break;
             int32_t c[U];
             float wt[U];
-            bool ok[U];
-            float v[U][VEC];
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 const int slot = WAVE ? (j0 + u) * G + sub : (j0 + u);          // entry of the chunk
                 const int from = WAVE ? slot : sub * LPR + slot;                // lane that fetched it
                 c[u] = __shfl(mycol, from);
                 wt[u] = __shfl(myw, from);
-                ok[u] = act && (base + slot < end);
             }
+            const int last = WAVE ? (j0 + U - 1) * G + sub : (j0 + U - 1);
+            const bool full = __all(base + last < end);
+            if (act) {
+                float v[U][VEC];
+                if (full) {
 #pragma unroll
-            for (int u = 0; u < U; ++u)
-                if (ok[u]) {
-                    if (DUAL) {
-                        const bool p = c[u] >= nsplit;
-                        const ST *row = p ? reinterpret_cast<const ST *>(part) + (int64_t)(c[u] - nsplit) * ldp
-                                          : src + (int64_t)c[u] * ld;
-                        RowLoad<ST, VEC>::load(row + cbase, v[u]);
-                    } else {
-                        RowLoad<ST, VEC>::load(src + (int64_t)(c[u] - bias) * ld + cbase, v[u]);
+                    for (int u = 0; u < U; ++u)
+                        RowLoad<ST, VEC>::load(
+                            reinterpret_cast<const ST *>(row_ptr<DUAL, OFF32>(c[u], xb, xld, pb, pld, nsplit, bias)),
+                            v[u]);
+#pragma unroll
+                    for (int u = 0; u < U; ++u)
+#pragma unroll
+                        for (int k = 0; k < VEC; ++k) acc[k] = fmaf(wt[u], v[u][k], acc[k]);
+                } else {
+                    // ragged end of a task: gather only the entries that exist (a dummy gather of one
+                    // fixed row from every lane group would pile onto a single L2 channel)
+                    bool ok[U];
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        const int slot = WAVE ? (j0 + u) * G + sub : (j0 + u);
+                        ok[u] = base + slot < end;
+                        if (ok[u])
+                            RowLoad<ST, VEC>::load(reinterpret_cast<const ST *>(
+                                                       row_ptr<DUAL, OFF32>(c[u], xb, xld, pb, pld, nsplit, bias)),
+                                                   v[u]);
                     }
-                }
 #pragma unroll
-            for (int u = 0; u < U; ++u)
-                if (ok[u]) {
+                    for (int u = 0; u < U; ++u)
+                        if (ok[u]) {
 #pragma unroll
-                    for (int k = 0; k < VEC; ++k) acc[k] = fmaf(wt[u], v[u][k], acc[k]);
+                            for (int k = 0; k < VEC; ++k) acc[k] = fmaf(wt[u], v[u][k], acc[k]);
+                        }
                 }
+            }
         }
     }
 }
 
 // PHASE 0: the partial-sum launches (no scaling); PHASE 1: the destination-row launch.  Same code; the
 // parameter only gives them distinct kernel names in profiles.
-template <typename XT, int VEC, int LPR, int PHASE>
-__global__ __launch_bounds__(256) void rof_rows_kernel(AggArgs a) {
+template <typename XT, int VEC, int LPR, int PHASE, bool OFF32>
+__global__ __launch_bounds__(256, ROF_MIN_BLOCKS) void rof_rows_kernel(AggArgs a) {
     constexpr int G = 64 / LPR;
     // XCD-aware renumbering: the hardware deals workgroup ids round-robin to the 8 XCDs; give each
     // XCD runs of `xcd_run` consecutive logical workgroups instead of every 8th one.
@@ -186,7 +238,6 @@ __global__ __launch_bounds__(256) void rof_rows_kernel(AggArgs a) {
     const int lane = threadIdx.x & 63;
     const int sub = lane / LPR, li = lane % LPR;
     const int gw = logical * kWavesPerBlock + (threadIdx.x >> 6);
-    const XT *x = reinterpret_cast<const XT *>(a.x);
 
     int32_t t, beg = 0, end = 0, mid = 0;
     bool valid;
@@ -203,26 +254,28 @@ __global__ __launch_bounds__(256) void rof_rows_kernel(AggArgs a) {
         end = a.task_ptr[t + 1];
         mid = beg + a.task_nref[t];
     }
+    const uint32_t xld = (uint32_t)(a.ldx * (int64_t)sizeof(XT)), pld = (uint32_t)(a.ldp * 4);
 
     for (int c0 = 0; c0 < a.feat; c0 += LPR * VEC) {
         const int cbase = c0 + li * VEC;
         const bool act = cbase < a.feat;
+        const char *xb = reinterpret_cast<const char *>(a.x) + (size_t)cbase * sizeof(XT);
+        const char *pb = reinterpret_cast<const char *>(a.part) + (size_t)cbase * 4;
         float acc[VEC];
 #pragma unroll
         for (int k = 0; k < VEC; ++k) acc[k] = 0.0f;
 
         constexpr bool kF32 = sizeof(XT) == 4;   // fp32 features: partial rows have the same element type
-        constexpr bool kRefs = true;   // segments of long rows may reference group rows too
         if (wave_mode) {
-            if (kF32 || !kRefs) {
-                gather_sum<XT, VEC, LPR, true, kRefs>(x, a.ldx, a.part, a.ldp, a.nsplit, 0, a.col, a.w, beg, end, lane,
-                                                      sub, li, cbase, act, acc);
+            if (kF32) {
+                gather_sum<XT, VEC, LPR, true, true, OFF32>(xb, xld, pb, pld, a.nsplit, 0, a.col, a.w, beg, end, lane,
+                                                            sub, li, act, acc);
             } else {
                 if (mid > beg)
-                    gather_sum<float, VEC, LPR, true, false>(a.part, a.ldp, nullptr, 0, 0, a.nsplit, a.col, a.w, beg,
-                                                             mid, lane, sub, li, cbase, act, acc);
-                gather_sum<XT, VEC, LPR, true, false>(x, a.ldx, nullptr, 0, 0, 0, a.col, a.w, mid, end, lane, sub, li,
-                                                      cbase, act, acc);
+                    gather_sum<float, VEC, LPR, true, false, OFF32>(pb, pld, nullptr, 0, 0, a.nsplit, a.col, a.w, beg,
+                                                                    mid, lane, sub, li, act, acc);
+                gather_sum<XT, VEC, LPR, true, false, OFF32>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, mid, end, lane, sub,
+                                                             li, act, acc);
             }
 #pragma unroll
             for (int off = LPR; off < 64; off <<= 1) {
@@ -230,15 +283,15 @@ __global__ __launch_bounds__(256) void rof_rows_kernel(AggArgs a) {
                 for (int k = 0; k < VEC; ++k) acc[k] += __shfl_xor(acc[k], off);
             }
         } else {
-            if (kF32 || !kRefs) {
-                gather_sum<XT, VEC, LPR, false, kRefs>(x, a.ldx, a.part, a.ldp, a.nsplit, 0, a.col, a.w, beg, end, lane,
-                                                       sub, li, cbase, act, acc);
+            if (kF32) {
+                gather_sum<XT, VEC, LPR, false, true, OFF32>(xb, xld, pb, pld, a.nsplit, 0, a.col, a.w, beg, end, lane,
+                                                             sub, li, act, acc);
             } else {
                 if (__any(mid > beg))
-                    gather_sum<float, VEC, LPR, false, false>(a.part, a.ldp, nullptr, 0, 0, a.nsplit, a.col, a.w, beg,
-                                                              mid, lane, sub, li, cbase, act, acc);
-                gather_sum<XT, VEC, LPR, false, false>(x, a.ldx, nullptr, 0, 0, 0, a.col, a.w, mid, end, lane, sub, li,
-                                                       cbase, act, acc);
+                    gather_sum<float, VEC, LPR, false, false, OFF32>(pb, pld, nullptr, 0, 0, a.nsplit, a.col, a.w, beg,
+                                                                     mid, lane, sub, li, act, acc);
+                gather_sum<XT, VEC, LPR, false, false, OFF32>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, mid, end, lane, sub,
+                                                              li, act, acc);
             }
         }
 
@@ -288,7 +341,7 @@ __global__ void rof_copy_kernel(const float4 *__restrict__ src, float4 *__restri
     for (; i < n16; i += stride) dst[i] = src[i];
 }
 
-template <typename XT, int VEC, int PHASE>
+template <typename XT, int VEC, int PHASE, bool OFF32>
 int launch_lpr(const AggArgs &a0, int lpr, hipStream_t st) {
     AggArgs a = a0;
     const int g = 64 / lpr;
@@ -300,23 +353,31 @@ int launch_lpr(const AggArgs &a0, int lpr, hipStream_t st) {
     const int64_t grid = (a.n_blocks + span - 1) / span * span;
     dim3 gr((unsigned)grid), bl(64 * kWavesPerBlock);
     switch (lpr) {
-        case 4: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 4, PHASE>), gr, bl, 0, st, a); break;
-        case 8: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 8, PHASE>), gr, bl, 0, st, a); break;
-        case 16: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 16, PHASE>), gr, bl, 0, st, a); break;
-        case 32: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 32, PHASE>), gr, bl, 0, st, a); break;
-        default: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 64, PHASE>), gr, bl, 0, st, a); break;
+        case 4: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 4, PHASE, OFF32>), gr, bl, g_lds_pad, st, a); break;
+        case 8: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 8, PHASE, OFF32>), gr, bl, g_lds_pad, st, a); break;
+        case 16: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 16, PHASE, OFF32>), gr, bl, g_lds_pad, st, a); break;
+        case 32: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 32, PHASE, OFF32>), gr, bl, g_lds_pad, st, a); break;
+        default: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 64, PHASE, OFF32>), gr, bl, g_lds_pad, st, a); break;
     }
     HIP_TRY(hipGetLastError());
     return ROF_OK;
 }
 
+// off32: every byte offset into the feature matrix and into the partial-sum workspace fits 32 bits and
+// every row id fits 24 bits, so the kernels may use the short address arithmetic.
 template <int PHASE>
-int launch_phase(const AggArgs &a, int dtype, int vec, hipStream_t st) {
+int launch_phase(const AggArgs &a, int dtype, int vec, bool off32, hipStream_t st) {
     int need = (a.feat + vec - 1) / vec, lpr = 4;
     while (lpr < need && lpr < 64) lpr <<= 1;
-    if (dtype == ROF_F32)
-        return vec == 4 ? launch_lpr<float, 4, PHASE>(a, lpr, st) : launch_lpr<float, 1, PHASE>(a, lpr, st);
-    return vec == 8 ? launch_lpr<uint16_t, 8, PHASE>(a, lpr, st) : launch_lpr<uint16_t, 1, PHASE>(a, lpr, st);
+    if (dtype == ROF_F32) {
+        if (vec == 4)
+            return off32 ? launch_lpr<float, 4, PHASE, true>(a, lpr, st) : launch_lpr<float, 4, PHASE, false>(a, lpr, st);
+        return launch_lpr<float, 1, PHASE, false>(a, lpr, st);
+    }
+    if (vec == 8)
+        return off32 ? launch_lpr<uint16_t, 8, PHASE, true>(a, lpr, st)
+                     : launch_lpr<uint16_t, 8, PHASE, false>(a, lpr, st);
+    return launch_lpr<uint16_t, 1, PHASE, false>(a, lpr, st);
 }
 
 int upload_phase(const rof_phase_host &h, rof_phase_dev &d, bool with_scale, hipStream_t st, int64_t *bytes) {
@@ -358,7 +419,7 @@ void free_phase(rof_phase_dev &d) {
 
 inline int64_t round_up(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
 
-int g_xcd_run_a = 1, g_xcd_run_b = 16;
+
 
 }  // namespace
 
@@ -387,6 +448,12 @@ const char *rof_strerror(int status) {
 int rof_version(void) { return 1; }
 
 // Tuning knob used by the benchmark sweeps: consecutive workgroups per XCD for launch 1 / launch 2.
+int rof_set_lds_pad(int bytes) {
+    if (bytes < 0 || bytes > 64 * 1024) return ROF_ERR_ARG;
+    g_lds_pad = bytes;
+    return ROF_OK;
+}
+
 int rof_set_xcd_run(int run_a, int run_b) {
     if (run_a < 1 || run_b < 1 || run_a > 4096 || run_b > 4096) return ROF_ERR_ARG;
     g_xcd_run_a = run_a;
@@ -468,8 +535,10 @@ static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64
     const int wide = x_dtype == ROF_F32 ? 4 : 8;
     const bool aligned = (ldx % wide == 0) && (((uintptr_t)x) % 16 == 0);
     const int vec = aligned ? wide : 1;
-    (void)esz;
     const int64_t ldp = round_up(feat, 8);
+    const int64_t rows_x = L->n, rows_p = L->n_slots;
+    const bool off32 = rows_x < (1 << 24) && rows_p < (1 << 24) && ldx * esz < (1 << 24) && ldp * 4 < (1 << 24) &&
+                       (rows_x + 1) * ldx * esz < ((int64_t)1 << 32) && (rows_p + 1) * ldp * 4 < ((int64_t)1 << 32);
 
     AggArgs a;
     memset(&a, 0, sizeof(a));
@@ -497,7 +566,7 @@ static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64
         a.n_tasks = d.n_tasks;
         a.xcd_run = g_xcd_run_a;
         a.vec_store = 1;
-        if ((rc = launch_phase<0>(a, x_dtype, vec, st))) return rc;
+        if ((rc = launch_phase<0>(a, x_dtype, vec, off32, st))) return rc;
     }
     if (L->db.n_tasks && (launches & 2)) {   // last launch: destination rows
         a.task_ptr = L->db.task_ptr;
@@ -512,7 +581,7 @@ static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64
         a.n_tasks = L->db.n_tasks;
         a.xcd_run = g_xcd_run_b;
         a.vec_store = (ldo % 4 == 0) && (((uintptr_t)out) % 16 == 0);
-        if ((rc = launch_phase<1>(a, x_dtype, vec, st))) return rc;
+        if ((rc = launch_phase<1>(a, x_dtype, vec, off32, st))) return rc;
     }
     return ROF_OK;
 }

@@ -22,8 +22,12 @@ namespace {
 typedef std::vector<int32_t> ivec;
 
 const int32_t kShortRow = 32;        // tasks up to this many entries share a wavefront
-const int32_t kHubSplitDefault = 2048;
-const int32_t kSegmentDefault = 512;
+// Default cut for long rows, per lane group of the kernel that will run the layout (G = 64 / lanes per
+// row): a wavefront works through a task G entries at a time with a few gathers in flight, so a task of
+// hub_split entries is a serial chain of hub_split / (4 G) memory round trips.  The cut is kept below
+// ~1/1000 of all entries so that the longest chain stays short against the whole launch on small graphs.
+const int32_t kHubSplitPerGroupMax = 1024;
+const int32_t kHubSplitPerGroupMin = 64;
 const int32_t kTileRows = 4096;      // short tasks are length-sorted inside tiles of this many rows
 
 bool ptr_ok(const int32_t *p, int64_t n, int64_t *total) {
@@ -119,8 +123,16 @@ void finalize_phase(const TaskList &tl, int64_t tile_rows, rof_phase_host &ph) {
 int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     const int32_t n = L->n;
     const int64_t G = (int64_t)L->group_ptr.size() - 1;
-    const int32_t hub_split = (o && o->hub_split > 0) ? o->hub_split : kHubSplitDefault;
-    const int32_t segment = (o && o->segment > 0) ? o->segment : kSegmentDefault;
+    int32_t lpr = (o && o->lanes_per_row > 0) ? o->lanes_per_row : 16;
+    if (lpr > 64) lpr = 64;
+    const int32_t groups = std::max(1, 64 / lpr);
+    const int64_t total = (int64_t)L->res_col.size() + (int64_t)L->group_dst.size();
+    const int64_t auto_split = std::max<int64_t>((int64_t)kHubSplitPerGroupMin * groups,
+                                                 std::min<int64_t>((int64_t)kHubSplitPerGroupMax * groups, total / 1024));
+    const int32_t hub_split = (o && o->hub_split > 0) ? o->hub_split : (int32_t)auto_split;
+    const int32_t segment = (o && o->segment > 0) ? o->segment : std::max(16, hub_split / 4);
+    L->hub_split = hub_split;
+    L->segment = segment;
     const bool disable = o && o->disable_reuse;
     const int32_t min_consumers = o ? o->min_consumers : 0;
 

@@ -39,6 +39,7 @@ struct rof_layout {
     std::vector<int32_t> group_ptr, group_col, group_dst_ptr, group_dst, res_ptr, res_col;
     // schedule
     rof_phase_host g, s, b;   // g: shared groups; s: segments of long rows (may read g's rows); b: destination rows
+    int32_t hub_split = 0, segment = 0;
     int64_t n_slots = 0;      // rows of the partial-sum workspace
     int64_t n_materialised = 0, n_segments = 0, gathered_rows = 0, partial_reads = 0, gathered_before_rows = 0;
     // device copies

@@ -25,13 +25,45 @@ EXPORT_NAMES = ("group_ptr", "group_col", "group_dst_ptr", "group_dst", "res_ptr
                 "b_task_ptr", "b_task_nref", "b_task_out", "b_col")
 
 
-def _opts(min_consumers=0, disable_reuse=False, hub_split=0, segment=0):
+def lanes_per_row(feat_dim, bf16=False):
+    """Lanes one gathered row occupies in the kernel: smallest power of two >= ceil(F / elements per
+    16-byte load), clamped to 4..64 (mirrors the dispatch in csrc/agg_kernels.hip)."""
+    need = -(-int(feat_dim) // (8 if bf16 else 4))
+    lpr = 4
+    while lpr < need and lpr < 64:
+        lpr <<= 1
+    return lpr
+
+
+def _opts(min_consumers=0, disable_reuse=False, hub_split=0, segment=0, lanes_per_row=0):
     o = LayoutOpts()
     o.min_consumers = int(min_consumers)
     o.disable_reuse = int(bool(disable_reuse))
     o.hub_split = int(hub_split)
     o.segment = int(segment)
+    o.lanes_per_row = int(lanes_per_row)
     return o
+
+
+class LayoutFamily:
+    """Layouts of one plan, one per lanes-per-row class: how finely long rows are segmented depends on
+    how many rows a wavefront gathers at once, i.e. on the feature width it will be used with."""
+
+    def __init__(self, build):
+        self._build = build            # callable(lanes_per_row) -> Layout
+        self._by_lpr = {}
+
+    def get(self, feat_dim, bf16=False):
+        lpr = lanes_per_row(feat_dim, bf16)
+        lay = self._by_lpr.get(lpr)
+        if lay is None:
+            lay = self._by_lpr[lpr] = self._build(lpr)
+        return lay
+
+    def close(self):
+        for lay in self._by_lpr.values():
+            lay.close()
+        self._by_lpr.clear()
 
 
 class Layout:

@@ -15,7 +15,7 @@ import torch
 
 from . import ROF
 from . import reuse_search_ext
-from .layout import Layout
+from .layout import Layout, LayoutFamily
 
 __all__ = ["ROF_GCNConvFunc", "ROF_GCNConv", "ROF_GINConv", "ROF_inputInfo", "build_input_info"]
 
@@ -47,7 +47,7 @@ class ROF_inputInfo:
         self.part2Node_col = part2Node_col
         self.dimWorker = 0
         self.part_result_cache = None
-        self.layouts = {}   # kernel_type -> Layout built from host arrays (skips the device->host round trip)
+        self.layouts = {}   # kernel_type -> LayoutFamily built from host arrays (skips the device->host round trip)
 
     def to(self, device):
         for name in _TENSOR_FIELDS:
@@ -92,8 +92,9 @@ def build_input_info(indptr, indices, part_size=3, device="cuda", warps_per_bloc
                          t(plan["column_index_cache"]), t(plan["uniqpart_column_index"]), t(plan["uniqpart_pointers"]),
                          t(plan["part2Node_ptr"]), t(plan["part2Node_col"]))
     if torch.device(device).type == "cuda":
-        info.layouts["ROF_v2"] = Layout.from_v2(plan["uniqpart_column_index"], plan["uniqpart_pointers"],
-                                                plan["part2Node_ptr"], plan["part2Node_col"], n, part_size)
+        info.layouts["ROF_v2"] = LayoutFamily(lambda lpr: Layout.from_v2(
+            plan["uniqpart_column_index"], plan["uniqpart_pointers"], plan["part2Node_ptr"], plan["part2Node_col"], n,
+            part_size, lanes_per_row=lpr))
     info.plan = plan
     return info
 
@@ -205,14 +206,14 @@ class _SumAggregate(torch.autograd.Function):
     gradient because the graphs are symmetric (the assumption upstream makes for GCN as well)."""
 
     @staticmethod
-    def forward(ctx, x, layout):
-        ctx.layout = layout
-        return layout.aggregate(ROF._padded(x.contiguous()), normalized=False, feat_dim=x.shape[1])
+    def forward(ctx, x, family):
+        ctx.family = family
+        return family.get(x.shape[1]).aggregate(ROF._padded(x.contiguous()), normalized=False, feat_dim=x.shape[1])
 
     @staticmethod
     def backward(ctx, grad):
         g = grad.contiguous()
-        return ctx.layout.aggregate(ROF._padded(g), normalized=False, feat_dim=g.shape[1]), None
+        return ctx.family.get(g.shape[1]).aggregate(ROF._padded(g), normalized=False, feat_dim=g.shape[1]), None
 
 
 class ROF_GINConv(torch.nn.Module):

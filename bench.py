@@ -104,6 +104,10 @@ def main():
     ap.add_argument("--xcd-run", type=int, default=0)
     ap.add_argument("--hub-split", type=int, default=0, help="layout tuning: rows longer than this are segmented")
     ap.add_argument("--segment", type=int, default=0, help="layout tuning: entries per segment")
+    ap.add_argument("--min-consumers", type=int, default=0, help="layout tuning: share groups with >= this many consumers")
+    ap.add_argument("--fold-sources", type=int, default=0,
+                    help="experiment: gather from source id %% K instead (all gathers hit cache); changes the result")
+    ap.add_argument("--lds-pad", type=int, default=-1, help="launch tuning: unused LDS bytes per workgroup")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB rof_copy_kernel launch (reference transfer for profiler byte counters)")
     args = ap.parse_args()
@@ -115,13 +119,15 @@ def main():
 
     from artifact_amd import _lib
     from artifact_amd.graphgen import features
-    from artifact_amd.layout import Layout
+    from artifact_amd.layout import Layout, lanes_per_row
 
     L = _lib.lib()   # raises if the HIP library is missing
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
     if args.xcd_run:
         _lib.check(L.rof_set_xcd_run(1, args.xcd_run))
+    if args.lds_pad >= 0:
+        _lib.check(L.rof_set_lds_pad(args.lds_pad))
     dev = torch.device("cuda:0")
     name, ps = args.workload, args.part_size
     feat = args.feat or FEAT[name]
@@ -144,11 +150,15 @@ def main():
         x32 = x.to(torch.float32).cpu().numpy()
     in_bytes = 2 if bf16 else 4
 
+    lpr = lanes_per_row(feat, bf16)
+    if args.fold_sources:
+        d["uniqpart_column_index"] = (d["uniqpart_column_index"] % args.fold_sources).astype(np.uint32)
     t0 = time.time()
     reuse = Layout.from_v2(d["uniqpart_column_index"], d["uniqpart_pointers"], d["part2Node_ptr"], d["part2Node_col"],
-                           n, ps, hub_split=args.hub_split, segment=args.segment)
+                           n, ps, hub_split=args.hub_split, segment=args.segment, lanes_per_row=lpr,
+                           min_consumers=args.min_consumers)
     plain = Layout.from_v2(d["uniqpart_column_index"], d["uniqpart_pointers"], d["part2Node_ptr"], d["part2Node_col"],
-                           n, ps, disable_reuse=True, hub_split=args.hub_split, segment=args.segment)
+                           n, ps, disable_reuse=True, hub_split=args.hub_split, segment=args.segment, lanes_per_row=lpr)
     t_layout = time.time() - t0
     for lay in (reuse, plain):
         lay.upload()
@@ -187,6 +197,55 @@ def main():
     pms_a, pms_b = plain.launch_times(x, max(5, args.steps // 2), normalized, out=out_plain, feat_dim=feat)
     torch.cuda.synchronize()
     max_diff = float((out - out_plain).abs().max())
+
+    # ---- the backward aggregation (same plan on the gradient, reuse_conv_kernel.cu:1021-1041): the gradient
+    # arrives packed [N, F]; when F is not a multiple of 4 it is re-strided first, which is timed too
+    extra = {}
+    if not bf16:
+        from artifact_amd import ROF as rof_api
+
+        grad = torch.randn((n, feat), device=dev)
+        ev0, ev1, ev2 = (torch.cuda.Event(enable_timing=True) for _ in range(3))
+        t_pad, t_agg = [], []
+        for _ in range(10):
+            ev0.record()
+            gp = rof_api._padded(grad)
+            ev1.record()
+            reuse.aggregate(gp, normalized, out=out_plain, feat_dim=feat)
+            ev2.record()
+            torch.cuda.synchronize()
+            t_pad.append(ev0.elapsed_time(ev1))
+            t_agg.append(ev1.elapsed_time(ev2))
+        extra["backward_aggregation"] = {"restride_ms": float(np.median(t_pad)), "aggregate_ms": float(np.median(t_agg))}
+        del grad, gp
+
+    # ---- continuity with the upstream micro-benchmark (ROF_evaluation/cuda/small-main.py:357-478): the whole
+    # ROF.reuse_forward_v2 call, dense update included, 10 warm-ups + 100 runs, events on the current stream
+    dims = {"c1": (32, 32), "c2": (128, 256), "c4": (100, 47)}.get(name)
+    if dims and not args.feat:
+        from artifact_amd import ROF as rof_api
+        from artifact_amd.layout import LayoutFamily
+
+        fam = LayoutFamily(lambda _lpr: reuse)
+        xin = torch.randn((n, dims[0]), device=dev)
+        wgt = torch.randn((dims[0], dims[1]), device=dev)
+        dummy = torch.zeros(1, dtype=torch.int32, device=dev)   # plan tensors are not read when a layout is passed
+        call = lambda: rof_api.reuse_forward_v2(xin, wgt, dummy, deg, dummy, dummy, dummy, ps, min(32, dims[1]), 4,
+                                                layout=fam)[0]
+        for _ in range(10):
+            call()
+        ts = []
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for _ in range(100):
+            e0.record()
+            call()
+            e1.record()
+            torch.cuda.synchronize()
+            ts.append(e0.elapsed_time(e1))
+        extra["whole_reuse_forward_v2"] = {"in_dim": dims[0], "out_dim": dims[1], "mean_ms": float(np.mean(ts)),
+                                           "std_ms": float(np.std(ts)), "median_ms": float(np.median(ts))}
+        fam._by_lpr.clear()   # the layout is owned by this function, not by the family
+        del xin, wgt
 
     if args.calibrate_copy:
         import ctypes
@@ -242,6 +301,8 @@ def main():
                  "saved_gathers_frac": 1.0 - st["gathered_rows"] / max(1, e),
                  "cpu_graph_s": t_gen, "cpu_plan_s": t_plan, "cpu_layout_s": t_layout},
     }
+
+    result.update(extra)
 
     if not args.no_cpu_baseline:
         from oracle import oracle as O  # checker + CPU baseline leg only

@@ -102,9 +102,13 @@ typedef struct rof_layout rof_layout;
 typedef struct {
     int32_t min_consumers;   /* a group is materialised iff it has >= this many consumers; 0 = cost model; -1 = all */
     int32_t disable_reuse;   /* 1: expand every group back into its consumers' rows (the comparator)      */
-    int32_t hub_split;       /* rows with more entries than this are cut into segments; 0 = default        */
-    int32_t segment;         /* entries per hub segment; 0 = default                                        */
-    int32_t reserved[4];
+    int32_t hub_split;       /* rows with more entries than this are cut into segments; 0 = choose from    */
+                             /* lanes_per_row and the plan size                                            */
+    int32_t segment;         /* entries per segment; 0 = hub_split / 4                                     */
+    int32_t lanes_per_row;   /* lanes one gathered row occupies in the kernel that will use this layout:   */
+                             /* smallest power of two >= ceil(feat_dim / 4) (fp32) or / 8 (bf16), 4..64;   */
+                             /* 0 = 16.  Only steers the default hub_split.                                 */
+    int32_t reserved[3];
 } rof_layout_opts;
 
 /* v2 tensors: replaces the plan arguments of reuse_forward_v2 / reuse_backward_v2
@@ -188,6 +192,10 @@ int rof_device_copy(void *dst, const void *src, size_t nbytes, void *stream);
  * has its own L2, so runs of neighbouring destination rows share gathered rows there).  Process-wide;
  * no upstream counterpart. */
 int rof_set_xcd_run(int run_launch1, int run_launch2);
+
+/* Launch tuning: request `bytes` (0..65536) of unused LDS per workgroup, which caps how many workgroups
+ * share a CU (160 KB LDS each) and with it the number of row gathers in flight.  Process-wide. */
+int rof_set_lds_pad(int bytes);
 
 #ifdef __cplusplus
 }
