@@ -109,7 +109,13 @@ def _update(x, weight):
 
 
 def _padded(t):
-    """A gradient arrives packed; re-stride it to a multiple of four floats when it is not."""
+    """Packed rows are gathered in place: the kernels read 16 bytes at any 4-byte boundary."""
+    return t
+
+
+def _restrided(t):
+    """Copy of `t` whose row stride is a multiple of four floats (rows then start on 16-byte boundaries and
+    straddle fewer cache lines).  Not used on the operator path; kept for measurements."""
     f = t.shape[1]
     pad = (-f) % 4
     if pad == 0:

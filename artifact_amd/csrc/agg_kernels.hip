@@ -90,8 +90,10 @@ struct RowLoad;
 #else
 #define ROF_LD16(T, p) (*reinterpret_cast<const T *>(p))
 #endif
-typedef float rof_f4 __attribute__((ext_vector_type(4)));
-typedef unsigned int rof_u4 __attribute__((ext_vector_type(4)));
+// 16-byte vectors that only promise 4-byte alignment: gfx950 executes global_load_dwordx4 at any dword
+// address, so packed rows (e.g. 47 floats = 188 bytes) are gathered with the same instruction as padded ones
+typedef float rof_f4 __attribute__((ext_vector_type(4), aligned(4)));
+typedef unsigned int rof_u4 __attribute__((ext_vector_type(4), aligned(4)));
 
 template <>
 struct RowLoad<float, 4> {
@@ -259,8 +261,13 @@ __global__ __launch_bounds__(256, ROF_MIN_BLOCKS) void rof_rows_kernel(AggArgs a
     for (int c0 = 0; c0 < a.feat; c0 += LPR * VEC) {
         const int cbase = c0 + li * VEC;
         const bool act = cbase < a.feat;
-        const char *xb = reinterpret_cast<const char *>(a.x) + (size_t)cbase * sizeof(XT);
-        const char *pb = reinterpret_cast<const char *>(a.part) + (size_t)cbase * 4;
+        // The lane that would run past the end of the row starts VEC elements before the end instead
+        // (its first `skip` elements repeat its neighbour's and are not stored), so no load ever leaves
+        // the row and rows need no padding.  The host guarantees feat >= VEC.
+        const int cstart = (VEC > 1 && cbase + VEC > a.feat) ? a.feat - VEC : cbase;
+        const int skip = cbase - cstart;
+        const char *xb = reinterpret_cast<const char *>(a.x) + (size_t)cstart * sizeof(XT);
+        const char *pb = reinterpret_cast<const char *>(a.part) + (size_t)cstart * 4;
         float acc[VEC];
 #pragma unroll
         for (int k = 0; k < VEC; ++k) acc[k] = 0.0f;
@@ -301,8 +308,8 @@ __global__ __launch_bounds__(256, ROF_MIN_BLOCKS) void rof_rows_kernel(AggArgs a
             // zero-initialised output upstream: reuse_conv_kernel.cu:303)
             float s = 1.0f;
             if (a.task_scale && end > beg) s = a.task_scale[t];
-            float *o = a.out + (int64_t)a.task_out[t] * a.ldo + cbase;
-            if (VEC >= 4 && a.vec_store && cbase + VEC <= a.feat) {
+            float *o = a.out + (int64_t)a.task_out[t] * a.ldo + cstart;
+            if (VEC >= 4 && a.vec_store && skip == 0) {
 #pragma unroll
                 for (int k = 0; k < VEC; k += 4)
                     *reinterpret_cast<float4 *>(o + k) =
@@ -310,7 +317,7 @@ __global__ __launch_bounds__(256, ROF_MIN_BLOCKS) void rof_rows_kernel(AggArgs a
             } else {
 #pragma unroll
                 for (int k = 0; k < VEC; ++k)
-                    if (cbase + k < a.feat) o[k] = acc[k] * s;
+                    if (k >= skip && cstart + k < a.feat) o[k] = acc[k] * s;
             }
         }
     }
@@ -533,8 +540,9 @@ static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64
 
     const int esz = x_dtype == ROF_F32 ? 4 : 2;
     const int wide = x_dtype == ROF_F32 ? 4 : 8;
-    const bool aligned = (ldx % wide == 0) && (((uintptr_t)x) % 16 == 0);
-    const int vec = aligned ? wide : 1;
+    // 16-byte gathers need rows that start on a 4-byte boundary and hold at least one full vector
+    const bool dword_rows = (((uintptr_t)x) % 4 == 0) && ((ldx * esz) % 4 == 0);
+    const int vec = (dword_rows && feat >= wide) ? wide : 1;
     const int64_t ldp = round_up(feat, 8);
     const int64_t rows_x = L->n, rows_p = L->n_slots;
     const bool off32 = rows_x < (1 << 24) && rows_p < (1 << 24) && ldx * esz < (1 << 24) && ldp * 4 < (1 << 24) &&

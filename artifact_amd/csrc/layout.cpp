@@ -28,6 +28,11 @@ const int32_t kShortRow = 32;        // tasks up to this many entries share a wa
 // ~1/1000 of all entries so that the longest chain stays short against the whole launch on small graphs.
 const int32_t kHubSplitPerGroupMax = 1024;
 const int32_t kHubSplitPerGroupMin = 64;
+// Sharing groups costs one more launch (~8 us on MI355X, the time of ~3*10^5 average row gathers), and the
+// gathers it saves are cheaper than average because the sources of a popular group are themselves popular
+// rows that sit in L2 (measured: 3-9 ps per saved gather against 24-90 ps per average gather).  Plans that
+// save fewer gathers than this are executed with every group folded back into its consumers.
+const int64_t kMinSavedGathers = 1000000;   // row gathers saved minus partial-row reads added
 const int32_t kTileRows = 4096;      // short tasks are length-sorted inside tiles of this many rows
 
 bool ptr_ok(const int32_t *p, int64_t n, int64_t *total) {
@@ -156,10 +161,18 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
         if (min_consumers > 0) return cnt >= min_consumers;
         return (cnt - 1) * len > cnt + 1;
     };
+    // a plan whose sharing would not repay its extra launch is executed with every group folded back
+    int64_t saved = 0;
+    for (int64_t g = 0; g < G; ++g) {
+        int64_t cnt = L->group_dst_ptr[g + 1] - L->group_dst_ptr[g], len = L->group_ptr[g + 1] - L->group_ptr[g];
+        if (worth(cnt, len)) saved += (cnt - 1) * len - cnt;
+    }
+    const bool too_small = min_consumers == 0 && saved < kMinSavedGathers;
     std::vector<int32_t> slot_of(G, -1);
     int64_t slots = 0;
     TaskList tg, ts, tb;
     for (int64_t g = 0; g < G; ++g) {
+        if (too_small) break;
         if (!worth(L->group_dst_ptr[g + 1] - L->group_dst_ptr[g], L->group_ptr[g + 1] - L->group_ptr[g])) continue;
         slot_of[g] = (int32_t)slots++;
         tg.begin_task(slot_of[g]);

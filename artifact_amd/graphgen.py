@@ -11,7 +11,7 @@ from __future__ import annotations
 
 import numpy as np
 
-__all__ = ["rmat_csr", "sbm_csr", "csr_from_pairs", "features", "glorot", "WORKLOADS", "make_workload"]
+__all__ = ["rmat_csr", "sbm_csr", "planted_reuse_csr", "csr_from_pairs", "features", "glorot", "WORKLOADS", "make_workload"]
 
 
 def csr_from_pairs(u, v, num_nodes, self_loops=False):
@@ -98,6 +98,24 @@ def sbm_csr(num_blocks, block_size, deg_in, deg_out, seed, self_loops=False):
     return csr_from_pairs(np.concatenate(us), np.concatenate(vs), n, self_loops)
 
 
+def planted_reuse_csr(num_nodes, set_size=12, members_per_set=64, extra_degree=4, seed=0):
+    """Graph with planted common-neighbour structure: nodes come in clubs of `members_per_set`; every
+    member of a club is linked to the same `set_size` anchor nodes (consecutive ids, so the chunks of a
+    member's sorted neighbour list coincide with those of its club mates), plus `extra_degree` random
+    neighbours.  Symmetric, duplicate-free.  Not one of the upstream-style workloads: it exists to show
+    what the reuse plan buys when a graph does contain shared neighbour subsets."""
+    rng = np.random.Generator(np.random.PCG64(seed))
+    clubs = max(1, num_nodes // (members_per_set + set_size))
+    n_anchor = clubs * set_size
+    members = np.arange(n_anchor, num_nodes, dtype=np.int64)
+    club = (members - n_anchor) % clubs
+    u = np.repeat(members, set_size)
+    v = (np.repeat(club * set_size, set_size) + np.tile(np.arange(set_size), len(members)))
+    ru = rng.integers(n_anchor, num_nodes, size=len(members) * extra_degree // 2)
+    rv = rng.integers(n_anchor, num_nodes, size=len(ru))
+    return csr_from_pairs(np.concatenate([u, ru]), np.concatenate([v, rv]), num_nodes, False)
+
+
 def features(num_nodes, dim, seed, kind="normal"):
     rng = np.random.Generator(np.random.PCG64(seed))
     if kind == "normal":
@@ -121,6 +139,9 @@ WORKLOADS = {
                dims=(64, 64)),
     "c4": dict(kind="rmat", num_nodes=2_400_000, avg_degree=26, self_loops=False, seed=1004, dims=(100, 47)),
     "c5": dict(kind="rmat", num_nodes=1 << 22, avg_degree=32, self_loops=True, seed=1005, dims=(256, 256)),
+    # planted reuse (see planted_reuse_csr): 2^20 nodes, 12 shared anchors + ~4 random neighbours per member
+    "hr": dict(kind="planted", num_nodes=1 << 20, set_size=12, members_per_set=64, extra_degree=4, seed=1006,
+               dims=(64, 64)),
 }
 
 
@@ -131,5 +152,8 @@ def make_workload(name, scale_down=0):
     if w["kind"] == "rmat":
         n = max(64, w["num_nodes"] >> scale_down)
         return rmat_csr(n, w["avg_degree"], w["seed"], self_loops=w["self_loops"])
+    if w["kind"] == "planted":
+        n = max(512, w["num_nodes"] >> scale_down)
+        return planted_reuse_csr(n, w["set_size"], w["members_per_set"], w["extra_degree"], w["seed"])
     nb = max(2, w["num_blocks"] >> scale_down)
     return sbm_csr(nb, w["block_size"], w["deg_in"], w["deg_out"], w["seed"], self_loops=w["self_loops"])

@@ -73,9 +73,10 @@ class ROF_inputInfo:
         return f"ROF_inputInfo(partSize={self.partSize}, warpPerBlock={self.warpPerBlock}, {shapes})"
 
 
-def build_input_info(indptr, indices, part_size=3, device="cuda", warps_per_block=4, plan=None):
+def build_input_info(indptr, indices, part_size=3, device="cuda", warps_per_block=4, plan=None, **layout_opts):
     """CSR (symmetric graph, in-neighbours = out-neighbours) -> ROF_inputInfo, following the glue of
-    ROF_main.py:71-178: plan on the CPU, arrays cast to int32, degrees = diff(indptr) as float32."""
+    ROF_main.py:71-178: plan on the CPU, arrays cast to int32, degrees = diff(indptr) as float32.
+    `layout_opts` (min_consumers, disable_reuse, hub_split, segment) go to the device layout."""
     indptr = np.asarray(indptr)
     indices = np.asarray(indices)
     if plan is None:
@@ -94,7 +95,7 @@ def build_input_info(indptr, indices, part_size=3, device="cuda", warps_per_bloc
     if torch.device(device).type == "cuda":
         info.layouts["ROF_v2"] = LayoutFamily(lambda lpr: Layout.from_v2(
             plan["uniqpart_column_index"], plan["uniqpart_pointers"], plan["part2Node_ptr"], plan["part2Node_col"], n,
-            part_size, lanes_per_row=lpr))
+            part_size, lanes_per_row=lpr, **layout_opts))
     info.plan = plan
     return info
 

@@ -32,8 +32,9 @@ DESCR = {
     "c3": "c3: SBM 2^20 nodes (256 blocks), deg 24+2, GIN sum aggregation, F=64, fp32",
     "c4": "c4: R-MAT 2.4M nodes, ~60M directed edges, GCN sym-norm, aggregated width 47, fp32",
     "c5": "c5: R-MAT 2^22 nodes, avg deg 32, self loops, GCN sym-norm, F=256, bf16 in / fp32 accumulate",
+    "hr": "hr: planted-reuse graph 2^20 nodes (12 shared anchors + ~4 random neighbours per node), GCN, F=64, fp32",
 }
-FEAT = {"c1": 32, "c2": 256, "c3": 64, "c4": 47, "c5": 256}
+FEAT = {"c1": 32, "c2": 256, "c3": 64, "c4": 47, "c5": 256, "hr": 64}
 
 
 def log(*a):
@@ -142,7 +143,7 @@ def main():
     # features: N(0,1) fp32 (uniform(-1,1) -> bf16 for c5), rows padded to a multiple of 4 (8) elements
     mult = 8 if bf16 else 4
     ld = (feat + mult - 1) // mult * mult
-    x32 = features(n, feat, seed=2000 + int(name[1]), kind="uniform" if bf16 else "normal")
+    x32 = features(n, feat, seed=2000 + (int(name[1]) if name[1].isdigit() else 6), kind="uniform" if bf16 else "normal")
     xbuf = torch.zeros((n, ld), dtype=torch.bfloat16 if bf16 else torch.float32, device=dev)
     xbuf[:, :feat] = torch.from_numpy(x32).to(dev)
     x = xbuf[:, :feat]
@@ -160,7 +161,14 @@ def main():
     plain = Layout.from_v2(d["uniqpart_column_index"], d["uniqpart_pointers"], d["part2Node_ptr"], d["part2Node_col"],
                            n, ps, disable_reuse=True, hub_split=args.hub_split, segment=args.segment, lanes_per_row=lpr)
     t_layout = time.time() - t0
-    for lay in (reuse, plain):
+    # when the cost model folds every group back (the plan saves too little), also time the plan with its
+    # profitable groups forced to be shared, so the cost of the reuse machinery stays visible
+    forced = None
+    if reuse.stats()["materialised_groups"] == 0 and len(d["index_picked"]) and not args.min_consumers:
+        forced = Layout.from_v2(d["uniqpart_column_index"], d["uniqpart_pointers"], d["part2Node_ptr"],
+                                d["part2Node_col"], n, ps, hub_split=args.hub_split, segment=args.segment,
+                                lanes_per_row=lpr, min_consumers=3)
+    for lay in (reuse, plain) + ((forced,) if forced else ()):
         lay.upload()
         if normalized:
             lay.set_degrees(deg)
@@ -193,13 +201,28 @@ def main():
         ev_r.append(reuse.aggregate_timed(x, per, normalized, out=out, feat_dim=feat)[0])
         ev_p.append(plain.aggregate_timed(x, per, normalized, out=out_plain, feat_dim=feat)[0])
     ev_ms, plain_ms = float(np.median(ev_r)), float(np.median(ev_p))
+    forced_info = None
+    if forced is not None:
+        out_f = torch.empty_like(out)
+        forced.aggregate(x, normalized, out=out_f, feat_dim=feat)
+        ev_f, ev_p2 = [], []
+        for _ in range(4):
+            ev_f.append(forced.aggregate_timed(x, per, normalized, out=out_f, feat_dim=feat)[0])
+            ev_p2.append(plain.aggregate_timed(x, per, normalized, out=out_plain, feat_dim=feat)[0])
+        fs = forced.stats()
+        forced_info = {"min_consumers": 3, "event_ms": float(np.median(ev_f)),
+                       "speedup_vs_reuse_disabled": float(np.median(ev_p2) / np.median(ev_f)),
+                       "materialised_groups": fs["materialised_groups"],
+                       "saved_gathers_frac": 1.0 - fs["gathered_rows"] / max(1, e),
+                       "max_abs_diff_vs_reuse_disabled": float((out_f - out_plain).abs().max())}
+        del out_f
     ms_a, ms_b = reuse.launch_times(x, max(5, args.steps // 2), normalized, out=out, feat_dim=feat)
     pms_a, pms_b = plain.launch_times(x, max(5, args.steps // 2), normalized, out=out_plain, feat_dim=feat)
     torch.cuda.synchronize()
     max_diff = float((out - out_plain).abs().max())
 
     # ---- the backward aggregation (same plan on the gradient, reuse_conv_kernel.cu:1021-1041): the gradient
-    # arrives packed [N, F]; when F is not a multiple of 4 it is re-strided first, which is timed too
+    # arrives packed [N, F]
     extra = {}
     if not bf16:
         from artifact_amd import ROF as rof_api
@@ -209,14 +232,24 @@ def main():
         t_pad, t_agg = [], []
         for _ in range(10):
             ev0.record()
-            gp = rof_api._padded(grad)
+            gp = rof_api._restrided(grad)
             ev1.record()
             reuse.aggregate(gp, normalized, out=out_plain, feat_dim=feat)
             ev2.record()
             torch.cuda.synchronize()
             t_pad.append(ev0.elapsed_time(ev1))
             t_agg.append(ev1.elapsed_time(ev2))
-        extra["backward_aggregation"] = {"restride_ms": float(np.median(t_pad)), "aggregate_ms": float(np.median(t_agg))}
+        t_packed = []
+        for _ in range(10):
+            ev0.record()
+            reuse.aggregate(grad, normalized, out=out_plain, feat_dim=feat)
+            ev1.record()
+            torch.cuda.synchronize()
+            t_packed.append(ev0.elapsed_time(ev1))
+        # packed_rows_ms is what the operator path does (rows gathered in place at 4-byte alignment); the other two
+        # numbers are the alternative of re-striding the gradient to 16-byte rows first
+        extra["backward_aggregation"] = {"packed_rows_ms": float(np.median(t_packed)),
+                                         "restride_ms": float(np.median(t_pad)), "aggregate_ms": float(np.median(t_agg))}
         del grad, gp
 
     # ---- continuity with the upstream micro-benchmark (ROF_evaluation/cuda/small-main.py:357-478): the whole
@@ -295,7 +328,9 @@ def main():
             "achieved_GBs": b_alg_plain / (plain_ms * 1e-3) / 1e9, "speedup_of_reuse": plain_ms / ev_ms,
             "max_abs_diff_vs_reuse": max_diff,
         },
+        "reuse_forced": forced_info,
         "plan": {"groups": st["groups"], "materialised_groups": st["materialised_groups"],
+                 "folded_by_cost_model": bool(st["materialised_groups"] == 0 and st["groups"] > 0),
                  "gathered_rows": st["gathered_rows"], "partial_reads": st["partial_reads"],
                  "partial_rows": st["partial_rows"], "hub_segments": st["hub_segments"],
                  "saved_gathers_frac": 1.0 - st["gathered_rows"] / max(1, e),

@@ -43,7 +43,8 @@ def test_gcn_widths_match_oracle(oracle, feat):
     n = len(indptr) - 1
     x = features(n, feat, seed=7)
     deg = np.diff(indptr).astype(np.float32)
-    lay = _layout(plan, n, 3)
+    lay = _layout(plan, n, 3, min_consumers=2)               # every picked part shared: exercises partial rows
+    assert lay.stats()["materialised_groups"] > 0
     xt = torch.from_numpy(x).cuda()
     lay.set_degrees(torch.from_numpy(deg).cuda())
     got = lay.aggregate(xt, normalized=True).cpu().numpy()
@@ -56,7 +57,7 @@ def test_gcn_widths_match_oracle(oracle, feat):
 
 
 @pytest.mark.parametrize("name,sd,ps", [("c1", 0, 3), ("c1", 0, 2), ("c1", 1, 5), ("c2", 3, 3), ("c3", 5, 2),
-                                        ("c4", 6, 3)])
+                                        ("c4", 6, 3), ("hr", 5, 3), ("hr", 6, 2)])
 def test_reuse_equals_no_reuse_and_closed_form(oracle, name, sd, ps):
     indptr, indices, plan = _case(name, sd, ps)
     n = len(indptr) - 1
@@ -68,7 +69,8 @@ def test_reuse_equals_no_reuse_and_closed_form(oracle, name, sd, ps):
     want = oracle.closed_form(indptr, indices, x, deg)
     mag = oracle.closed_form(indptr, indices, np.abs(x), deg)
     outs = []
-    for opts in (dict(), dict(disable_reuse=True), dict(min_consumers=2), dict(hub_split=64, segment=16)):
+    for opts in (dict(min_consumers=3), dict(disable_reuse=True), dict(min_consumers=2),
+                 dict(min_consumers=2, hub_split=64, segment=16), dict()):
         lay = _layout(plan, n, ps, **opts)
         lay.set_degrees(degt)
         out = torch.full((n, feat), float("nan"), device="cuda")   # every element must be overwritten
@@ -85,20 +87,40 @@ def test_sum_aggregation_unnormalised(oracle):
     indptr, indices, plan = _case("c3", 5, 2)
     n = len(indptr) - 1
     x = features(n, 64, seed=5)
-    lay = _layout(plan, n, 2)
+    lay = _layout(plan, n, 2, min_consumers=2)
     got = lay.aggregate(torch.from_numpy(x).cuda(), normalized=False).cpu().numpy()
     want = oracle.closed_form(indptr, indices, x, normalized=False)
     _close(got, want, oracle.closed_form(indptr, indices, np.abs(x), normalized=False))
 
 
-def test_unaligned_rows_take_scalar_path(oracle):
+@pytest.mark.parametrize("feat,ld,shift", [(47, 47, 0), (5, 5, 0), (7, 9, 1), (101, 101, 3), (255, 255, 0), (2, 2, 1)])
+def test_packed_and_misaligned_rows(oracle, feat, ld, shift):
+    """Rows that start on arbitrary 4-byte boundaries (packed widths, odd strides, an offset base pointer):
+    the last lane of a row is shifted back so that no load leaves the row, even in the last row of the buffer."""
     indptr, indices, plan = _case("c1", 3, 3)
     n = len(indptr) - 1
-    x = features(n, 47, seed=3)                              # packed rows of 188 bytes: not 16-byte aligned
+    x = features(n, feat, seed=3)
     deg = np.diff(indptr).astype(np.float32)
-    lay = _layout(plan, n, 3)
+    flat = torch.full((n * ld + shift,), float("nan"), device="cuda")          # nothing readable beyond the last row
+    xt = flat[shift:shift + n * ld].view(n, ld)[:, :feat]
+    xt.copy_(torch.from_numpy(x))
+    lay = _layout(plan, n, 3, min_consumers=2)
     lay.set_degrees(torch.from_numpy(deg).cuda())
-    got = lay.aggregate(torch.from_numpy(x).cuda(), normalized=True).cpu().numpy()
+    got = lay.aggregate(xt, normalized=True, feat_dim=feat).cpu().numpy()
+    assert np.isfinite(got).all()                                               # no NaN padding was ever summed
+    _close(got, oracle.closed_form(indptr, indices, x, deg), oracle.closed_form(indptr, indices, np.abs(x), deg))
+
+
+@pytest.mark.parametrize("feat", [41, 6, 24])
+def test_bf16_odd_widths(oracle, feat):
+    indptr, indices, plan = _case("c1", 3, 3)
+    n = len(indptr) - 1
+    xb = torch.from_numpy(features(n, feat, seed=4, kind="uniform")).to(torch.bfloat16)
+    x = xb.to(torch.float32).numpy()
+    deg = np.diff(indptr).astype(np.float32)
+    lay = _layout(plan, n, 3, min_consumers=2)
+    lay.set_degrees(torch.from_numpy(deg).cuda())
+    got = lay.aggregate(xb.cuda(), normalized=True).cpu().numpy()
     _close(got, oracle.closed_form(indptr, indices, x, deg), oracle.closed_form(indptr, indices, np.abs(x), deg))
 
 
@@ -109,7 +131,7 @@ def test_bf16_inputs_fp32_accumulate(oracle, feat):
     xb = torch.from_numpy(features(n, feat, seed=9, kind="uniform")).to(torch.bfloat16)
     x = xb.to(torch.float32).numpy()                         # the oracle sees the bf16-rounded values
     deg = np.diff(indptr).astype(np.float32)
-    lay = _layout(plan, n, 3)
+    lay = _layout(plan, n, 3, min_consumers=2)
     lay.set_degrees(torch.from_numpy(deg).cuda())
     got = lay.aggregate(xb.cuda(), normalized=True).cpu().numpy()
     want = oracle.closed_form(indptr, indices, x, deg)
@@ -121,7 +143,7 @@ def test_bf16_inputs_fp32_accumulate(oracle, feat):
 def test_deterministic_run_to_run():
     indptr, indices, plan = _case("c1", 1, 3)
     n = len(indptr) - 1
-    lay = _layout(plan, n, 3)
+    lay = _layout(plan, n, 3, min_consumers=2)
     lay.set_degrees(torch.from_numpy(np.diff(indptr).astype(np.float32)).cuda())
     xt = torch.from_numpy(features(n, 64, seed=1)).cuda()
     a = lay.aggregate(xt).clone()

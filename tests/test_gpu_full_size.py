@@ -19,7 +19,7 @@ def big():
     plan = R.build_plan(ip, ix, 3)
     n = len(ip) - 1
     args = (plan["uniqpart_column_index"], plan["uniqpart_pointers"], plan["part2Node_ptr"], plan["part2Node_col"], n, 3)
-    return ip, ix, n, Layout.from_v2(*args), Layout.from_v2(*args, disable_reuse=True)
+    return ip, ix, n, Layout.from_v2(*args, min_consumers=3), Layout.from_v2(*args, disable_reuse=True)
 
 
 def test_full_size_properties(big):

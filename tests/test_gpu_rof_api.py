@@ -19,7 +19,7 @@ DEV = "cuda"
 def _setup(wl="c1", sd=2, ps=3, fin=20, fout=47):
     ip, ix = make_workload(wl, sd)
     n = len(ip) - 1
-    info = build_input_info(ip, ix, part_size=ps, device=DEV)
+    info = build_input_info(ip, ix, part_size=ps, device=DEV, min_consumers=2)
     x = features(n, fin, seed=21)
     w = glorot(fin, fout, seed=22)
     return ip, ix, n, info, x, w
@@ -140,7 +140,7 @@ def test_two_layer_gcn_forward_matches_dense_reference(oracle):
     """Workload 2 in miniature: 128 -> 256 -> 40 with ReLU between the layers."""
     ip, ix = make_workload("c2", 6)
     n = len(ip) - 1
-    info = build_input_info(ip, ix, part_size=3, device=DEV)
+    info = build_input_info(ip, ix, part_size=3, device=DEV, min_consumers=2)
     x = features(n, 128, seed=2002)
     w1, w2 = glorot(128, 256, 3002), glorot(256, 40, 3003)
     c1 = ROF_GCNConv(128, 256, bias=False, add_self_loops=False, kernel_type="ROF_v2").to(DEV)
@@ -158,7 +158,7 @@ def test_two_layer_gcn_forward_matches_dense_reference(oracle):
 def test_gin_layer_sum_aggregation_and_gradient(oracle):
     ip, ix = make_workload("c3", 6)
     n = len(ip) - 1
-    info = build_input_info(ip, ix, part_size=2, device=DEV)
+    info = build_input_info(ip, ix, part_size=2, device=DEV, min_consumers=2)
     gin = ROF_GINConv(64, 64, eps=0.0).to(DEV)
     x = features(n, 64, seed=2003)
     xt = torch.from_numpy(x).to(DEV).requires_grad_(True)
