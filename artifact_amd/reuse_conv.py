@@ -62,6 +62,30 @@ class ROF_inputInfo:
     def reuse_size(self):
         return int(self.part_pointers_cache.shape[0]) - 1
 
+    # ---- on-disk form of the (expensive) plan; upstream caches the whole object with torch.save
+    # (ROF_evaluation/cuda/middle-main.py:440-452), which also works; this form is plain numpy
+    def save(self, path):
+        """Write every plan tensor plus the two scalars to an .npz file."""
+        arrays = {name: getattr(self, name).detach().cpu().numpy() for name in _TENSOR_FIELDS}
+        np.savez(path, partSize=np.int64(self.partSize), warpPerBlock=np.int64(self.warpPerBlock), **arrays)
+
+    @classmethod
+    def load(cls, path, device="cuda", **layout_opts):
+        """Inverse of save(); rebuilds the device layout from the stored v2 arrays without a plan search."""
+        z = np.load(path if str(path).endswith(".npz") else str(path) + ".npz")
+        t = {name: torch.from_numpy(z[name]).to(device) for name in _TENSOR_FIELDS}
+        info = cls(t["row_pointers"], t["column_index"], t["degrees"], t["part_pointers"], t["part2Node"],
+                   int(z["partSize"]), int(z["warpPerBlock"]), t["part_cache_flagindex"], t["part_pointers_cache"],
+                   t["column_index_cache"], t["uniqpart_column_index"], t["uniqpart_pointers"], t["part2Node_ptr"],
+                   t["part2Node_col"])
+        if torch.device(device).type == "cuda":
+            n, ps = len(z["row_pointers"]) - 1, int(z["partSize"])
+            v2 = tuple(np.array(z[k]) for k in ("uniqpart_column_index", "uniqpart_pointers", "part2Node_ptr",
+                                                 "part2Node_col"))
+            info.layouts["ROF_v2"] = LayoutFamily(lambda lpr: Layout.from_v2(*v2, n, ps, lanes_per_row=lpr,
+                                                                             **layout_opts))
+        return info
+
     def __getstate__(self):
         d = dict(self.__dict__)
         d["layouts"] = {}   # device handles are rebuilt on demand
