@@ -18,7 +18,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "librof.so")
 
 HOST_SOURCES = ["plan_builder.cpp", "layout.cpp"]
-HIP_SOURCES = ["agg_kernels.hip"]
+HIP_SOURCES = ["agg_kernels.hip", "agg_rows_f32.hip", "agg_rows_bf16.hip"]
 
 # packed fp32 instructions stay off: the compiler must not form v_pk_{add,mul,fma}_f32
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang",
@@ -42,10 +42,17 @@ def build_library(verbose=True):
         o = os.path.join(objdir, s + ".o")
         _run([gxx] + HOST_FLAGS + inc + ["-c", os.path.join(CSRC, s), "-o", o])
         objs.append(o)
+    # the kernel translation units are independent: compile them side by side
+    procs = []
     for s in HIP_SOURCES:
         o = os.path.join(objdir, s + ".o")
-        _run([hipcc] + HIP_FLAGS + inc + ["-c", os.path.join(CSRC, s), "-o", o])
+        cmd = [hipcc] + HIP_FLAGS + inc + ["-c", os.path.join(CSRC, s), "-o", o]
+        print("+", " ".join(cmd), flush=True)
+        procs.append((cmd, subprocess.Popen(cmd)))
         objs.append(o)
+    for cmd, pr in procs:
+        if pr.wait() != 0:
+            raise subprocess.CalledProcessError(pr.returncode, cmd)
     _run([hipcc, "-shared", "-fPIC", "-o", LIB] + objs + ["-fopenmp", "-lgomp"])
     return LIB
 

@@ -1,0 +1,364 @@
+// Row-gather kernel of the reuse-aware aggregation and its launcher template, shared by the two
+// translation units that instantiate it (fp32 and bf16 features are compiled separately so that the
+// build can run them in parallel).  See agg_kernels.hip for the description of the scheme.
+#ifndef ROF_AGG_ROWS_H_
+#define ROF_AGG_ROWS_H_
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "rof.h"
+#include "rof_internal.h"
+
+#define HIP_TRY(expr)                                                                  \
+    do {                                                                               \
+        hipError_t e_ = (expr);                                                        \
+        if (e_ != hipSuccess) {                                                        \
+            rof_set_device_error(#expr, hipGetErrorString(e_));                        \
+            return ROF_ERR_DEVICE;                                                     \
+        }                                                                              \
+    } while (0)
+
+namespace rofk {
+
+// process-wide launch tuning (rof_set_xcd_run, rof_set_lds_pad); defined in agg_kernels.hip
+extern int g_xcd_run_a, g_xcd_run_b;
+extern int g_lds_pad;   // bytes of unused LDS requested per workgroup: caps the workgroups resident per CU
+
+struct AggArgs {
+    const void *x;         // feature rows
+    int64_t ldx;
+    const float *part;     // partial-sum rows (ids >= nsplit)
+    int64_t ldp;
+    int32_t nsplit;
+    const int32_t *task_ptr, *task_nref, *task_out;
+    const float *task_scale;   // null: no scaling
+    const int32_t *col;
+    const float *w;            // null: unweighted
+    float *out;
+    int64_t ldo;
+    int32_t feat;
+    int32_t n_wave, n_tasks;
+    int32_t n_blocks;          // logical workgroups
+    int32_t xcd_run;           // consecutive logical workgroups kept on one XCD
+    int32_t vec_store;         // output rows allow aligned 16-byte stores
+};
+
+// Row gathers a lane group keeps in flight.  Measured on MI355X with all eight wave slots per SIMD
+// occupied: 2 beats 4 by ~10 % on the miss-dominated workloads (more outstanding gathers per CU slow the
+// L1/L2 miss path down) and loses ~2 % where gathers hit in L2; 8 loses everywhere.
+#ifndef ROF_UNROLL
+#define ROF_UNROLL 2
+#endif
+#ifndef ROF_MIN_BLOCKS
+#define ROF_MIN_BLOCKS 1
+#endif
+constexpr int kWavesPerBlock = 4;
+constexpr int kXcds = 8;
+
+template <typename XT, int VEC>
+struct RowLoad;
+
+#ifdef ROF_NT_LOADS
+#define ROF_LD16(T, p) __builtin_nontemporal_load(reinterpret_cast<const T *>(p))
+#else
+#define ROF_LD16(T, p) (*reinterpret_cast<const T *>(p))
+#endif
+// 16-byte vectors that only promise 4-byte alignment: gfx950 executes global_load_dwordx4 at any dword
+// address, so packed rows (e.g. 47 floats = 188 bytes) are gathered with the same instruction as padded ones
+typedef float rof_f4 __attribute__((ext_vector_type(4), aligned(4)));
+typedef unsigned int rof_u4 __attribute__((ext_vector_type(4), aligned(4)));
+
+template <>
+struct RowLoad<float, 4> {
+    static __device__ __forceinline__ void load(const float *p, float (&v)[4]) {
+        rof_f4 t = ROF_LD16(rof_f4, p);
+        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+    }
+};
+template <>
+struct RowLoad<float, 8> {
+    static __device__ __forceinline__ void load(const float *p, float (&v)[8]) {
+        rof_f4 t = ROF_LD16(rof_f4, p);
+        rof_f4 u = ROF_LD16(rof_f4, p + 4);
+        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+        v[4] = u.x; v[5] = u.y; v[6] = u.z; v[7] = u.w;
+    }
+};
+template <>
+struct RowLoad<float, 1> {
+    static __device__ __forceinline__ void load(const float *p, float (&v)[1]) { v[0] = *p; }
+};
+// bf16 is the upper half of an fp32
+template <>
+struct RowLoad<uint16_t, 8> {
+    static __device__ __forceinline__ void load(const uint16_t *p, float (&v)[8]) {
+        rof_u4 t = ROF_LD16(rof_u4, p);
+        v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u);
+        v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
+        v[4] = __uint_as_float(t.z << 16); v[5] = __uint_as_float(t.z & 0xffff0000u);
+        v[6] = __uint_as_float(t.w << 16); v[7] = __uint_as_float(t.w & 0xffff0000u);
+    }
+};
+template <>
+struct RowLoad<uint16_t, 1> {
+    static __device__ __forceinline__ void load(const uint16_t *p, float (&v)[1]) {
+        v[0] = __uint_as_float(((uint32_t)*p) << 16);
+    }
+};
+
+// Address of this lane's slice of gathered row `c`.  xb / pb already include the lane's column
+// offset; ld in bytes.  With DUAL ids >= nsplit name partial-sum rows (pb), chosen by selects, not
+// branches.  OFF32: all byte offsets fit 32 bits and row ids fit 24 (checked on the host), so one
+// 24-bit multiply and a 32-bit add replace the 64-bit multiply.
+template <bool DUAL, bool OFF32>
+__device__ __forceinline__ const char *row_ptr(int32_t c, const char *xb, uint32_t xld, const char *pb, uint32_t pld,
+                                               int32_t nsplit, int32_t bias) {
+    uint32_t r = (uint32_t)(c - bias), l = xld;
+    const char *b = xb;
+    if (DUAL) {
+        const bool p = c >= nsplit;
+        r = p ? (uint32_t)(c - nsplit) : r;
+        l = p ? pld : xld;
+        b = p ? pb : xb;
+    }
+    if (OFF32) return b + __umul24(r, l);
+    return b + (uint64_t)r * l;
+}
+
+// Sum the entries [beg, end) of one task into acc.  WAVE: all lane groups of the wavefront share
+// the task (beg/end wave-uniform) and take every G-th entry; otherwise each lane group owns its
+// task.  ST is the element type of the source rows.  Blocks of U entries that are complete for every
+// lane group run without any per-entry predicate; ragged ends are predicated entry by entry.
+template <typename ST, int VEC, int LPR, bool WAVE, bool DUAL, bool OFF32>
+__device__ __forceinline__ void gather_sum(const char *xb, uint32_t xld, const char *pb, uint32_t pld, int32_t nsplit,
+                                           int32_t bias, const int32_t *__restrict__ col,
+                                           const float *__restrict__ w, int32_t beg, int32_t end, int lane, int sub,
+                                           int li, bool act, float (&acc)[VEC]) {
+    constexpr int G = 64 / LPR;             // lane groups per wavefront; lanes >= G*LPR stay idle
+    constexpr int U = LPR >= ROF_UNROLL ? ROF_UNROLL : LPR;   // row gathers in flight per lane group
+    constexpr int CH = WAVE ? G * LPR : LPR;   // entries fetched per step by the wave / by the lane group
+    static_assert(LPR % U == 0, "the unroll factor must divide the lanes per row");
+    const bool idle = (G * LPR < 64) && lane >= G * LPR;
+    for (int32_t base = beg; __any(!idle && base < end); base += CH) {
+        const int32_t mine = base + (WAVE ? lane : li);
+        int32_t mycol = bias;               // past the end: row 0 of the source, weight 0
+        float myw = 0.0f;
+        if (!idle && mine < end) {
+            mycol = col[mine];
+            myw = w ? w[mine] : 1.0f;
+        }
+#pragma unroll
+        for (int j0 = 0; j0 < LPR; j0 += U) {
+            const int first = WAVE ? j0 * G + sub : j0;
+            if (!__any(!idle && base + first < end)) break;
+            int32_t c[U];
+            float wt[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int slot = WAVE ? (j0 + u) * G + sub : (j0 + u);          // entry of the chunk
+                const int from = WAVE ? slot : sub * LPR + slot;                // lane that fetched it
+                c[u] = __shfl(mycol, from);
+                wt[u] = __shfl(myw, from);
+            }
+            const int last = WAVE ? (j0 + U - 1) * G + sub : (j0 + U - 1);
+            const bool full = __all(idle || base + last < end);
+            if (act) {
+                float v[U][VEC];
+                if (full) {
+#pragma unroll
+                    for (int u = 0; u < U; ++u)
+                        RowLoad<ST, VEC>::load(
+                            reinterpret_cast<const ST *>(row_ptr<DUAL, OFF32>(c[u], xb, xld, pb, pld, nsplit, bias)),
+                            v[u]);
+#pragma unroll
+                    for (int u = 0; u < U; ++u)
+#pragma unroll
+                        for (int k = 0; k < VEC; ++k) acc[k] = fmaf(wt[u], v[u][k], acc[k]);
+                } else {
+                    // ragged end of a task: gather only the entries that exist (a dummy gather of one
+                    // fixed row from every lane group would pile onto a single L2 channel)
+                    bool ok[U];
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        const int slot = WAVE ? (j0 + u) * G + sub : (j0 + u);
+                        ok[u] = base + slot < end;
+                        if (ok[u])
+                            RowLoad<ST, VEC>::load(reinterpret_cast<const ST *>(
+                                                       row_ptr<DUAL, OFF32>(c[u], xb, xld, pb, pld, nsplit, bias)),
+                                                   v[u]);
+                    }
+#pragma unroll
+                    for (int u = 0; u < U; ++u)
+                        if (ok[u]) {
+#pragma unroll
+                            for (int k = 0; k < VEC; ++k) acc[k] = fmaf(wt[u], v[u][k], acc[k]);
+                        }
+                }
+            }
+        }
+    }
+}
+
+// PHASE 0: the partial-sum launches (no scaling); PHASE 1: the destination-row launch.  Same code; the
+// parameter only gives them distinct kernel names in profiles.
+template <typename XT, int VEC, int LPR, int PHASE, bool OFF32>
+__global__ __launch_bounds__(256, ROF_MIN_BLOCKS) void rof_rows_kernel(AggArgs a) {
+    constexpr int G = 64 / LPR;
+    // XCD-aware renumbering: the hardware deals workgroup ids round-robin to the 8 XCDs; give each
+    // XCD runs of `xcd_run` consecutive logical workgroups instead of every 8th one.
+    const int hw = blockIdx.x;
+    const int xcd = hw % kXcds, nth = hw / kXcds;
+    const int run = a.xcd_run;
+    const int logical = ((nth / run) * kXcds + xcd) * run + (nth % run);
+    if (logical >= a.n_blocks) return;
+
+    const int lane = threadIdx.x & 63;
+    const int sub = lane / LPR, li = lane % LPR;
+    const int gw = logical * kWavesPerBlock + (threadIdx.x >> 6);
+
+    int32_t t, beg = 0, end = 0, mid = 0;
+    bool valid;
+    const bool wave_mode = gw < a.n_wave;
+    const bool idle = (G * LPR < 64) && lane >= G * LPR;   // lanes left over when LPR does not divide 64
+    if (wave_mode) {
+        t = gw;
+        valid = true;
+    } else {
+        t = a.n_wave + (gw - a.n_wave) * G + sub;
+        valid = !idle && t < a.n_tasks;
+    }
+    if (valid) {
+        beg = a.task_ptr[t];
+        end = a.task_ptr[t + 1];
+        mid = beg + a.task_nref[t];
+    }
+    const uint32_t xld = (uint32_t)(a.ldx * (int64_t)sizeof(XT)), pld = (uint32_t)(a.ldp * 4);
+
+    for (int c0 = 0; c0 < a.feat; c0 += LPR * VEC) {
+        const int cbase = c0 + li * VEC;
+        const bool act = !idle && cbase < a.feat;
+        // The lane that would run past the end of the row starts VEC elements before the end instead
+        // (its first `skip` elements repeat its neighbour's and are not stored), so no load ever leaves
+        // the row and rows need no padding.  The host guarantees feat >= VEC.
+        const int cstart = (VEC > 1 && cbase + VEC > a.feat) ? a.feat - VEC : cbase;
+        const int skip = cbase - cstart;
+        const char *xb = reinterpret_cast<const char *>(a.x) + (size_t)cstart * sizeof(XT);
+        const char *pb = reinterpret_cast<const char *>(a.part) + (size_t)cstart * 4;
+        float acc[VEC];
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) acc[k] = 0.0f;
+
+        constexpr bool kF32 = sizeof(XT) == 4;   // fp32 features: partial rows have the same element type
+        if (wave_mode) {
+            if (kF32) {
+                gather_sum<XT, VEC, LPR, true, true, OFF32>(xb, xld, pb, pld, a.nsplit, 0, a.col, a.w, beg, end, lane,
+                                                            sub, li, act, acc);
+            } else {
+                if (mid > beg)
+                    gather_sum<float, VEC, LPR, true, false, OFF32>(pb, pld, nullptr, 0, 0, a.nsplit, a.col, a.w, beg,
+                                                                    mid, lane, sub, li, act, acc);
+                gather_sum<XT, VEC, LPR, true, false, OFF32>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, mid, end, lane, sub,
+                                                             li, act, acc);
+            }
+            if ((G & (G - 1)) == 0) {   // power-of-two group count: butterfly
+#pragma unroll
+                for (int off = LPR; off < 64; off <<= 1) {
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) acc[k] += __shfl_xor(acc[k], off);
+                }
+            } else {                    // otherwise group 0 collects the others one by one
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) {
+                    float tot = acc[k];
+#pragma unroll
+                    for (int g = 1; g < G; ++g) tot += __shfl(acc[k], (li + g * LPR) & 63);
+                    acc[k] = tot;
+                }
+            }
+        } else {
+            if (kF32) {
+                gather_sum<XT, VEC, LPR, false, true, OFF32>(xb, xld, pb, pld, a.nsplit, 0, a.col, a.w, beg, end, lane,
+                                                             sub, li, act, acc);
+            } else {
+                if (__any(mid > beg))
+                    gather_sum<float, VEC, LPR, false, false, OFF32>(pb, pld, nullptr, 0, 0, a.nsplit, a.col, a.w, beg,
+                                                                     mid, lane, sub, li, act, acc);
+                gather_sum<XT, VEC, LPR, false, false, OFF32>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, mid, end, lane, sub,
+                                                              li, act, acc);
+            }
+        }
+
+        const bool writer = valid && act && (!wave_mode || sub == 0);
+        if (writer) {
+            // an empty task writes zeros whatever its scale is (a node without in-edges keeps the
+            // zero-initialised output upstream: reuse_conv_kernel.cu:303)
+            float s = 1.0f;
+            if (a.task_scale && end > beg) s = a.task_scale[t];
+            float *o = a.out + (int64_t)a.task_out[t] * a.ldo + cstart;
+            if (VEC >= 4 && a.vec_store && skip == 0) {
+#pragma unroll
+                for (int k = 0; k < VEC; k += 4)
+                    *reinterpret_cast<float4 *>(o + k) =
+                        make_float4(acc[k] * s, acc[k + 1] * s, acc[k + 2] * s, acc[k + 3] * s);
+            } else {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k)
+                    if (k >= skip && cstart + k < a.feat) o[k] = acc[k] * s;
+            }
+        }
+    }
+}
+
+// Lanes one gathered row occupies: the smallest supported count that covers ceil(feat / vec).  Counts
+// that do not divide 64 (10, 12, 20) leave 4 lanes idle but fit 6, 5 or 3 rows into one load instruction
+// where the next power of two would fit 4, 4 or 2.
+inline int rof_lanes_per_row(int feat, int vec) {
+    static const int kChoices[] = {4, 8, 10, 12, 16, 20, 32, 64};
+    const int need = (feat + vec - 1) / vec;
+    for (int c : kChoices)
+        if (c >= need && (vec > 1 || (c & (c - 1)) == 0)) return c;   // the scalar fallback is built for powers of two
+    return 64;
+}
+
+template <typename XT, int VEC, int PHASE, bool OFF32>
+int launch_lpr(const AggArgs &a0, int lpr, hipStream_t st) {
+    AggArgs a = a0;
+    const int g = 64 / lpr;
+    const int64_t shorts = (int64_t)a.n_tasks - a.n_wave;
+    const int64_t waves = a.n_wave + (shorts + g - 1) / g;
+    if (waves == 0) return ROF_OK;
+    a.n_blocks = (int32_t)((waves + kWavesPerBlock - 1) / kWavesPerBlock);
+    const int64_t span = (int64_t)kXcds * a.xcd_run;
+    const int64_t grid = (a.n_blocks + span - 1) / span * span;
+    dim3 gr((unsigned)grid), bl(64 * kWavesPerBlock);
+    switch (lpr) {
+        case 4: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 4, PHASE, OFF32>), gr, bl, g_lds_pad, st, a); break;
+        case 8: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 8, PHASE, OFF32>), gr, bl, g_lds_pad, st, a); break;
+        case 10:
+            if constexpr (VEC > 1) hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 10, PHASE, OFF32>), gr, bl, g_lds_pad, st, a);
+            break;
+        case 12:
+            if constexpr (VEC > 1) hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 12, PHASE, OFF32>), gr, bl, g_lds_pad, st, a);
+            break;
+        case 20:
+            if constexpr (VEC > 1) hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 20, PHASE, OFF32>), gr, bl, g_lds_pad, st, a);
+            break;
+        case 16: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 16, PHASE, OFF32>), gr, bl, g_lds_pad, st, a); break;
+        case 32: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 32, PHASE, OFF32>), gr, bl, g_lds_pad, st, a); break;
+        default: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 64, PHASE, OFF32>), gr, bl, g_lds_pad, st, a); break;
+    }
+    HIP_TRY(hipGetLastError());
+    return ROF_OK;
+}
+
+// Instantiated in agg_rows_f32.hip / agg_rows_bf16.hip.  phase 0: partial-sum launches, 1: destination rows.
+// off32: every byte offset into the feature matrix and into the partial-sum workspace fits 32 bits and
+// every row id fits 24 bits, so the kernels may use the short address arithmetic.
+int launch_rows_f32(const AggArgs &a, int phase, int vec, bool off32, hipStream_t st);
+int launch_rows_bf16(const AggArgs &a, int phase, int vec, bool off32, hipStream_t st);
+
+}  // namespace rofk
+
+#endif

@@ -26,13 +26,13 @@ EXPORT_NAMES = ("group_ptr", "group_col", "group_dst_ptr", "group_dst", "res_ptr
 
 
 def lanes_per_row(feat_dim, bf16=False):
-    """Lanes one gathered row occupies in the kernel: smallest power of two >= ceil(F / elements per
-    16-byte load), clamped to 4..64 (mirrors the dispatch in csrc/agg_kernels.hip)."""
+    """Lanes one gathered row occupies in the kernel: the smallest of 4, 8, 10, 12, 16, 20, 32, 64 that
+    covers ceil(F / elements per 16-byte load) (mirrors rof_lanes_per_row in csrc/agg_kernels.hip)."""
     need = -(-int(feat_dim) // (8 if bf16 else 4))
-    lpr = 4
-    while lpr < need and lpr < 64:
-        lpr <<= 1
-    return lpr
+    for lpr in (4, 8, 10, 12, 16, 20, 32, 64):
+        if lpr >= need:
+            return lpr
+    return 64
 
 
 def _opts(min_consumers=0, disable_reuse=False, hub_split=0, segment=0, lanes_per_row=0):

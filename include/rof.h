@@ -106,8 +106,8 @@ typedef struct {
                              /* lanes_per_row and the plan size                                            */
     int32_t segment;         /* entries per segment; 0 = hub_split / 4                                     */
     int32_t lanes_per_row;   /* lanes one gathered row occupies in the kernel that will use this layout:   */
-                             /* smallest power of two >= ceil(feat_dim / 4) (fp32) or / 8 (bf16), 4..64;   */
-                             /* 0 = 16.  Only steers the default hub_split.                                 */
+                             /* smallest of 4,8,10,12,16,20,32,64 >= ceil(feat_dim / 4) (fp32) or / 8      */
+                             /* (bf16); 0 = 16.  Only steers the default hub_split.                         */
     int32_t reserved[3];
 } rof_layout_opts;
 
