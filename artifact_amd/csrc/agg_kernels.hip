@@ -116,8 +116,6 @@ void free_phase(rof_phase_dev &d) {
 
 inline int64_t round_up(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
 
-
-
 }  // namespace
 
 void rof_set_device_error(const char *what, const char *text) {
@@ -144,7 +142,7 @@ const char *rof_strerror(int status) {
 
 int rof_version(void) { return 1; }
 
-// Tuning knob used by the benchmark sweeps: consecutive workgroups per XCD for launch 1 / launch 2.
+// Tuning knobs used by the benchmark sweeps.
 int rof_set_lds_pad(int bytes) {
     if (bytes < 0 || bytes > 64 * 1024) return ROF_ERR_ARG;
     g_lds_pad = bytes;
@@ -173,9 +171,15 @@ int rof_layout_upload(rof_layout *L, void *stream) {
     hipStream_t st = (hipStream_t)stream;
     HIP_TRY(hipGetDevice(&L->device));
     int rc;
-    if ((rc = upload_phase(L->g, L->dg, false, st, &L->device_bytes))) return rc;
-    if ((rc = upload_phase(L->s, L->ds, false, st, &L->device_bytes))) return rc;
-    if ((rc = upload_phase(L->b, L->db, true, st, &L->device_bytes))) return rc;
+    if ((rc = upload_phase(L->g, L->dg, false, st, &L->device_bytes)) ||
+        (rc = upload_phase(L->s, L->ds, false, st, &L->device_bytes)) ||
+        (rc = upload_phase(L->b, L->db, true, st, &L->device_bytes))) {
+        free_phase(L->dg);   // nothing half-uploaded is kept
+        free_phase(L->ds);
+        free_phase(L->db);
+        L->device_bytes = 0;
+        return rc;
+    }
     HIP_TRY(hipStreamSynchronize(st));   // the host vectors may be released after this call
     L->uploaded = true;
     return ROF_OK;

@@ -26,6 +26,12 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 
+# HBM-side bytes per destination-row launch measured offline with rocprofv3 (FETCH_SIZE x 2.0 + WRITE_SIZE, the
+# factors coming from a 1 GiB copy of known size; see profiles/rof_rows_kernel_c4_f47.md).  Counters cannot be
+# read from inside this script, so the figure is carried here and reported only for the configuration it was
+# measured on: (workload, part size, width) with default layout options.
+PROFILED_TRAFFIC_BYTES = {("c4", 3, 47): 8.88e9}
+
 DESCR = {
     "c1": "c1: R-MAT 2^14 nodes, avg deg 16, self loops, GCN sym-norm, F=32, fp32",
     "c2": "c2: R-MAT 2^18 nodes, avg deg 14, self loops, GCN sym-norm, F=256, fp32",
@@ -296,6 +302,8 @@ def main():
     b_alg_plain = plain.algorithmic_bytes(feat, in_bytes)
     b_noreuse_model = e * (4 + feat * in_bytes) + n * (feat * 4 + 8)
     achieved_b = bytes_b / (ms_b * 1e-3) / 1e9
+    default_opts = not (args.hub_split or args.segment or args.min_consumers or args.fold_sources)
+    traffic = PROFILED_TRAFFIC_BYTES.get((name, ps, feat)) if default_opts else None
 
     result = {
         "metric": "GEdges/s per aggregation layer (reuse plan), 1 MI355X",
@@ -315,7 +323,7 @@ def main():
         "roofline": {
             "bound": "hbm", "kernel": "rof_rows_kernel (destination-row launch)",
             "achieved": achieved_b, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved_b / HBM_PEAK_GBS,
-            "traffic": None, "bytes_per_launch": bytes_b, "ms_per_launch": ms_b,
+            "traffic": traffic, "bytes_per_launch": bytes_b, "ms_per_launch": ms_b,
         },
         "layer": {
             "event_ms": ev_ms, "event_ms_runs": ev_r, "launch1_ms": ms_a, "launch2_ms": ms_b,
