@@ -39,7 +39,7 @@
 #include "rof_internal.h"
 
 namespace rofk {
-int g_xcd_run_a = 1, g_xcd_run_b = 16;
+int g_xcd_run_a = 1, g_xcd_run_b = 64;
 int g_lds_pad = 0;
 }  // namespace rofk
 

@@ -22,12 +22,17 @@ namespace {
 typedef std::vector<int32_t> ivec;
 
 const int32_t kShortRow = 32;        // tasks up to this many entries share a wavefront
-// Default cut for long rows, per lane group of the kernel that will run the layout (G = 64 / lanes per
-// row): a wavefront works through a task G entries at a time with a few gathers in flight, so a task of
-// hub_split entries is a serial chain of hub_split / (4 G) memory round trips.  The cut is kept below
-// ~1/1000 of all entries so that the longest chain stays short against the whole launch on small graphs.
-const int32_t kHubSplitPerGroupMax = 1024;
-const int32_t kHubSplitPerGroupMin = 64;
+// Default cut for long rows.  A wavefront works through a task G entries at a time (G = 64 / lanes per
+// row) with two gathers in flight, so a task of L entries is a serial chain of L / (2G) memory round
+// trips; the longest chain has to stay well below the duration of the launch, which grows with the number
+// of entries and with the row size (~1/G).  Measured optima on MI355X: 1024 entries at 3.6 M entries with
+// G = 1, 5000-6000 at 60 M with G = 5, 8192 at 132 M with G = 2; beyond 8192 the tail always loses.
+// Cutting finer than needed costs too: every segment writes and re-reads one partial row (bigger for
+// small G), and the launch that runs the segments has few tasks, so segments are a quarter of the cut.
+// (Giving rows between one and four cuts a whole workgroup instead -- four wavefronts combined through
+// LDS -- was measured as well: no faster than segments on any workload, so it is not built in.)
+const int64_t kEntriesPerSplitUnit = 11000;   // hub_split ~ entries / this
+const int32_t kHubSplitMax = 8192;
 // Sharing groups costs one more launch (~8 us on MI355X, the time of ~3*10^5 average row gathers), and the
 // gathers it saves are cheaper than average because the sources of a popular group are themselves popular
 // rows that sit in L2 (measured: 3-9 ps per saved gather against 24-90 ps per average gather).  Plans that
@@ -132,8 +137,8 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     if (lpr > 64) lpr = 64;
     const int32_t groups = std::max(1, 64 / lpr);
     const int64_t total = (int64_t)L->res_col.size() + (int64_t)L->group_dst.size();
-    const int64_t auto_split = std::max<int64_t>((int64_t)kHubSplitPerGroupMin * groups,
-                                                 std::min<int64_t>((int64_t)kHubSplitPerGroupMax * groups, total / 1024));
+    const int64_t floor_split = std::max<int64_t>(64 * groups, 1024 / groups);
+    const int64_t auto_split = std::max<int64_t>(floor_split, std::min<int64_t>(kHubSplitMax, total / kEntriesPerSplitUnit));
     const int32_t hub_split = (o && o->hub_split > 0) ? o->hub_split : (int32_t)auto_split;
     const int32_t segment = (o && o->segment > 0) ? o->segment : std::max(16, hub_split / 4);
     L->hub_split = hub_split;

@@ -37,7 +37,9 @@ def test_full_size_properties(big):
     out = reuse.aggregate(x, normalized=False, feat_dim=47)
     lhs = out.double().sum(0).cpu().numpy()
     rhs = (x.double() * torch.from_numpy(deg).to(dev).double()[:, None]).sum(0).cpu().numpy()
-    assert np.allclose(lhs, rhs, rtol=1e-6, atol=1e-2)
+    # fp32 rounding of 2.4 M outputs accumulates to ~1e-2 in these column sums; one lost or doubled edge
+    # would move a sum by ~1
+    assert np.allclose(lhs, rhs, rtol=1e-6, atol=0.1)
     # (3) reuse path == reuse-disabled path (same kernels) on the normalised layer
     degt = torch.from_numpy(deg).to(dev)
     reuse.set_degrees(degt)
