@@ -21,12 +21,19 @@ __all__ = ["ROF_GCN", "ROF_GIN", "ROF_inputInfo"]
 
 class ROF_GCN(torch.nn.Module):
     def __init__(self, in_feats, n_hidden, n_classes, n_layers, activation, dropout, add_self_loops=False,
-                 reuse_size=0, kernel_type="ROF_v1", bias=True):
+                 reuse_size=0, kernel_type="ROF_v1", bias=True, order="update_first", fuse_epilogue=True):
+        """`order` and `fuse_epilogue` are passed to every ROF_GCNConv (not upstream).  A ReLU activation is
+        then applied by the aggregation kernel of each hidden layer rather than as a pass of its own."""
         super().__init__()
         dims = [in_feats] + [n_hidden] * n_layers + [n_classes]
+        last = len(dims) - 2
+        self._fused_act = bool(fuse_epilogue) and kernel_type != "ROF_v1" and activation in (
+            torch.relu, torch.nn.functional.relu)
         self.layers = torch.nn.ModuleList(
             ROF_GCNConv(dims[i], dims[i + 1], bias=bias, add_self_loops=add_self_loops, reuse_size=reuse_size,
-                        kernel_type=kernel_type) for i in range(len(dims) - 1))
+                        kernel_type=kernel_type, order=order, fuse_epilogue=fuse_epilogue,
+                        activation="relu" if self._fused_act and i != last else None)
+            for i in range(len(dims) - 1))
         self.activation = activation
         self.dropout = torch.nn.Dropout(p=dropout)
 
@@ -38,7 +45,7 @@ class ROF_GCN(torch.nn.Module):
             if i != 0:
                 h = self.dropout(h)
             h = layer(h, inputInfo)
-            if i != last and self.activation is not None:
+            if i != last and self.activation is not None and not self._fused_act:
                 h = self.activation(h)
         return h
 

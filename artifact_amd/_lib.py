@@ -19,7 +19,7 @@ SYMBOLS = (
     "rof_part_intersect_count", "rof_part_intersect_lists", "rof_greedy_max_reuse", "rof_reorganize",
     "rof_transpose_csr", "rof_plan_build", "rof_layout_from_v2", "rof_layout_from_v1", "rof_layout_from_parts",
     "rof_layout_export", "rof_layout_stats", "rof_layout_upload", "rof_layout_set_degrees",
-    "rof_layout_workspace_bytes", "rof_layout_free", "rof_aggregate", "rof_aggregate_timed", "rof_set_xcd_run", "rof_aggregate_launch_times", "rof_device_copy", "rof_set_lds_pad",
+    "rof_plan_hub_patterns", "rof_layout_workspace_bytes", "rof_layout_free", "rof_aggregate", "rof_aggregate_epilogue", "rof_aggregate_timed", "rof_set_xcd_run", "rof_aggregate_launch_times", "rof_device_copy", "rof_set_lds_pad",
 )
 
 
@@ -29,7 +29,8 @@ class RofError(RuntimeError):
 
 class LayoutOpts(C.Structure):
     _fields_ = [("min_consumers", C.c_int32), ("disable_reuse", C.c_int32), ("hub_split", C.c_int32),
-                ("segment", C.c_int32), ("lanes_per_row", C.c_int32), ("reserved", C.c_int32 * 3)]
+                ("segment", C.c_int32), ("lanes_per_row", C.c_int32), ("entry_order", C.c_int32),
+                ("reserved", C.c_int32 * 2)]
 
 
 def lib():
@@ -56,6 +57,7 @@ def lib():
     L.rof_reorganize.argtypes = [vp, u64, vp, u64, vp, u64, vp, vp, vp, u32, vp, ci, ci, pp]
     L.rof_transpose_csr.argtypes = [vp, vp, u32, u64, pp]
     L.rof_plan_build.argtypes = [vp, vp, vp, vp, u32, u64, ci, ci, pp]
+    L.rof_plan_hub_patterns.argtypes = [vp, vp, u32, u64, u32, ci, pp]
     L.rof_layout_from_v2.argtypes = [vp, vp, vp, vp, i64, i32, ci, vp, pp]
     L.rof_layout_from_v1.argtypes = [vp, vp, vp, i64, vp, vp, vp, i64, i32, ci, vp, pp]
     L.rof_layout_from_parts.argtypes = [vp, vp, vp, i64, i32, ci, vp, pp]
@@ -67,6 +69,7 @@ def lib():
     L.rof_layout_workspace_bytes.argtypes = [vp, ci]
     L.rof_layout_free.argtypes = [vp]
     L.rof_aggregate.argtypes = [vp, vp, ci, i64, vp, i64, ci, ci, vp, C.c_size_t, vp]
+    L.rof_aggregate_epilogue.argtypes = [vp, vp, ci, i64, vp, i64, ci, ci, vp, ci, vp, C.c_size_t, vp]
     L.rof_aggregate_timed.argtypes = [vp, vp, ci, i64, vp, i64, ci, ci, vp, C.c_size_t, vp, ci, C.POINTER(C.c_float)]
     L.rof_set_xcd_run.argtypes = [ci, ci]
     L.rof_set_lds_pad.argtypes = [ci]

@@ -222,7 +222,7 @@ void rof_layout_free(rof_layout *L) {
 
 static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64_t ldx, float *out, int64_t ldo,
                           int feat, int normalized, void *workspace, size_t workspace_bytes, void *stream,
-                          int launches) {
+                          int launches, const float *bias = nullptr, int relu = 0) {
     if (!L || !x || !out || feat < 1 || ldx < feat || ldo < feat) return ROF_ERR_ARG;
     if (x_dtype != ROF_F32 && x_dtype != ROF_BF16) return ROF_ERR_UNSUPPORTED;
     if (!L->uploaded || (normalized && !L->weights_set)) return ROF_ERR_STATE;
@@ -283,6 +283,8 @@ static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64
         a.n_tasks = L->db.n_tasks;
         a.xcd_run = g_xcd_run_b;
         a.vec_store = (ldo % 4 == 0) && (((uintptr_t)out) % 16 == 0);
+        a.bias = bias;
+        a.relu = relu ? 1 : 0;
         if ((rc = (x_dtype == ROF_F32 ? rofk::launch_rows_f32(a, 1, vec, off32, st) : rofk::launch_rows_bf16(a, 1, vec, off32, st)))) return rc;
     }
     return ROF_OK;
@@ -291,6 +293,13 @@ static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64
 int rof_aggregate(const rof_layout *L, const void *x, int x_dtype, int64_t ldx, float *out, int64_t ldo, int feat,
                   int normalized, void *workspace, size_t workspace_bytes, void *stream) {
     return aggregate_impl(L, x, x_dtype, ldx, out, ldo, feat, normalized, workspace, workspace_bytes, stream, 3);
+}
+
+int rof_aggregate_epilogue(const rof_layout *L, const void *x, int x_dtype, int64_t ldx, float *out, int64_t ldo,
+                           int feat, int normalized, const float *bias, int relu, void *workspace,
+                           size_t workspace_bytes, void *stream) {
+    return aggregate_impl(L, x, x_dtype, ldx, out, ldo, feat, normalized, workspace, workspace_bytes, stream, 3, bias,
+                          relu);
 }
 
 int rof_aggregate_timed(const rof_layout *L, const void *x, int x_dtype, int64_t ldx, float *out, int64_t ldo,

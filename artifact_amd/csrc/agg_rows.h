@@ -43,6 +43,8 @@ struct AggArgs {
     int32_t n_blocks;          // logical workgroups
     int32_t xcd_run;           // consecutive logical workgroups kept on one XCD
     int32_t vec_store;         // output rows allow aligned 16-byte stores
+    const float *bias;         // destination-row launch only: added to every output row (null: none)
+    int32_t relu;              // destination-row launch only: clamp the output at zero
 };
 
 // Row gathers a lane group keeps in flight.  Measured on MI355X with all eight wave slots per SIMD
@@ -297,15 +299,27 @@ __global__ __launch_bounds__(256, ROF_MIN_BLOCKS) void rof_rows_kernel(AggArgs a
             float s = 1.0f;
             if (a.task_scale && end > beg) s = a.task_scale[t];
             float *o = a.out + (int64_t)a.task_out[t] * a.ldo + cstart;
+            float r[VEC];
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) r[k] = acc[k] * s;
+            if (PHASE == 1) {   // epilogue of the layer: + bias, then ReLU (columns cstart .. cstart+VEC-1 exist)
+                if (a.bias) {
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) r[k] = __fadd_rn(r[k], a.bias[cstart + k]);   // never fused into the scaling: same bits as a separate pass
+                }
+                if (a.relu) {
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) r[k] = fmaxf(r[k], 0.0f);
+                }
+            }
             if (VEC >= 4 && a.vec_store && skip == 0) {
 #pragma unroll
                 for (int k = 0; k < VEC; k += 4)
-                    *reinterpret_cast<float4 *>(o + k) =
-                        make_float4(acc[k] * s, acc[k + 1] * s, acc[k + 2] * s, acc[k + 3] * s);
+                    *reinterpret_cast<float4 *>(o + k) = make_float4(r[k], r[k + 1], r[k + 2], r[k + 3]);
             } else {
 #pragma unroll
                 for (int k = 0; k < VEC; ++k)
-                    if (k >= skip && cstart + k < a.feat) o[k] = acc[k] * s;
+                    if (k >= skip && cstart + k < a.feat) o[k] = r[k];
             }
         }
     }

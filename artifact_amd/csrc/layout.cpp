@@ -7,6 +7,7 @@
 //       launch, both filling partial-sum rows that the last launch (one task per destination) reads.  Tasks are ordered long-to-short, short ones tile by tile, so that the lanes
 //       of a wavefront that share one launch slot do the same amount of work.
 #include <algorithm>
+#include <functional>
 #include <cstdint>
 #include <cstring>
 #include <new>
@@ -33,11 +34,12 @@ const int32_t kShortRow = 32;        // tasks up to this many entries share a wa
 // LDS -- was measured as well: no faster than segments on any workload, so it is not built in.)
 const int64_t kEntriesPerSplitUnit = 11000;   // hub_split ~ entries / this
 const int32_t kHubSplitMax = 8192;
-// Sharing groups costs one more launch (~8 us on MI355X, the time of ~3*10^5 average row gathers), and the
-// gathers it saves are cheaper than average because the sources of a popular group are themselves popular
-// rows that sit in L2 (measured: 3-9 ps per saved gather against 24-90 ps per average gather).  Plans that
-// save fewer gathers than this are executed with every group folded back into its consumers.
-const int64_t kMinSavedGathers = 1000000;   // row gathers saved minus partial-row reads added
+// Sharing groups costs one more launch (~4-6 us on MI355X).  Measured gain of sharing, net of that launch,
+// against the bytes it saves ((row gathers saved - partial-row reads added) x bytes per gathered row), on two
+// machines: 128 MB -> +5 .. +18 us, 75 MB -> -1 .. +7 us, 59 MB -> -5 .. +2.5 us, 47 MB -> -8 .. +2.6 us,
+// 4 MB -> -6 us.  Sharing repays its launch somewhere between 60 and 80 MB; plans that save less than the
+// figure below are executed with every group folded back into its consumers.
+const int64_t kMinSavedBytes = 100000000;
 const int32_t kTileRows = 4096;      // short tasks are length-sorted inside tiles of this many rows
 
 bool ptr_ok(const int32_t *p, int64_t n, int64_t *total) {
@@ -145,6 +147,7 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     L->segment = segment;
     const bool disable = o && o->disable_reuse;
     const int32_t min_consumers = o ? o->min_consumers : 0;
+    const int32_t entry_order = o ? o->entry_order : 0;
 
     // node -> groups it consumes (ascending group index)
     ivec ng_ptr((size_t)n + 1, 0), ng;
@@ -172,7 +175,7 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
         int64_t cnt = L->group_dst_ptr[g + 1] - L->group_dst_ptr[g], len = L->group_ptr[g + 1] - L->group_ptr[g];
         if (worth(cnt, len)) saved += (cnt - 1) * len - cnt;
     }
-    const bool too_small = min_consumers == 0 && saved < kMinSavedGathers;
+    const bool too_small = min_consumers == 0 && saved * lpr * 16 < kMinSavedBytes;   // a lane holds 16 bytes of a row
     std::vector<int32_t> slot_of(G, -1);
     int64_t slots = 0;
     TaskList tg, ts, tb;
@@ -206,6 +209,11 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
                 row.insert(row.end(), L->group_col.begin() + L->group_ptr[g], L->group_col.begin() + L->group_ptr[g + 1]);
         }
         row.insert(row.end(), L->res_col.begin() + L->res_ptr[v], L->res_col.begin() + L->res_ptr[v + 1]);
+        // The order of the summands is free.  Walking the feature matrix monotonically keeps consecutive
+        // gathers of a task close in memory (same pages, neighbouring lines); measured on MI355X against the
+        // plan's own order: descending ids 2-3 % faster, ascending 1 % faster, a random order 20 % slower.
+        if (entry_order == 0) std::sort(row.begin() + refs, row.end(), std::greater<int32_t>());
+        else if (entry_order == 2) std::sort(row.begin() + refs, row.end());
         const int64_t len = (int64_t)row.size();
         gathered += len - refs;
         reads += refs;

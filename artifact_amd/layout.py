@@ -35,13 +35,17 @@ def lanes_per_row(feat_dim, bf16=False):
     return 64
 
 
-def _opts(min_consumers=0, disable_reuse=False, hub_split=0, segment=0, lanes_per_row=0):
+ENTRY_ORDERS = {"descending": 0, "plan": 1, "ascending": 2}
+
+
+def _opts(min_consumers=0, disable_reuse=False, hub_split=0, segment=0, lanes_per_row=0, entry_order="descending"):
     o = LayoutOpts()
     o.min_consumers = int(min_consumers)
     o.disable_reuse = int(bool(disable_reuse))
     o.hub_split = int(hub_split)
     o.segment = int(segment)
     o.lanes_per_row = int(lanes_per_row)
+    o.entry_order = ENTRY_ORDERS[entry_order]
     return o
 
 
@@ -194,16 +198,22 @@ class Layout:
             workspace = self._workspace
         return dt, f, out, workspace
 
-    def aggregate(self, x, normalized=True, out=None, feat_dim=None, workspace=None):
-        """out[v] = s(v) * sum_u w(u) x[u] through the plan; x may be a column-padded view."""
+    def aggregate(self, x, normalized=True, out=None, feat_dim=None, workspace=None, bias=None, relu=False):
+        """out[v] = act(s(v) * sum_u w(u) x[u] + bias) through the plan; x may be a column-padded view.
+        bias (float32 [feat_dim] on the device) and relu are applied as each output row is stored."""
         import torch
 
         dt, f, out, workspace = self._args(x, out, feat_dim, workspace)
         st = torch.cuda.current_stream().cuda_stream
         self.upload(st)
-        check(_lib.lib().rof_aggregate(self._h, C.c_void_p(x.data_ptr()), dt, x.stride(0), C.c_void_p(out.data_ptr()),
-                                       out.stride(0), f, int(bool(normalized)), C.c_void_p(workspace.data_ptr()),
-                                       workspace.numel() * workspace.element_size(), C.c_void_p(st)))
+        if bias is not None:
+            if (bias.dtype != torch.float32 or bias.device != x.device or bias.dim() != 1 or bias.numel() != f
+                    or not bias.is_contiguous()):
+                raise ValueError("bias must be a contiguous float32 vector of feat_dim elements on the device of x")
+        check(_lib.lib().rof_aggregate_epilogue(
+            self._h, C.c_void_p(x.data_ptr()), dt, x.stride(0), C.c_void_p(out.data_ptr()), out.stride(0), f,
+            int(bool(normalized)), C.c_void_p(bias.data_ptr() if bias is not None else None), int(bool(relu)),
+            C.c_void_p(workspace.data_ptr()), workspace.numel() * workspace.element_size(), C.c_void_p(st)))
         return out
 
     def aggregate_timed(self, x, iters, normalized=True, out=None, feat_dim=None, workspace=None):

@@ -17,7 +17,7 @@ from . import ROF
 from . import reuse_search_ext
 from .layout import Layout, LayoutFamily
 
-__all__ = ["ROF_GCNConvFunc", "ROF_GCNConv", "ROF_GINConv", "ROF_inputInfo", "build_input_info"]
+__all__ = ["ROF_GCNConvFunc", "ROF_GCNLayerFunc", "ROF_GCNConv", "ROF_GINConv", "ROF_inputInfo", "build_input_info"]
 
 _TENSOR_FIELDS = ("row_pointers", "column_index", "degrees", "part_pointers", "part2Node", "part_cache_flagindex",
                   "part_pointers_cache", "column_index_cache", "uniqpart_column_index", "uniqpart_pointers",
@@ -97,13 +97,25 @@ class ROF_inputInfo:
         return f"ROF_inputInfo(partSize={self.partSize}, warpPerBlock={self.warpPerBlock}, {shapes})"
 
 
-def build_input_info(indptr, indices, part_size=3, device="cuda", warps_per_block=4, plan=None, **layout_opts):
+def build_input_info(indptr, indices, part_size=3, device="cuda", warps_per_block=4, plan=None, search="upstream",
+                     hubs=16384, **layout_opts):
     """CSR (symmetric graph, in-neighbours = out-neighbours) -> ROF_inputInfo, following the glue of
     ROF_main.py:71-178: plan on the CPU, arrays cast to int32, degrees = diff(indptr) as float32.
-    `layout_opts` (min_consumers, disable_reuse, hub_split, segment) go to the device layout."""
+    `layout_opts` (min_consumers, disable_reuse, hub_split, segment) go to the device layout.
+    search="hub_patterns" (not upstream) fills the v2 tensors from reuse_search_ext.hub_pattern_plan with
+    `hubs` hubs in blocks of `part_size`; the GNNA / v1 tensors then describe the graph without reuse."""
     indptr = np.asarray(indptr)
     indices = np.asarray(indices)
-    if plan is None:
+    if search not in ("upstream", "hub_patterns"):
+        raise ValueError("search must be 'upstream' or 'hub_patterns'")
+    if plan is None and search == "hub_patterns":
+        plan = reuse_search_ext.hub_pattern_plan(indptr, indices, hubs, part_size)
+        empty = np.zeros(0, np.uint32)
+        ptr, p2n, _ = reuse_search_ext.py_split_part(empty, empty, indptr, part_size)
+        plan.update(new_indices_src=np.asarray(indices), part_ptr=ptr, part2Node=p2n,
+                    part_cache_flagindex=np.zeros(len(p2n), np.uint32), part_pointers_cache=np.zeros(1, np.uint32),
+                    column_index_cache=np.zeros(0, np.uint32))
+    elif plan is None:
         plan = reuse_search_ext.build_plan(indptr, indices, part_size)
     n = len(indptr) - 1
 
@@ -177,9 +189,95 @@ class ROF_GCNConvFunc(torch.autograd.Function):
         return d_input, d_weight, None, None, None
 
 
+def _family(ii, kernel_type, num_nodes):
+    """LayoutFamily for a plan container: the one built with it, else from its device tensors."""
+    fam = getattr(ii, "layouts", {}).get(kernel_type)
+    if fam is not None:
+        return fam
+    if kernel_type == "GNNA":
+        return ROF._layout_parts(ii.column_index, ii.part_pointers, ii.part2Node, num_nodes, ii.partSize)
+    if kernel_type == "ROF_v1":
+        return ROF._layout_v1(ii.column_index, ii.part_pointers, ii.part2Node, ii.part_cache_flagindex,
+                              ii.part_pointers_cache, ii.column_index_cache, num_nodes, ii.partSize)
+    if kernel_type == "ROF_v2":
+        return ROF._layout_v2(ii.uniqpart_column_index, ii.uniqpart_pointers, ii.part2Node_ptr, ii.part2Node_col,
+                              num_nodes, ii.partSize)
+    raise NotImplementedError
+
+
+class ROF_GCNLayerFunc(torch.autograd.Function):
+    """Whole GCN layer  act(A_hat (x W) + b)  as one autograd node (not upstream, which runs the bias and the
+    activation as separate passes over the output: reuse_conv.py:147-150, ROF_main.py:181).
+
+    update-first (upstream's order, reuse_conv_kernel.cu:971-1000): bias and ReLU are applied by the
+    aggregation kernel as it stores each output row.  aggregate-first evaluates (A_hat x) W instead, which
+    gathers rows of width in_channels; it is the cheaper order when in_channels < out_channels.  Both orders
+    give the same layer up to fp32 re-association.  Backward: with g = grad * (out > 0),
+    update-first  dT = A_hat g, dX = dT W^T, dW = x^T dT;  aggregate-first  dW = (A_hat x)^T g, dX = A_hat (g W^T);
+    db = column sums of g.  A_hat is symmetric, as upstream assumes (reuse_conv_kernel.cu:1021-1041)."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, inputInfo, kernel_type, relu, aggregate_first):
+        ROF._check(input=x, weight=weight)
+        fam = _family(inputInfo, kernel_type, x.shape[0])
+        deg = inputInfo.degrees
+        ctx.fam, ctx.deg, ctx.relu, ctx.aggregate_first = fam, deg, bool(relu), bool(aggregate_first)
+        ctx.has_bias = bias is not None
+        b = None if bias is None else bias.detach().contiguous()
+        if aggregate_first:
+            f = x.shape[1]
+            lay = fam.get(f)
+            lay.set_degrees(deg)
+            h = lay.aggregate(x, normalized=True, feat_dim=f)
+            out = torch.mm(h, weight) if b is None else torch.addmm(b, h, weight)
+            if relu:
+                out.relu_()
+            ctx.save_for_backward(h, weight, out if relu else None)
+        else:
+            tmp, f = ROF._update(x, weight)
+            lay = fam.get(f)
+            lay.set_degrees(deg)
+            out = lay.aggregate(tmp, normalized=True, feat_dim=f, bias=b, relu=relu)
+            ctx.save_for_backward(x, weight, out if relu else None)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        saved, weight, out = ctx.saved_tensors
+        g = grad_output.contiguous()
+        if ctx.relu:
+            g = g * (out > 0)
+        d_bias = g.sum(0) if ctx.has_bias and ctx.needs_input_grad[2] else None
+        d_x = d_w = None
+        if ctx.aggregate_first:
+            if ctx.needs_input_grad[1]:
+                d_w = torch.mm(saved.transpose(0, 1), g)
+            if ctx.needs_input_grad[0]:
+                dh = torch.mm(g, weight.transpose(0, 1))
+                lay = ctx.fam.get(dh.shape[1])
+                lay.set_degrees(ctx.deg)
+                d_x = lay.aggregate(dh, normalized=True, feat_dim=dh.shape[1])
+        elif ctx.needs_input_grad[0] or ctx.needs_input_grad[1]:
+            lay = ctx.fam.get(g.shape[1])
+            lay.set_degrees(ctx.deg)
+            dt = lay.aggregate(g, normalized=True, feat_dim=g.shape[1])
+            if ctx.needs_input_grad[0]:
+                d_x = torch.mm(dt, weight.transpose(0, 1))
+            if ctx.needs_input_grad[1]:
+                d_w = torch.mm(saved.transpose(0, 1), dt)
+        return d_x, d_w, d_bias, None, None, None, None
+
+
 class ROF_GCNConv(torch.nn.Module):
     """reuse_conv.py:96-150.  Note the upstream default add_self_loops=True raises at call time
-    (reuse_conv.py:102 with :72-73); pass add_self_loops=False as the upstream drivers do."""
+    (reuse_conv.py:102 with :72-73); pass add_self_loops=False as the upstream drivers do.
+
+    Keyword arguments beyond upstream's (all optional; the defaults reproduce upstream's arithmetic):
+      fuse_epilogue (default True)  add the bias inside the aggregation kernel instead of a separate pass
+                                    (same bits); False runs upstream's literal sequence
+      activation   None | "relu"    also apply ReLU there, so the layer returns relu(A_hat x W + b)
+      order  "update_first" (default, upstream) | "aggregate_first" | "auto" (aggregate first when
+             in_channels < out_channels)"""
 
     def __init__(self, in_channels, out_channels, bias=True, **kwargs):
         super().__init__()
@@ -200,6 +298,14 @@ class ROF_GCNConv(torch.nn.Module):
         self.dimWorker = kwargs.get("dimWorker", 0)
         if self.dimWorker == 0:
             self.dimWorker = 32 if out_channels > 32 else out_channels   # reuse_conv.py:115-120
+        self.fuse_epilogue = bool(kwargs.get("fuse_epilogue", True))
+        self.activation = kwargs.get("activation", None)
+        if self.activation not in (None, "relu"):
+            raise NotImplementedError("activation must be None or 'relu'")
+        order = kwargs.get("order", "update_first")
+        if order not in ("update_first", "aggregate_first", "auto"):
+            raise ValueError("order must be 'update_first', 'aggregate_first' or 'auto'")
+        self.aggregate_first = order == "aggregate_first" or (order == "auto" and in_channels < out_channels)
         self.reset_parameters()
 
     def reset_parameters(self):
@@ -222,8 +328,16 @@ class ROF_GCNConv(torch.nn.Module):
     def forward(self, x, inputInfo):
         inputInfo.part_result_cache = self.part_result_cache
         inputInfo.dimWorker = self.dimWorker
-        out = ROF_GCNConvFunc.apply(x, self.weight, inputInfo, self.add_self_loops, self.kernel_type)
-        return out if self.bias is None else out + self.bias
+        plain = self.activation is None and not self.aggregate_first and (self.bias is None or not self.fuse_epilogue)
+        if plain or self.kernel_type == "ROF_v1":
+            # upstream's sequence; the v1 entry points also fill the caller's cache (reuse_conv_kernel.cu:476-485)
+            out = ROF_GCNConvFunc.apply(x, self.weight, inputInfo, self.add_self_loops, self.kernel_type)
+            out = out if self.bias is None else out + self.bias
+            return torch.relu(out) if self.activation == "relu" else out
+        if self.add_self_loops:
+            raise NotImplementedError   # reuse_conv.py:72-73
+        return ROF_GCNLayerFunc.apply(x, self.weight, self.bias, inputInfo, self.kernel_type,
+                                      self.activation == "relu", self.aggregate_first)
 
 
 class _SumAggregate(torch.autograd.Function):
@@ -251,13 +365,5 @@ class ROF_GINConv(torch.nn.Module):
         self.mlp = torch.nn.Linear(in_channels, out_channels)
 
     def forward(self, x, inputInfo):
-        lay = inputInfo.layouts.get(self.kernel_type)
-        if lay is None:
-            ii = inputInfo
-            if self.kernel_type == "GNNA":
-                lay = ROF._layout_parts(ii.column_index, ii.part_pointers, ii.part2Node, x.shape[0], ii.partSize)
-            else:
-                lay = ROF._layout_v2(ii.uniqpart_column_index, ii.uniqpart_pointers, ii.part2Node_ptr,
-                                     ii.part2Node_col, x.shape[0], ii.partSize)
-        agg = _SumAggregate.apply(x, lay)
+        agg = _SumAggregate.apply(x, _family(inputInfo, self.kernel_type, x.shape[0]))
         return self.mlp((1.0 + self.eps) * x + agg)

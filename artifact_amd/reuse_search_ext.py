@@ -17,7 +17,8 @@ from . import _lib
 from ._lib import bag_take, check, ptr, u32
 
 __all__ = ["py_inverse_csc_or_csr", "py_split_part", "py_get_part_intersect", "py_greedy_max_reuse",
-           "py_reorganize_indices", "py_reorganize_indices_uniquely", "PartIntersectList", "build_plan"]
+           "py_reorganize_indices", "py_reorganize_indices_uniquely", "PartIntersectList", "build_plan",
+           "hub_pattern_plan"]
 
 
 class PartIntersectList:
@@ -165,6 +166,22 @@ def build_plan(indptr_dst, indices_src, part_size, indptr_src=None, indices_dst=
                                     None if idst is None else ptr(idst), len(ipd) - 1, len(isrc), int(part_size),
                                     int(bool(discard_remainder_part)), C.byref(h)))
     return bag_take(h, PLAN_ARRAYS)
+
+
+def hub_pattern_plan(indptr_dst, indices_src, hubs=16384, block=8):
+    """A different reuse search (not upstream's; see rof_plan_hub_patterns in include/rof.h): shared parts are
+    subsets of popularity-ranked hub blocks that many rows have in common.  Returns the four v2 arrays (same
+    format as py_reorganize_indices_uniquely, reuse_search_ext.cc:214-257) plus "hub_ids", "shared_parts" and
+    "part_size" (= block), the partSize to pass along with them."""
+    ipd, isrc = u32(indptr_dst), u32(indices_src)
+    h = C.c_void_p()
+    check(_lib.lib().rof_plan_hub_patterns(ptr(ipd), ptr(isrc), len(ipd) - 1, len(isrc), int(hubs), int(block),
+                                           C.byref(h)))
+    plan = bag_take(h, ("uniqpart_column_index", "uniqpart_pointers", "part2Node_ptr", "part2Node_col", "hub_ids",
+                        "shared_parts"))
+    plan["shared_parts"] = int(plan["shared_parts"][0])
+    plan["part_size"] = int(block)
+    return plan
 
 
 def reuse_statistics(plan, part_size, num_edges):

@@ -90,6 +90,18 @@ int rof_plan_build(const uint32_t *indptr_dst, const uint32_t *indices_src, cons
                    const uint32_t *indices_dst, uint32_t n, uint64_t e, int part_size, int discard_remainder_part,
                    rof_bag **out);
 
+/* A different reuse search, off by default: "hub patterns".  No counterpart in upstream, whose comment block at
+ * reuse_search_ext.h:305-406 sketches a stronger search than its one-part-per-source greedy and leaves it
+ * unfinished.  The `hubs` most frequent sources are tied into blocks of `block` (2..16) by popularity rank;
+ * for every destination row and block, the subset of the block's hubs among the row's in-neighbours is a
+ * pattern; a (block, pattern) of >= 2 hubs shown by enough rows becomes a shared part whose consumers are
+ * exactly those rows.  A source may thus take part in many shared parts, never in two of one row.
+ * The plan comes out in upstream's v2 format (h:537-636) with part size = block:
+ * bag: "uniqpart_column_index", "uniqpart_pointers"[U+1], "part2Node_ptr"[U+1], "part2Node_col",
+ *      "hub_ids"[<= hubs] (by rank), "shared_parts"[1]. */
+int rof_plan_hub_patterns(const uint32_t *indptr_dst, const uint32_t *indices_src, uint32_t n, uint64_t e,
+                          uint32_t hubs, int block, rof_bag **out);
+
 /* ------------------------------------------------------------------------------------------
  * Host side 2: the device layout.  A plan in any of the three upstream tensor formats is
  * re-laid out into (a) a CSR of reuse groups with their consumers and (b) a destination-centric
@@ -108,7 +120,10 @@ typedef struct {
     int32_t lanes_per_row;   /* lanes one gathered row occupies in the kernel that will use this layout:   */
                              /* smallest of 4,8,10,12,16,20,32,64 >= ceil(feat_dim / 4) (fp32) or / 8      */
                              /* (bf16); 0 = 16.  Only steers the default hub_split.                         */
-    int32_t reserved[3];
+    int32_t entry_order;     /* feature rows inside one task are gathered 0: by source id, descending      */
+                             /* (default; measured 2-3 % faster than plan order and 20 % faster than a      */
+                             /* random order on MI355X), 1: in the order the plan lists them, 2: ascending   */
+    int32_t reserved[2];
 } rof_layout_opts;
 
 /* v2 tensors: replaces the plan arguments of reuse_forward_v2 / reuse_backward_v2
@@ -169,6 +184,16 @@ enum { ROF_F32 = 0, ROF_BF16 = 1 };
 
 int rof_aggregate(const rof_layout *layout, const void *x, int x_dtype, int64_t ldx, float *out, int64_t ldo,
                   int feat_dim, int normalized, void *workspace, size_t workspace_bytes, void *stream);
+
+/* rof_aggregate with the rest of the layer fused into the store of each output row:
+ *     out[v,:] = act( aggregate(v) + bias )
+ * bias: device float32[feat_dim] or NULL (upstream adds it in a separate pass after the operator,
+ * reuse_conv.py:147-150); relu != 0 clamps at zero (upstream's models apply F.relu to the layer output
+ * as one more pass: activation=F.relu, ROF_evaluation/ROF_main.py:181-200).  Rows of nodes without in-edges become act(bias).
+ * With bias NULL and relu 0 the call is rof_aggregate. */
+int rof_aggregate_epilogue(const rof_layout *layout, const void *x, int x_dtype, int64_t ldx, float *out, int64_t ldo,
+                           int feat_dim, int normalized, const float *bias, int relu, void *workspace,
+                           size_t workspace_bytes, void *stream);
 
 /* Timing helper for benchmarks: runs rof_aggregate `iters` times on `stream` between two HIP
  * events recorded on that same stream and returns the mean milliseconds per call. */

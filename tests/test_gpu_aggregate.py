@@ -166,3 +166,46 @@ def test_empty_rows_and_isolated_nodes(oracle):
     want[3] = r[1] * (r[0] * x[1])
     assert np.allclose(got, want, rtol=1e-5, atol=1e-6)
     assert (got[[0, 2, 4, 5, 6, 7, 8, 9]] == 0).all()
+
+
+@pytest.mark.parametrize("feat,bf16", [(3, False), (47, False), (64, False), (100, False), (40, True), (256, True)])
+def test_bias_and_relu_epilogue_equal_separate_passes(oracle, feat, bf16):
+    """out = relu(aggregate + bias) stored by the kernel is bit-identical to the aggregate followed by the two
+    elementwise passes upstream runs (reuse_conv.py:147-150 adds the bias, the model applies F.relu), and
+    matches the float64 closed form; nodes without in-edges come out as relu(bias)."""
+    indptr, indices, plan = _case("c4", 6, 3)            # R-MAT with isolated nodes and no self loops
+    n = len(indptr) - 1
+    assert (np.diff(indptr) == 0).any()
+    x = features(n, feat, seed=17)
+    bias = features(1, feat, seed=18)[0] * 0.5
+    deg = np.diff(indptr).astype(np.float32)
+    lay = _layout(plan, n, 3, min_consumers=2)
+    xt = torch.from_numpy(x).cuda()
+    if bf16:
+        xt = xt.to(torch.bfloat16)
+        x = xt.float().cpu().numpy()
+    bt = torch.from_numpy(bias).cuda()
+    lay.set_degrees(torch.from_numpy(deg).cuda())
+    plain = lay.aggregate(xt, normalized=True).clone()
+    with_bias = lay.aggregate(xt, normalized=True, bias=bt).clone()
+    fused = lay.aggregate(xt, normalized=True, bias=bt, relu=True).clone()
+    only_relu = lay.aggregate(xt, normalized=True, relu=True).clone()
+    assert torch.equal(with_bias, plain + bt)
+    assert torch.equal(fused, torch.relu(plain + bt))
+    assert torch.equal(only_relu, torch.relu(plain))
+    want = np.maximum(oracle.closed_form(indptr, indices, x, deg) + bias.astype(np.float64), 0.0)
+    mag = oracle.closed_form(indptr, indices, np.abs(x), deg) + np.abs(bias)
+    _close(fused.cpu().numpy(), want, mag)
+    empty = np.flatnonzero(np.diff(indptr) == 0)
+    assert np.array_equal(fused.cpu().numpy()[empty], np.broadcast_to(np.maximum(bias, 0), (len(empty), feat)))
+
+
+def test_epilogue_rejects_a_bias_of_the_wrong_shape():
+    indptr, indices, plan = _case("c1", 4, 3)
+    n = len(indptr) - 1
+    lay = _layout(plan, n, 3)
+    xt = torch.zeros((n, 8), device="cuda")
+    with pytest.raises(ValueError, match="bias must be"):
+        lay.aggregate(xt, normalized=False, bias=torch.zeros(7, device="cuda"))
+    with pytest.raises(ValueError, match="bias must be"):
+        lay.aggregate(xt, normalized=False, bias=torch.zeros(8))

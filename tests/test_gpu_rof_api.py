@@ -136,6 +136,89 @@ def test_gcn_layer_forward_and_autograd(oracle, kernel_type):
     assert np.allclose(conv.bias.grad.cpu().numpy(), coef.sum(0).cpu().numpy(), rtol=1e-4, atol=1e-3)
 
 
+@pytest.mark.parametrize("kernel_type", ["GNNA", "ROF_v2"])
+@pytest.mark.parametrize("fin,fout", [(16, 40), (40, 16)])
+def test_layer_orders_and_fused_epilogue_agree(oracle, kernel_type, fin, fout):
+    """relu(A_hat x W + b) four ways: upstream's sequence (separate bias and ReLU passes), the fused epilogue,
+    aggregate-first, and 'auto'; outputs and all three gradients against the float64 closed form."""
+    ip, ix, n, info, x, w = _setup(fin=fin, fout=fout)
+    deg = np.diff(ip).astype(np.float32)
+    bias = features(1, fout, seed=33)[0]
+    coef = features(n, fout, seed=31)
+    pre = oracle.closed_form(ip, ix, x.astype(np.float64) @ w.astype(np.float64), deg) + bias
+    want = np.maximum(pre, 0)
+    variants = {"upstream": dict(fuse_epilogue=False), "fused": dict(activation="relu"),
+                "aggregate_first": dict(activation="relu", order="aggregate_first"),
+                "auto": dict(activation="relu", order="auto")}
+    outs = {}
+    for name, kw in variants.items():
+        conv = ROF_GCNConv(fin, fout, add_self_loops=False, kernel_type=kernel_type, reuse_size=info.reuse_size,
+                           **kw).to(DEV)
+        assert conv.aggregate_first == (name == "aggregate_first" or (name == "auto" and fin < fout))
+        with torch.no_grad():
+            conv.weight.copy_(torch.from_numpy(w))
+            conv.bias.copy_(torch.from_numpy(bias))
+        xt = torch.from_numpy(x).to(DEV).requires_grad_(True)
+        out = conv(xt, info)
+        if name == "upstream":
+            out = torch.relu(out)
+        (out * torch.from_numpy(coef).to(DEV)).sum().backward()
+        outs[name] = out.detach().cpu().numpy()
+        assert np.allclose(outs[name], want, rtol=2e-5, atol=2e-5), name
+        # the ReLU mask is taken from the layer's own output (a pre-activation within rounding of zero may
+        # land on either side in fp32); everything after the mask is checked in float64
+        mask = outs[name] > 0
+        assert (mask == (pre > 0)).mean() > 0.9999
+        g = coef * mask                                           # d loss / d pre-activation
+        ag = oracle.closed_form(ip, ix, g, deg)                   # symmetric graph
+        assert np.allclose(xt.grad.cpu().numpy(), ag @ w.astype(np.float64).T, rtol=1e-4, atol=1e-4), name
+        assert np.allclose(conv.weight.grad.cpu().numpy(), x.astype(np.float64).T @ ag, rtol=1e-4, atol=1e-3), name
+        assert np.allclose(conv.bias.grad.cpu().numpy(), g.sum(0), rtol=1e-4, atol=1e-3), name
+    assert np.array_equal(outs["upstream"], outs["fused"])       # the fused epilogue changes no bit
+
+
+def test_first_layer_without_input_gradient_skips_nothing_it_needs(oracle):
+    """x.requires_grad False (the first layer of a model): both orders still produce dW and db."""
+    ip, ix, n, info, x, w = _setup(fin=16, fout=40)
+    deg = np.diff(ip).astype(np.float32)
+    coef = features(n, 40, seed=31)
+    ag = oracle.closed_form(ip, ix, coef, deg)
+    for order in ("update_first", "aggregate_first"):
+        conv = ROF_GCNConv(16, 40, add_self_loops=False, kernel_type="ROF_v2", order=order).to(DEV)
+        with torch.no_grad():
+            conv.weight.copy_(torch.from_numpy(w))
+        xt = torch.from_numpy(x).to(DEV)
+        (conv(xt, info) * torch.from_numpy(coef).to(DEV)).sum().backward()
+        assert xt.grad is None
+        assert np.allclose(conv.weight.grad.cpu().numpy(), x.astype(np.float64).T @ ag, rtol=1e-4, atol=1e-3), order
+        assert np.allclose(conv.bias.grad.cpu().numpy(), coef.sum(0), rtol=1e-4, atol=1e-3), order
+
+
+@pytest.mark.parametrize("kernel_type", ["GNNA", "ROF_v1", "ROF_v2"])
+def test_hub_pattern_plan_through_the_operator_api(oracle, kernel_type):
+    """The plan of the hub-pattern search travels in upstream's v2 tensors; all three kernel types give the
+    closed form on it (v1 / GNNA see the same graph without reuse)."""
+    ip, ix = make_workload("c4", 5)
+    n = len(ip) - 1
+    info = build_input_info(ip, ix, part_size=8, device=DEV, search="hub_patterns", hubs=4096, min_consumers=3)
+    assert info.layouts["ROF_v2"].get(40).stats()["materialised_groups"] > 100
+    x, w = features(n, 24, seed=51), glorot(24, 40, seed=52)
+    conv = ROF_GCNConv(24, 40, add_self_loops=False, kernel_type=kernel_type, reuse_size=info.reuse_size).to(DEV)
+    with torch.no_grad():
+        conv.weight.copy_(torch.from_numpy(w))
+        conv.bias.zero_()
+        out = conv(torch.from_numpy(x).to(DEV), info).cpu().numpy()
+    deg = np.diff(ip).astype(np.float32)
+    tmp = x.astype(np.float64) @ w.astype(np.float64)
+    _close(out, oracle.closed_form(ip, ix, tmp, deg), oracle.closed_form(ip, ix, np.abs(tmp), deg), rtol=2e-5)
+    if kernel_type == "ROF_v2":                               # and through the bare operator with the device tensors
+        ii = info
+        out2 = ROF.reuse_forward_v2(torch.from_numpy(x).to(DEV), torch.from_numpy(w).to(DEV),
+                                    ii.uniqpart_column_index, ii.degrees, ii.uniqpart_pointers, ii.part2Node_ptr,
+                                    ii.part2Node_col, ii.partSize, 32, 4)[0].cpu().numpy()
+        _close(out2, oracle.closed_form(ip, ix, tmp, deg), oracle.closed_form(ip, ix, np.abs(tmp), deg), rtol=2e-5)
+
+
 def test_two_layer_gcn_forward_matches_dense_reference(oracle):
     """Workload 2 in miniature: 128 -> 256 -> 40 with ReLU between the layers."""
     ip, ix = make_workload("c2", 6)

@@ -53,11 +53,21 @@ def test_toy_layout_literal():
     assert sorted(ex["g_task_out"].tolist()) == [0, 1]
     rows = {int(o): ex["b_col"][ex["b_task_ptr"][t]:ex["b_task_ptr"][t + 1]].tolist()
             for t, o in enumerate(ex["b_task_out"])}
-    assert rows[0] == [10] and rows[2] == [10, 6] and rows[3] == [11, 7] and rows[6] == [2, 7] and rows[9] == [5]
+    # feature rows of a task are listed by descending id (the default entry order), after the partial rows
+    assert rows[0] == [10] and rows[2] == [10, 6] and rows[3] == [11, 7] and rows[6] == [7, 2] and rows[9] == [5]
+    ex = _v2(plan, 10, 3, min_consumers=2, entry_order="plan").export()
+    rows = {int(o): ex["b_col"][ex["b_task_ptr"][t]:ex["b_task_ptr"][t + 1]].tolist()
+            for t, o in enumerate(ex["b_task_out"])}
+    assert rows[6] == [2, 7] and rows[7] == [3, 6]
+    ex = _v2(plan, 10, 3, min_consumers=2, entry_order="ascending").export()
+    rows = {int(o): ex["b_col"][ex["b_task_ptr"][t]:ex["b_task_ptr"][t + 1]].tolist()
+            for t, o in enumerate(ex["b_task_out"])}
+    assert rows[6] == [2, 7] and rows[2] == [10, 6]
 
 
 OPTS = [dict(), dict(disable_reuse=True), dict(min_consumers=2), dict(min_consumers=-1), dict(hub_split=24, segment=8),
-        dict(hub_split=33, segment=32, min_consumers=2)]
+        dict(hub_split=33, segment=32, min_consumers=2), dict(entry_order="plan", min_consumers=2),
+        dict(entry_order="ascending", hub_split=24, segment=8)]
 
 
 @pytest.mark.parametrize("opts", OPTS, ids=[str(o) for o in OPTS])
@@ -83,6 +93,25 @@ def test_schedule_computes_the_closed_form(oracle, opts):
         if opts.get("min_consumers") == 2:                   # every group shared: the upstream saving (h:537-605)
             cnt = plan["intersect_count"][plan["index_picked"]].astype(np.int64)
             assert len(ix) - st["gathered_rows"] == ps * int((cnt - 1).sum())
+
+
+def test_sharing_is_gated_by_the_bytes_it_saves():
+    """The same plan is executed with its groups shared when rows are wide and folded back when they are
+    narrow: what one more launch has to repay is bytes (net saved gathers x row bytes, 16 per lane)."""
+    ip, ix = make_workload("hr", 5)                          # 32 768 nodes, most neighbours in shared anchor sets
+    n = len(ip) - 1
+    plan = R.build_plan(ip, ix, 3)
+    cnt = plan["intersect_count"][plan["index_picked"]].astype(np.int64)
+    cnt = cnt[cnt >= 3]                                      # groups the per-group rule shares at ps = 3
+    net = int(((cnt - 1) * 3 - cnt).sum())
+    assert net * 8 * 16 < 100_000_000 <= net * 16 * 16       # 128-byte rows: below the gate; 256-byte rows: above
+    narrow = _v2(plan, n, 3, lanes_per_row=8).stats()
+    wide = _v2(plan, n, 3, lanes_per_row=16).stats()
+    assert narrow["materialised_groups"] == 0 and narrow["gathered_rows"] == len(ix)
+    assert wide["materialised_groups"] == len(cnt)
+    assert len(ix) - wide["gathered_rows"] - wide["partial_reads"] == net
+    forced = _v2(plan, n, 3, lanes_per_row=8, min_consumers=3).stats()   # an explicit threshold bypasses the gate
+    assert forced["materialised_groups"] == len(cnt)
 
 
 def test_long_tasks_come_first_and_short_tasks_are_sorted_inside_tiles():
