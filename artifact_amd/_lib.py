@@ -19,7 +19,7 @@ SYMBOLS = (
     "rof_part_intersect_count", "rof_part_intersect_lists", "rof_greedy_max_reuse", "rof_reorganize",
     "rof_transpose_csr", "rof_plan_build", "rof_layout_from_v2", "rof_layout_from_v1", "rof_layout_from_parts",
     "rof_layout_export", "rof_layout_stats", "rof_layout_upload", "rof_layout_set_degrees",
-    "rof_plan_hub_patterns", "rof_layout_workspace_bytes", "rof_layout_free", "rof_aggregate", "rof_aggregate_epilogue", "rof_aggregate_timed", "rof_set_xcd_run", "rof_aggregate_launch_times", "rof_device_copy", "rof_set_lds_pad",
+    "rof_plan_hub_patterns", "rof_column_sums", "rof_column_sums_workspace_bytes", "rof_layout_workspace_bytes", "rof_layout_free", "rof_aggregate", "rof_aggregate_epilogue", "rof_aggregate_timed", "rof_set_xcd_run", "rof_aggregate_launch_times", "rof_device_copy", "rof_set_lds_pad",
 )
 
 
@@ -69,9 +69,12 @@ def lib():
     L.rof_layout_workspace_bytes.argtypes = [vp, ci]
     L.rof_layout_free.argtypes = [vp]
     L.rof_aggregate.argtypes = [vp, vp, ci, i64, vp, i64, ci, ci, vp, C.c_size_t, vp]
-    L.rof_aggregate_epilogue.argtypes = [vp, vp, ci, i64, vp, i64, ci, ci, vp, ci, vp, C.c_size_t, vp]
+    L.rof_aggregate_epilogue.argtypes = [vp, vp, ci, i64, vp, ci, i64, ci, ci, vp, ci, vp, C.c_size_t, vp]
     L.rof_aggregate_timed.argtypes = [vp, vp, ci, i64, vp, i64, ci, ci, vp, C.c_size_t, vp, ci, C.POINTER(C.c_float)]
     L.rof_set_xcd_run.argtypes = [ci, ci]
+    L.rof_column_sums_workspace_bytes.argtypes = [i64, ci]
+    L.rof_column_sums_workspace_bytes.restype = C.c_size_t
+    L.rof_column_sums.argtypes = [vp, ci, i64, i64, ci, vp, vp, C.c_size_t, vp]
     L.rof_set_lds_pad.argtypes = [ci]
     L.rof_device_copy.argtypes = [vp, vp, C.c_size_t, vp]
     L.rof_aggregate_launch_times.argtypes = [vp, vp, ci, i64, vp, i64, ci, ci, vp, C.c_size_t, vp, ci,

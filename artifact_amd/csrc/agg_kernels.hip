@@ -77,6 +77,54 @@ __global__ void rof_copy_kernel(const float4 *__restrict__ src, float4 *__restri
     for (; i < n16; i += stride) dst[i] = src[i];
 }
 
+// Column sums of a row-major [n, f] matrix (the bias gradient of a layer), in two launches with a fixed
+// order of summation.  A workgroup owns a run of rows; its four wavefronts take every fourth row of the run,
+// 64 lanes across 64 consecutive columns, so each load instruction reads one contiguous piece of a row.
+constexpr int kColsumBlocks = 2048;
+
+template <typename XT>
+__device__ __forceinline__ float colsum_load(const XT *p);
+template <>
+__device__ __forceinline__ float colsum_load<float>(const float *p) { return *p; }
+template <>
+__device__ __forceinline__ float colsum_load<uint16_t>(const uint16_t *p) { return __uint_as_float(((uint32_t)*p) << 16); }
+
+template <typename XT>
+__global__ __launch_bounds__(256) void rof_colsum_partial_kernel(const XT *__restrict__ x, int64_t ldx, int64_t n, int f,
+                                                                  int64_t rows_per_block, float *__restrict__ partial) {
+    __shared__ float red[4][64];
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    const int64_t r0 = (int64_t)blockIdx.x * rows_per_block;
+    const int64_t r1 = r0 + rows_per_block < n ? r0 + rows_per_block : n;
+    for (int c0 = 0; c0 < f; c0 += 64) {
+        const int c = c0 + tx;
+        float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+        if (c < f) {
+            const XT *p = x + c;
+            int64_t r = r0 + ty;
+            for (; r + 12 < r1; r += 16) {   // four independent loads in flight per lane
+                a0 += colsum_load<XT>(p + r * ldx);
+                a1 += colsum_load<XT>(p + (r + 4) * ldx);
+                a2 += colsum_load<XT>(p + (r + 8) * ldx);
+                a3 += colsum_load<XT>(p + (r + 12) * ldx);
+            }
+            for (; r < r1; r += 4) a0 += colsum_load<XT>(p + r * ldx);
+        }
+        red[ty][tx] = (a0 + a1) + (a2 + a3);
+        __syncthreads();
+        if (ty == 0 && c < f) partial[(int64_t)blockIdx.x * f + c] = (red[0][tx] + red[1][tx]) + (red[2][tx] + red[3][tx]);
+        __syncthreads();
+    }
+}
+
+__global__ void rof_colsum_final_kernel(const float *__restrict__ partial, int blocks, int f, float *__restrict__ out) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= f) return;
+    float acc = 0.f;
+    for (int b = 0; b < blocks; ++b) acc += partial[(int64_t)b * f + c];
+    out[c] = acc;
+}
+
 int upload_phase(const rof_phase_host &h, rof_phase_dev &d, bool with_scale, hipStream_t st, int64_t *bytes) {
     d.n_wave = h.n_wave;
     d.n_tasks = h.n_tasks;
@@ -156,6 +204,33 @@ int rof_set_xcd_run(int run_a, int run_b) {
     return ROF_OK;
 }
 
+size_t rof_column_sums_workspace_bytes(int64_t n, int f) {
+    if (n <= 0 || f <= 0) return 0;
+    return (size_t)kColsumBlocks * (size_t)f * sizeof(float);
+}
+
+int rof_column_sums(const void *x, int x_dtype, int64_t ldx, int64_t n, int f, float *out, void *workspace,
+                    size_t workspace_bytes, void *stream) {
+    if (!out || n < 0 || f < 1 || ldx < f || (n && !x)) return ROF_ERR_ARG;
+    if (x_dtype != ROF_F32 && x_dtype != ROF_BF16) return ROF_ERR_UNSUPPORTED;
+    if (!workspace || workspace_bytes < rof_column_sums_workspace_bytes(n > 0 ? n : 1, f)) return ROF_ERR_WORKSPACE;
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t want = (n + 63) / 64;   // at least 64 rows per workgroup
+    const int blocks = (int)(want < 1 ? 1 : (want > kColsumBlocks ? kColsumBlocks : want));
+    const int64_t rows_per_block = n ? (n + blocks - 1) / blocks : 0;
+    float *partial = (float *)workspace;
+    if (x_dtype == ROF_F32)
+        hipLaunchKernelGGL(rof_colsum_partial_kernel<float>, dim3(blocks), dim3(256), 0, st, (const float *)x, ldx, n, f,
+                           rows_per_block, partial);
+    else
+        hipLaunchKernelGGL(rof_colsum_partial_kernel<uint16_t>, dim3(blocks), dim3(256), 0, st, (const uint16_t *)x, ldx,
+                           n, f, rows_per_block, partial);
+    HIP_TRY(hipGetLastError());
+    hipLaunchKernelGGL(rof_colsum_final_kernel, dim3((f + 255) / 256), dim3(256), 0, st, partial, blocks, f, out);
+    HIP_TRY(hipGetLastError());
+    return ROF_OK;
+}
+
 int rof_device_copy(void *dst, const void *src, size_t nbytes, void *stream) {
     if (!dst || !src || (nbytes & 15) || (((uintptr_t)dst | (uintptr_t)src) & 15)) return ROF_ERR_ARG;
     if (nbytes == 0) return ROF_OK;
@@ -220,11 +295,13 @@ void rof_layout_free(rof_layout *L) {
     delete L;
 }
 
-static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64_t ldx, float *out, int64_t ldo,
+static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64_t ldx, void *out, int64_t ldo,
                           int feat, int normalized, void *workspace, size_t workspace_bytes, void *stream,
-                          int launches, const float *bias = nullptr, int relu = 0) {
+                          int launches, const float *bias = nullptr, int relu = 0, int out_dtype = ROF_F32) {
     if (!L || !x || !out || feat < 1 || ldx < feat || ldo < feat) return ROF_ERR_ARG;
     if (x_dtype != ROF_F32 && x_dtype != ROF_BF16) return ROF_ERR_UNSUPPORTED;
+    if (out_dtype != ROF_F32 && out_dtype != ROF_BF16) return ROF_ERR_UNSUPPORTED;
+    if (((uintptr_t)out) % (out_dtype == ROF_F32 ? 4 : 2)) return ROF_ERR_ARG;
     if (!L->uploaded || (normalized && !L->weights_set)) return ROF_ERR_STATE;
     if ((int64_t)L->n * ldx >= ((int64_t)1 << 40) || (int64_t)L->n * ldo >= ((int64_t)1 << 40)) return ROF_ERR_UNSUPPORTED;
     const size_t need = rof_layout_workspace_bytes(L, feat);
@@ -282,7 +359,8 @@ static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64
         a.n_wave = L->db.n_wave;
         a.n_tasks = L->db.n_tasks;
         a.xcd_run = g_xcd_run_b;
-        a.vec_store = (ldo % 4 == 0) && (((uintptr_t)out) % 16 == 0);
+        a.out_bf16 = out_dtype == ROF_BF16;
+        a.vec_store = (ldo % 4 == 0) && (((uintptr_t)out) % (a.out_bf16 ? 8 : 16) == 0);
         a.bias = bias;
         a.relu = relu ? 1 : 0;
         if ((rc = (x_dtype == ROF_F32 ? rofk::launch_rows_f32(a, 1, vec, off32, st) : rofk::launch_rows_bf16(a, 1, vec, off32, st)))) return rc;
@@ -295,11 +373,11 @@ int rof_aggregate(const rof_layout *L, const void *x, int x_dtype, int64_t ldx, 
     return aggregate_impl(L, x, x_dtype, ldx, out, ldo, feat, normalized, workspace, workspace_bytes, stream, 3);
 }
 
-int rof_aggregate_epilogue(const rof_layout *L, const void *x, int x_dtype, int64_t ldx, float *out, int64_t ldo,
-                           int feat, int normalized, const float *bias, int relu, void *workspace,
+int rof_aggregate_epilogue(const rof_layout *L, const void *x, int x_dtype, int64_t ldx, void *out, int out_dtype,
+                           int64_t ldo, int feat, int normalized, const float *bias, int relu, void *workspace,
                            size_t workspace_bytes, void *stream) {
     return aggregate_impl(L, x, x_dtype, ldx, out, ldo, feat, normalized, workspace, workspace_bytes, stream, 3, bias,
-                          relu);
+                          relu, out_dtype);
 }
 
 int rof_aggregate_timed(const rof_layout *L, const void *x, int x_dtype, int64_t ldx, float *out, int64_t ldo,

@@ -36,7 +36,7 @@ struct AggArgs {
     const float *task_scale;   // null: no scaling
     const int32_t *col;
     const float *w;            // null: unweighted
-    float *out;
+    void *out;                 // float rows, or bf16 rows when out_bf16 (destination-row launch only)
     int64_t ldo;
     int32_t feat;
     int32_t n_wave, n_tasks;
@@ -45,7 +45,15 @@ struct AggArgs {
     int32_t vec_store;         // output rows allow aligned 16-byte stores
     const float *bias;         // destination-row launch only: added to every output row (null: none)
     int32_t relu;              // destination-row launch only: clamp the output at zero
+    int32_t out_bf16;          // destination-row launch only: store bf16 (round to nearest even)
 };
+
+// fp32 -> bf16, round to nearest even, NaN -> quiet NaN (the conversion PyTorch's .to(bfloat16) performs)
+__device__ __forceinline__ uint32_t rof_bf16_bits(float f) {
+    const uint32_t u = __float_as_uint(f);
+    if (f != f) return 0x7fc0u;
+    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
 
 // Row gathers a lane group keeps in flight.  Measured on MI355X with all eight wave slots per SIMD
 // occupied: 2 beats 4 by ~10 % on the miss-dominated workloads (more outstanding gathers per CU slow the
@@ -298,7 +306,7 @@ __global__ __launch_bounds__(256, ROF_MIN_BLOCKS) void rof_rows_kernel(AggArgs a
             // zero-initialised output upstream: reuse_conv_kernel.cu:303)
             float s = 1.0f;
             if (a.task_scale && end > beg) s = a.task_scale[t];
-            float *o = a.out + (int64_t)a.task_out[t] * a.ldo + cstart;
+            const int64_t at = (int64_t)a.task_out[t] * a.ldo + cstart;
             float r[VEC];
 #pragma unroll
             for (int k = 0; k < VEC; ++k) r[k] = acc[k] * s;
@@ -312,14 +320,30 @@ __global__ __launch_bounds__(256, ROF_MIN_BLOCKS) void rof_rows_kernel(AggArgs a
                     for (int k = 0; k < VEC; ++k) r[k] = fmaxf(r[k], 0.0f);
                 }
             }
-            if (VEC >= 4 && a.vec_store && skip == 0) {
+            if (PHASE == 1 && a.out_bf16) {
+                uint16_t *o = reinterpret_cast<uint16_t *>(a.out) + at;
+                if (VEC >= 4 && a.vec_store && skip == 0) {
 #pragma unroll
-                for (int k = 0; k < VEC; k += 4)
-                    *reinterpret_cast<float4 *>(o + k) = make_float4(r[k], r[k + 1], r[k + 2], r[k + 3]);
+                    for (int k = 0; k < VEC; k += 4)
+                        *reinterpret_cast<uint2 *>(o + k) =
+                            make_uint2(rof_bf16_bits(r[k]) | (rof_bf16_bits(r[k + 1]) << 16),
+                                       rof_bf16_bits(r[k + 2]) | (rof_bf16_bits(r[k + 3]) << 16));
+                } else {
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k)
+                        if (k >= skip && cstart + k < a.feat) o[k] = (uint16_t)rof_bf16_bits(r[k]);
+                }
             } else {
+                float *o = reinterpret_cast<float *>(a.out) + at;
+                if (VEC >= 4 && a.vec_store && skip == 0) {
 #pragma unroll
-                for (int k = 0; k < VEC; ++k)
-                    if (k >= skip && cstart + k < a.feat) o[k] = r[k];
+                    for (int k = 0; k < VEC; k += 4)
+                        *reinterpret_cast<float4 *>(o + k) = make_float4(r[k], r[k + 1], r[k + 2], r[k + 3]);
+                } else {
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k)
+                        if (k >= skip && cstart + k < a.feat) o[k] = r[k];
+                }
             }
         }
     }

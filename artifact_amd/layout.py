@@ -25,6 +25,27 @@ EXPORT_NAMES = ("group_ptr", "group_col", "group_dst_ptr", "group_dst", "res_ptr
                 "b_task_ptr", "b_task_nref", "b_task_out", "b_col")
 
 
+def column_sums(t):
+    """float32 column sums of a 2-D float32 / bfloat16 CUDA tensor with unit column stride (rof_column_sums):
+    the bias gradient of a layer.  Fixed summation order, so the result is bitwise repeatable."""
+    import torch
+
+    if not t.is_cuda or t.dim() != 2 or t.stride(1) != 1 or t.dtype not in (torch.float32, torch.bfloat16):
+        raise RofError("column_sums needs a 2-D float32 or bfloat16 CUDA tensor with unit column stride")
+    n, f = t.shape
+    out = torch.empty(f, dtype=torch.float32, device=t.device)
+    if f == 0:
+        return out
+    L = _lib.lib()
+    nbytes = L.rof_column_sums_workspace_bytes(max(n, 1), f)
+    ws = torch.empty(nbytes // 4, dtype=torch.float32, device=t.device)
+    with torch.cuda.device(t.device):
+        check(L.rof_column_sums(C.c_void_p(t.data_ptr()), ROF_BF16 if t.dtype == torch.bfloat16 else ROF_F32,
+                                t.stride(0) if n > 1 else max(f, t.stride(0)), n, f, C.c_void_p(out.data_ptr()),
+                                C.c_void_p(ws.data_ptr()), nbytes, C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    return out
+
+
 def lanes_per_row(feat_dim, bf16=False):
     """Lanes one gathered row occupies in the kernel: the smallest of 4, 8, 10, 12, 16, 20, 32, 64 that
     covers ceil(F / elements per 16-byte load) (mirrors rof_lanes_per_row in csrc/agg_kernels.hip)."""
@@ -171,7 +192,7 @@ class Layout:
     def workspace_bytes(self, feat_dim):
         return int(_lib.lib().rof_layout_workspace_bytes(self._h, int(feat_dim)))
 
-    def _args(self, x, out, feat_dim, workspace):
+    def _args(self, x, out, feat_dim, workspace, out_dtype=None):
         import torch
 
         if not x.is_cuda or x.dim() != 2 or x.stride(1) != 1:
@@ -186,9 +207,10 @@ class Layout:
             raise RofError("x must be float32 or bfloat16")
         f = x.shape[1] if feat_dim is None else int(feat_dim)
         if out is None:
-            out = torch.empty((self.num_nodes, f), dtype=torch.float32, device=x.device)
-        if out.dtype != torch.float32 or not out.is_cuda or out.dim() != 2 or out.stride(1) != 1:
-            raise RofError("out must be a 2-D float32 CUDA tensor with unit column stride")
+            out = torch.empty((self.num_nodes, f), dtype=out_dtype or torch.float32, device=x.device)
+        if (out.dtype != (out_dtype or torch.float32) or not out.is_cuda or out.dim() != 2 or out.stride(1) != 1):
+            raise RofError("out must be a 2-D CUDA tensor of the requested dtype (float32 unless out_dtype says "
+                           "bfloat16) with unit column stride")
         if out.shape[0] < self.num_nodes or out.shape[1] < f:
             raise RofError("out is too small")
         need = self.workspace_bytes(f)
@@ -198,12 +220,16 @@ class Layout:
             workspace = self._workspace
         return dt, f, out, workspace
 
-    def aggregate(self, x, normalized=True, out=None, feat_dim=None, workspace=None, bias=None, relu=False):
+    def aggregate(self, x, normalized=True, out=None, feat_dim=None, workspace=None, bias=None, relu=False,
+                  out_dtype=None):
         """out[v] = act(s(v) * sum_u w(u) x[u] + bias) through the plan; x may be a column-padded view.
-        bias (float32 [feat_dim] on the device) and relu are applied as each output row is stored."""
+        bias (float32 [feat_dim] on the device) and relu are applied as each output row is stored;
+        out_dtype=torch.bfloat16 stores the fp32 sums rounded to bf16 (default: float32)."""
         import torch
 
-        dt, f, out, workspace = self._args(x, out, feat_dim, workspace)
+        if out_dtype not in (None, torch.float32, torch.bfloat16):
+            raise RofError("out_dtype must be float32 or bfloat16")
+        dt, f, out, workspace = self._args(x, out, feat_dim, workspace, out_dtype)
         st = torch.cuda.current_stream().cuda_stream
         self.upload(st)
         if bias is not None:
@@ -211,7 +237,8 @@ class Layout:
                     or not bias.is_contiguous()):
                 raise ValueError("bias must be a contiguous float32 vector of feat_dim elements on the device of x")
         check(_lib.lib().rof_aggregate_epilogue(
-            self._h, C.c_void_p(x.data_ptr()), dt, x.stride(0), C.c_void_p(out.data_ptr()), out.stride(0), f,
+            self._h, C.c_void_p(x.data_ptr()), dt, x.stride(0), C.c_void_p(out.data_ptr()),
+            ROF_BF16 if out.dtype == torch.bfloat16 else ROF_F32, out.stride(0), f,
             int(bool(normalized)), C.c_void_p(bias.data_ptr() if bias is not None else None), int(bool(relu)),
             C.c_void_p(workspace.data_ptr()), workspace.numel() * workspace.element_size(), C.c_void_p(st)))
         return out

@@ -15,7 +15,7 @@ import torch
 
 from . import ROF
 from . import reuse_search_ext
-from .layout import Layout, LayoutFamily
+from .layout import Layout, LayoutFamily, column_sums
 
 __all__ = ["ROF_GCNConvFunc", "ROF_GCNLayerFunc", "ROF_GCNConv", "ROF_GINConv", "ROF_inputInfo", "build_input_info"]
 
@@ -205,6 +205,18 @@ def _family(ii, kernel_type, num_nodes):
     raise NotImplementedError
 
 
+def _bf16_rows(t):
+    """`t` as bfloat16 rows that start on 16-byte boundaries (row stride a multiple of 8 elements), so that the
+    kernels gather them with 16-byte loads; one pass at most (the cast writes straight into the padded buffer)."""
+    if t.dtype == torch.bfloat16 and t.stride(1) == 1 and t.stride(0) % 8 == 0:
+        return t
+    f = t.shape[1]
+    buf = torch.empty((t.shape[0], f + (-f) % 8), dtype=torch.bfloat16, device=t.device)
+    view = buf[:, :f]
+    view.copy_(t)
+    return view
+
+
 class ROF_GCNLayerFunc(torch.autograd.Function):
     """Whole GCN layer  act(A_hat (x W) + b)  as one autograd node (not upstream, which runs the bias and the
     activation as separate passes over the output: reuse_conv.py:147-150, ROF_main.py:181).
@@ -214,30 +226,52 @@ class ROF_GCNLayerFunc(torch.autograd.Function):
     gathers rows of width in_channels; it is the cheaper order when in_channels < out_channels.  Both orders
     give the same layer up to fp32 re-association.  Backward: with g = grad * (out > 0),
     update-first  dT = A_hat g, dX = dT W^T, dW = x^T dT;  aggregate-first  dW = (A_hat x)^T g, dX = A_hat (g W^T);
-    db = column sums of g.  A_hat is symmetric, as upstream assumes (reuse_conv_kernel.cu:1021-1041)."""
+    db = column sums of g.  A_hat is symmetric, as upstream assumes (reuse_conv_kernel.cu:1021-1041).
+
+    bf16=True is the mixed-precision form: every gathered row and every GEMM operand is bfloat16 (x may already
+    be), every neighbour sum is accumulated in fp32, parameters and their gradients stay fp32.  out_bf16 makes
+    the layer's output bfloat16 as well (rounded once, in the aggregation store), which is what the next such
+    layer consumes."""
 
     @staticmethod
-    def forward(ctx, x, weight, bias, inputInfo, kernel_type, relu, aggregate_first):
+    def forward(ctx, x, weight, bias, inputInfo, kernel_type, relu, aggregate_first, bf16=False, out_bf16=False):
         ROF._check(input=x, weight=weight)
         fam = _family(inputInfo, kernel_type, x.shape[0])
         deg = inputInfo.degrees
-        ctx.fam, ctx.deg, ctx.relu, ctx.aggregate_first = fam, deg, bool(relu), bool(aggregate_first)
+        ctx.fam, ctx.deg, ctx.relu, ctx.aggregate_first, ctx.bf16 = fam, deg, bool(relu), bool(aggregate_first), bool(bf16)
         ctx.has_bias = bias is not None
+        ctx.x_dtype = x.dtype
         b = None if bias is None else bias.detach().contiguous()
+        half = torch.bfloat16
+        odt = half if (bf16 and out_bf16) else torch.float32
+        if bf16:
+            x = _bf16_rows(x)
+            wb = weight.detach().to(half)
+        elif x.dtype != torch.float32:
+            raise RuntimeError("input must be float32 (or bfloat16 with compute_dtype='bf16')")
         if aggregate_first:
             f = x.shape[1]
-            lay = fam.get(f)
+            lay = fam.get(f, bf16)
             lay.set_degrees(deg)
-            h = lay.aggregate(x, normalized=True, feat_dim=f)
-            out = torch.mm(h, weight) if b is None else torch.addmm(b, h, weight)
+            h = lay.aggregate(x, normalized=True, feat_dim=f, out_dtype=half if bf16 else None)
+            if bf16:
+                out = torch.mm(h, wb)
+                out = out.to(odt) if b is None else (out.float() + b).to(odt)
+            else:
+                out = torch.mm(h, weight) if b is None else torch.addmm(b, h, weight)
             if relu:
                 out.relu_()
             ctx.save_for_backward(h, weight, out if relu else None)
         else:
-            tmp, f = ROF._update(x, weight)
-            lay = fam.get(f)
+            if bf16:
+                f = weight.shape[1]
+                pad = (-f) % 8                        # rows of the update are gathered 8 bf16 at a time
+                tmp = torch.mm(x, wb if pad == 0 else torch.cat([wb, wb.new_zeros(wb.shape[0], pad)], dim=1))
+            else:
+                tmp, f = ROF._update(x, weight)
+            lay = fam.get(f, bf16)
             lay.set_degrees(deg)
-            out = lay.aggregate(tmp, normalized=True, feat_dim=f, bias=b, relu=relu)
+            out = lay.aggregate(tmp, normalized=True, feat_dim=f, bias=b, relu=relu, out_dtype=odt)
             ctx.save_for_backward(x, weight, out if relu else None)
         return out
 
@@ -247,25 +281,33 @@ class ROF_GCNLayerFunc(torch.autograd.Function):
         g = grad_output.contiguous()
         if ctx.relu:
             g = g * (out > 0)
-        d_bias = g.sum(0) if ctx.has_bias and ctx.needs_input_grad[2] else None
+        d_bias = column_sums(g) if ctx.has_bias and ctx.needs_input_grad[2] else None
         d_x = d_w = None
+        half = torch.bfloat16
+        if ctx.bf16:
+            g = _bf16_rows(g)
+            wb = weight.to(half)
+        else:
+            wb = weight
+        gdt = half if ctx.bf16 else None
         if ctx.aggregate_first:
             if ctx.needs_input_grad[1]:
-                d_w = torch.mm(saved.transpose(0, 1), g)
+                d_w = ROF._weight_grad(saved, g)
             if ctx.needs_input_grad[0]:
-                dh = torch.mm(g, weight.transpose(0, 1))
-                lay = ctx.fam.get(dh.shape[1])
+                dh = torch.mm(g, wb.transpose(0, 1))
+                dh = _bf16_rows(dh) if ctx.bf16 else dh
+                lay = ctx.fam.get(dh.shape[1], ctx.bf16)
                 lay.set_degrees(ctx.deg)
-                d_x = lay.aggregate(dh, normalized=True, feat_dim=dh.shape[1])
+                d_x = lay.aggregate(dh, normalized=True, feat_dim=dh.shape[1], out_dtype=gdt).to(ctx.x_dtype)
         elif ctx.needs_input_grad[0] or ctx.needs_input_grad[1]:
-            lay = ctx.fam.get(g.shape[1])
+            lay = ctx.fam.get(g.shape[1], ctx.bf16)
             lay.set_degrees(ctx.deg)
-            dt = lay.aggregate(g, normalized=True, feat_dim=g.shape[1])
+            dt = lay.aggregate(g, normalized=True, feat_dim=g.shape[1], out_dtype=gdt)
             if ctx.needs_input_grad[0]:
-                d_x = torch.mm(dt, weight.transpose(0, 1))
+                d_x = torch.mm(dt, wb.transpose(0, 1)).to(ctx.x_dtype)
             if ctx.needs_input_grad[1]:
-                d_w = torch.mm(saved.transpose(0, 1), dt)
-        return d_x, d_w, d_bias, None, None, None, None
+                d_w = ROF._weight_grad(saved, dt)
+        return d_x, d_w, d_bias, None, None, None, None, None, None
 
 
 class ROF_GCNConv(torch.nn.Module):
@@ -277,7 +319,10 @@ class ROF_GCNConv(torch.nn.Module):
                                     (same bits); False runs upstream's literal sequence
       activation   None | "relu"    also apply ReLU there, so the layer returns relu(A_hat x W + b)
       order  "update_first" (default, upstream) | "aggregate_first" | "auto" (aggregate first when
-             in_channels < out_channels)"""
+             in_channels < out_channels)
+      compute_dtype  None | "bf16"  gather bfloat16 rows and run the GEMMs on bfloat16 operands; sums are
+                                    accumulated in fp32, parameters stay fp32
+      out_dtype      None | "bf16"  with compute_dtype="bf16": return bfloat16 (rounded once, as rows are stored)"""
 
     def __init__(self, in_channels, out_channels, bias=True, **kwargs):
         super().__init__()
@@ -306,6 +351,10 @@ class ROF_GCNConv(torch.nn.Module):
         if order not in ("update_first", "aggregate_first", "auto"):
             raise ValueError("order must be 'update_first', 'aggregate_first' or 'auto'")
         self.aggregate_first = order == "aggregate_first" or (order == "auto" and in_channels < out_channels)
+        self.bf16 = kwargs.get("compute_dtype", None) in ("bf16", torch.bfloat16)
+        if kwargs.get("compute_dtype", None) not in (None, "bf16", torch.bfloat16, "fp32", torch.float32):
+            raise ValueError("compute_dtype must be None or 'bf16'")
+        self.out_bf16 = self.bf16 and kwargs.get("out_dtype", None) in ("bf16", torch.bfloat16)
         self.reset_parameters()
 
     def reset_parameters(self):
@@ -328,8 +377,9 @@ class ROF_GCNConv(torch.nn.Module):
     def forward(self, x, inputInfo):
         inputInfo.part_result_cache = self.part_result_cache
         inputInfo.dimWorker = self.dimWorker
-        plain = self.activation is None and not self.aggregate_first and (self.bias is None or not self.fuse_epilogue)
-        if plain or self.kernel_type == "ROF_v1":
+        plain = (self.activation is None and not self.aggregate_first and not self.bf16
+                 and (self.bias is None or not self.fuse_epilogue))
+        if plain or (self.kernel_type == "ROF_v1" and not self.bf16):
             # upstream's sequence; the v1 entry points also fill the caller's cache (reuse_conv_kernel.cu:476-485)
             out = ROF_GCNConvFunc.apply(x, self.weight, inputInfo, self.add_self_loops, self.kernel_type)
             out = out if self.bias is None else out + self.bias
@@ -337,7 +387,7 @@ class ROF_GCNConv(torch.nn.Module):
         if self.add_self_loops:
             raise NotImplementedError   # reuse_conv.py:72-73
         return ROF_GCNLayerFunc.apply(x, self.weight, self.bias, inputInfo, self.kernel_type,
-                                      self.activation == "relu", self.aggregate_first)
+                                      self.activation == "relu", self.aggregate_first, self.bf16, self.out_bf16)
 
 
 class _SumAggregate(torch.autograd.Function):

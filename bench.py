@@ -109,6 +109,98 @@ def cpu_baseline(indptr, indices, x32, normalized, budget_s=20.0):
     return float(np.median(times)), len(times), threads, out
 
 
+MODEL_STEPS = {
+    "c2": "2-layer GCN forward 128->256->40, ReLU between",
+    "c3": "3-layer GIN forward 64->64->64->64 (sum aggregation, eps = 0), ReLU between",
+    "c4": "one GCN layer 100->47, forward + backward (loss = sum of outputs)",
+    "c5": "2-layer GCN training step 256->256->256: forward, cross-entropy, backward through both aggregations",
+}
+
+
+def model_step(name, d, n, ps, deg, dev, timed):
+    """Milliseconds per model step of the named workload: `upstream_sequence_ms` runs update -> aggregate ->
+    bias pass -> ReLU pass per layer in fp32 as upstream's layers do; `fused_ms` lets each layer pick the
+    cheaper order and apply bias and ReLU in the aggregation store (c5: bfloat16 rows and GEMM operands)."""
+    import types
+
+    import torch
+    import torch.nn.functional as F
+
+    from artifact_amd.layout import Layout, LayoutFamily
+    from artifact_amd.reuse_conv import ROF_GCNConv, ROF_GINConv
+
+    fam = LayoutFamily(lambda lpr: Layout.from_v2(d["uniqpart_column_index"], d["uniqpart_pointers"],
+                                                  d["part2Node_ptr"], d["part2Node_col"], n, ps, lanes_per_row=lpr))
+    dummy = torch.zeros(1, dtype=torch.int32, device=dev)   # the plan tensors are not read when a layout is attached
+    info = types.SimpleNamespace(degrees=deg, layouts={"ROF_v2": fam}, partSize=ps, warpPerBlock=4,
+                                 **{k: dummy for k in ("column_index", "part_pointers", "part2Node",
+                                                       "part_cache_flagindex", "part_pointers_cache",
+                                                       "column_index_cache", "uniqpart_column_index",
+                                                       "uniqpart_pointers", "part2Node_ptr", "part2Node_col")})
+    torch.manual_seed(0)
+    res = {"what": MODEL_STEPS[name]}
+    if name == "c3":
+        layers = [ROF_GINConv(64, 64).to(dev) for _ in range(3)]
+        x = torch.randn((n, 64), device=dev)
+
+        def gin():
+            h = x
+            with torch.no_grad():
+                for i, layer in enumerate(layers):
+                    h = layer(h, info)
+                    if i != 2:
+                        h = torch.relu_(h)
+            return h
+
+        res["forward_ms"] = timed(gin, 10)
+        fam.close()
+        return res
+    dims = {"c2": [128, 256, 40], "c4": [100, 47], "c5": [256, 256, 256]}[name]
+    train = name in ("c4", "c5")
+    x = torch.randn((n, dims[0]), device=dev)
+    if name == "c5":
+        x = (torch.rand((n, dims[0]), device=dev) * 2 - 1).to(torch.bfloat16)
+        labels = torch.randint(0, dims[-1], (n,), device=dev)
+    nl = len(dims) - 1
+
+    def build(**kw):
+        return [ROF_GCNConv(dims[i], dims[i + 1], add_self_loops=False, kernel_type="ROF_v2",
+                            **{k: (v(i) if callable(v) else v) for k, v in kw.items()}).to(dev) for i in range(nl)]
+
+    base = build(bias=False)                       # bias and ReLU as separate passes, as upstream
+    base_b = [torch.zeros(dims[i + 1], device=dev, requires_grad=train) for i in range(nl)]
+    fused = build(order="auto", activation=lambda i: "relu" if i != nl - 1 else None,
+                  compute_dtype="bf16" if name == "c5" else None, out_dtype=lambda i: "bf16" if i != nl - 1 else None)
+    xf = x.float() if name == "c5" else x
+
+    def loss_of(out):
+        return F.cross_entropy(out, labels) if name == "c5" else out.sum()
+
+    def run_base():
+        with torch.set_grad_enabled(train):
+            h = xf
+            for i, layer in enumerate(base):
+                h = layer(h, info) + base_b[i]
+                if i != nl - 1:
+                    h = torch.relu(h)
+            if train:
+                loss_of(h).backward()
+
+    def run_fused():
+        with torch.set_grad_enabled(train):
+            h = x
+            for layer in fused:
+                h = layer(h, info)
+            if train:
+                loss_of(h).backward()
+
+    res["upstream_sequence_ms"] = timed(run_base, 10)
+    res["fused_ms"] = timed(run_fused, 10)
+    res["speedup"] = res["upstream_sequence_ms"] / res["fused_ms"]
+    fam.close()
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -372,6 +464,11 @@ def main():
             if lay is not reuse:
                 lay.close()
         del xin, wgt, hbuf, obuf
+
+    # ---- the workload's model step end to end (dense updates, bias, activation, backward where the workload has
+    # one), upstream's sequence of separate passes against the fused layer; the aggregation layouts are shared
+    if not args.feat and name in MODEL_STEPS:
+        extra["model_step"] = model_step(name, d, n, ps, deg, dev, timed)
 
     if args.calibrate_copy:
         import ctypes

@@ -189,10 +189,13 @@ int rof_aggregate(const rof_layout *layout, const void *x, int x_dtype, int64_t 
  *     out[v,:] = act( aggregate(v) + bias )
  * bias: device float32[feat_dim] or NULL (upstream adds it in a separate pass after the operator,
  * reuse_conv.py:147-150); relu != 0 clamps at zero (upstream's models apply F.relu to the layer output
- * as one more pass: activation=F.relu, ROF_evaluation/ROF_main.py:181-200).  Rows of nodes without in-edges become act(bias).
- * With bias NULL and relu 0 the call is rof_aggregate. */
-int rof_aggregate_epilogue(const rof_layout *layout, const void *x, int x_dtype, int64_t ldx, float *out, int64_t ldo,
-                           int feat_dim, int normalized, const float *bias, int relu, void *workspace,
+ * as one more pass: activation=F.relu, ROF_evaluation/ROF_main.py:181-200).  Rows of nodes without in-edges
+ * become act(bias).  out_dtype ROF_F32 or ROF_BF16: the sum is always accumulated in fp32; with ROF_BF16 the
+ * finished row is rounded to nearest even and stored as bf16 (row stride ldo in elements), ready to be the
+ * bf16 input of the next layer's GEMM or aggregation without a conversion pass.  With bias NULL, relu 0 and
+ * ROF_F32 the call is rof_aggregate. */
+int rof_aggregate_epilogue(const rof_layout *layout, const void *x, int x_dtype, int64_t ldx, void *out, int out_dtype,
+                           int64_t ldo, int feat_dim, int normalized, const float *bias, int relu, void *workspace,
                            size_t workspace_bytes, void *stream);
 
 /* Timing helper for benchmarks: runs rof_aggregate `iters` times on `stream` between two HIP
@@ -207,6 +210,14 @@ int rof_aggregate_timed(const rof_layout *layout, const void *x, int x_dtype, in
 int rof_aggregate_launch_times(const rof_layout *layout, const void *x, int x_dtype, int64_t ldx, float *out,
                                int64_t ldo, int feat_dim, int normalized, void *workspace, size_t workspace_bytes,
                                void *stream, int iters, float ms_launch[2]);
+
+/* Column sums of a row-major device matrix: out[c] = sum_r x[r, c], x float32 or bfloat16 [n, f] with row
+ * stride ldx (elements), out float32[f].  This is the bias gradient of a layer (upstream leaves it to autograd's
+ * reduction of `out + self.bias`, reuse_conv.py:147-150); summed in fp32 in a fixed order (bitwise repeatable).
+ * workspace: rof_column_sums_workspace_bytes(n, f) bytes of device memory. */
+size_t rof_column_sums_workspace_bytes(int64_t n, int f);
+int rof_column_sums(const void *x, int x_dtype, int64_t ldx, int64_t n, int f, float *out, void *workspace,
+                    size_t workspace_bytes, void *stream);
 
 /* Plain device-to-device streaming copy (nbytes a multiple of 16, pointers 16-byte aligned).  Exists so
  * that a profiler's FETCH_SIZE / WRITE_SIZE counters can be calibrated against a transfer of known size.

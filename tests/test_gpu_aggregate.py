@@ -209,3 +209,62 @@ def test_epilogue_rejects_a_bias_of_the_wrong_shape():
         lay.aggregate(xt, normalized=False, bias=torch.zeros(7, device="cuda"))
     with pytest.raises(ValueError, match="bias must be"):
         lay.aggregate(xt, normalized=False, bias=torch.zeros(8))
+
+
+@pytest.mark.parametrize("feat,bf16_in", [(3, False), (47, False), (64, False), (40, True), (256, True), (13, True)])
+def test_bf16_output_is_the_fp32_result_rounded_once(feat, bf16_in):
+    """out_dtype=bfloat16: the fp32 sums (+ bias, ReLU) rounded to nearest even as each row is stored -- the
+    same bits as the float32 output followed by PyTorch's .to(bfloat16); packed and padded output rows."""
+    indptr, indices, plan = _case("c4", 6, 3)
+    n = len(indptr) - 1
+    x = torch.from_numpy(features(n, feat, seed=19)).cuda()
+    if bf16_in:
+        x = x.to(torch.bfloat16)
+    bt = torch.from_numpy(features(1, feat, seed=20)[0]).cuda()
+    lay = _layout(plan, n, 3, min_consumers=2)
+    lay.set_degrees(torch.from_numpy(np.diff(indptr).astype(np.float32)).cuda())
+    want = lay.aggregate(x, normalized=True, bias=bt, relu=True).to(torch.bfloat16)
+    got = lay.aggregate(x, normalized=True, bias=bt, relu=True, out_dtype=torch.bfloat16)
+    assert got.dtype == torch.bfloat16 and torch.equal(got.view(torch.int16), want.view(torch.int16))
+    padded = torch.zeros((n, feat + (-feat) % 8 + 8), dtype=torch.bfloat16, device="cuda")
+    lay.aggregate(x, normalized=True, bias=bt, relu=True, out=padded[:, :feat], out_dtype=torch.bfloat16)
+    assert torch.equal(padded[:, :feat].view(torch.int16), want.view(torch.int16)) and (padded[:, feat:] == 0).all()
+    with pytest.raises(Exception, match="out must be"):
+        lay.aggregate(x, normalized=True, out=torch.empty((n, feat), device="cuda"), out_dtype=torch.bfloat16)
+
+
+@pytest.mark.parametrize("n,f,dtype", [(100_003, 47, "f32"), (70_000, 256, "f32"), (33_333, 300, "bf16"), (5, 3, "f32"),
+                                       (1, 8, "bf16"), (0, 4, "f32")])
+def test_column_sums_bias_gradient(n, f, dtype):
+    """rof_column_sums against a float64 sum; padded rows; repeatable bit for bit."""
+    from artifact_amd.layout import column_sums
+
+    g = torch.Generator(device="cuda").manual_seed(n + f)
+    buf = torch.randn((n, f + 5), device="cuda", generator=g)
+    if dtype == "bf16":
+        buf = buf.to(torch.bfloat16)
+    t = buf[:, :f]                                            # row stride f + 5
+    got = column_sums(t)
+    want = t.double().sum(0)
+    scale = t.double().abs().sum(0)
+    assert got.dtype == torch.float32 and got.shape == (f,)
+    assert ((got.double() - want).abs() <= 1e-6 * scale + 1e-30).all()
+    assert torch.equal(got, column_sums(t)) and torch.equal(got, column_sums(t.contiguous()))
+
+
+def test_weight_gradient_in_row_slabs():
+    """x^T d cut into row slabs and batched (ROF._weight_grad) equals the plain product; row counts that the slab
+    size does not divide, strided operands, bfloat16 operands with a float32 result."""
+    from artifact_amd.ROF import _weight_grad
+
+    g = torch.Generator(device="cuda").manual_seed(5)
+    for n, fi, fo in ((50_001, 100, 47), (16_384, 32, 40), (3_000, 7, 5)):
+        x = torch.randn((n, fi + 3), device="cuda", generator=g)[:, :fi]
+        d = torch.randn((n, fo), device="cuda", generator=g)
+        want = x.double().t() @ d.double()
+        got = _weight_grad(x, d)
+        assert got.dtype == torch.float32
+        assert (got.double() - want).norm() <= 1e-5 * want.norm()
+        gb = _weight_grad(x.to(torch.bfloat16), d.to(torch.bfloat16))
+        wantb = x.to(torch.bfloat16).double().t() @ d.to(torch.bfloat16).double()
+        assert gb.dtype == torch.float32 and (gb.double() - wantb).norm() <= 5e-3 * wantb.norm()

@@ -11,7 +11,7 @@ torch = pytest.importorskip("torch")
 import torch.nn.functional as F                                         # noqa: E402
 
 from artifact_amd.graphgen import features, make_workload               # noqa: E402
-from artifact_amd.reuse_conv import ROF_inputInfo, build_input_info     # noqa: E402
+from artifact_amd.reuse_conv import ROF_GCNConv, ROF_inputInfo, build_input_info  # noqa: E402
 from artifact_amd.ROF_models import ROF_GCN, ROF_GIN                    # noqa: E402
 from artifact_amd.train import synthetic_labels, train                  # noqa: E402
 
@@ -55,6 +55,93 @@ def test_one_training_step_matches_dense_float64_reference(kernel_type):
     # both upstream call conventions
     out3 = model(xt, None, info)
     assert out3.shape == (n, 5)
+
+
+def _bf(t):
+    """Round to bfloat16 and come back to float64: the roundings of the mixed-precision layer, restated."""
+    return t.to(torch.float32).to(torch.bfloat16).double()
+
+
+def test_bf16_training_step_matches_float64_with_the_same_roundings():
+    """The mixed-precision step of the bf16 workload in miniature: bfloat16 features, gathered rows and GEMM
+    operands, fp32 sums and parameters.  Checked twice: tightly (2e-3 in the Frobenius norm) against a float64
+    evaluation that rounds to bfloat16 at exactly the points the layer does -- operands of every GEMM, the
+    update before it is gathered, the hidden activation and the gradients handed from layer to layer -- and
+    loosely (1e-2 logits and loss, 2e-2 gradients) against plain float64 on the bf16-rounded features."""
+    ip, ix = make_workload("c5", 10)                                     # 4096 nodes, self loops
+    n = len(ip) - 1
+    info = build_input_info(ip, ix, 3, device=DEV, min_consumers=2)
+    x = torch.from_numpy(features(n, 64, seed=45, kind="uniform")).to(torch.bfloat16)
+    y = torch.from_numpy(synthetic_labels(ip, ix, x.float().numpy(), 7, seed=46))
+    torch.manual_seed(7)
+    model = ROF_GCN(64, 48, 7, 1, F.relu, 0.0, add_self_loops=False, reuse_size=info.reuse_size,
+                    kernel_type="ROF_v2", compute_dtype="bf16").to(DEV)
+    with torch.no_grad():
+        model.layers[0].bias.uniform_(-0.1, 0.1)
+        model.layers[1].bias.uniform_(-0.1, 0.1)
+    hidden = model.layers[0](x.to(DEV), info)
+    assert hidden.dtype == torch.bfloat16 and (hidden >= 0).all()       # ReLU applied in the store, bf16 hand-over
+    logits = model(x.to(DEV), info)
+    assert logits.dtype == torch.float32
+    loss = F.cross_entropy(logits, y.to(DEV))
+    loss.backward()
+    assert model.layers[0].weight.grad.dtype == torch.float32
+
+    a = _dense_norm_adj(ip, ix)
+    w1, w2 = (l.weight.detach().cpu().double() for l in model.layers)
+    b1, b2 = (l.bias.detach().cpu().double() for l in model.layers)
+    xd = x.double()
+
+    # (1) float64 with the layer's roundings, forward and backward written out
+    h = _bf(torch.relu(a @ _bf(xd @ _bf(w1)) + b1))
+    lg = (a @ _bf(h @ _bf(w2)) + b2).requires_grad_(True)
+    F.cross_entropy(lg, y).backward()
+    g2 = lg.grad
+    dt2 = _bf(a @ _bf(g2))
+    want = {"logits": lg.detach(), "db2": g2.sum(0), "dW2": h.T @ dt2}
+    g1 = _bf(dt2 @ _bf(w2).T) * (h > 0)
+    dt1 = _bf(a @ g1)
+    want.update(db1=g1.sum(0), dW1=xd.T @ dt1)
+    got = {"logits": logits, "dW1": model.layers[0].weight.grad, "db1": model.layers[0].bias.grad,
+           "dW2": model.layers[1].weight.grad, "db2": model.layers[1].bias.grad}
+    for k, w in want.items():
+        diff = (got[k].detach().cpu().double() - w).norm().item()
+        assert diff <= 2e-3 * w.norm().item(), f"{k} against the rounded evaluation: {diff / w.norm().item():.2e}"
+
+    # (2) plain float64: what the roundings cost
+    w1r, w2r, b1r, b2r = (t.clone().requires_grad_(True) for t in (w1, w2, b1, b2))
+    ref_logits = a @ (torch.relu(a @ (xd @ w1r) + b1r) @ w2r) + b2r
+    ref = F.cross_entropy(ref_logits, y)
+    ref.backward()
+    assert abs(loss.item() - ref.item()) < 1e-2 * ref.item()
+    for k, w, rel in (("logits", ref_logits.detach(), 1e-2), ("dW1", w1r.grad, 2e-2), ("db1", b1r.grad, 2e-2),
+                      ("dW2", w2r.grad, 2e-2), ("db2", b2r.grad, 2e-2)):
+        diff = (got[k].detach().cpu().double() - w).norm().item()
+        assert diff <= rel * w.norm().item(), f"{k} against plain float64: {diff / w.norm().item():.2e}"
+
+
+def test_bf16_layer_orders_agree():
+    """aggregate-first in bfloat16 (the sum is rounded before the GEMM instead of after) stays within 1e-2 of
+    update-first on the outputs and 3e-2 on the gradients (Frobenius norm)."""
+    ip, ix = make_workload("c5", 10)
+    n = len(ip) - 1
+    info = build_input_info(ip, ix, 3, device=DEV, min_consumers=2)
+    x = torch.from_numpy(features(n, 40, seed=47, kind="uniform")).to(torch.bfloat16).to(DEV)
+    coef = torch.from_numpy(features(n, 56, seed=48)).to(DEV)
+    res = {}
+    for order in ("update_first", "aggregate_first"):
+        torch.manual_seed(11)
+        conv = ROF_GCNConv(40, 56, add_self_loops=False, kernel_type="ROF_v2", compute_dtype="bf16", order=order,
+                           activation="relu").to(DEV)
+        xg = x.clone().requires_grad_(True)
+        out = conv(xg, info)
+        assert out.dtype == torch.float32
+        (out * coef).sum().backward()
+        res[order] = (out.detach(), xg.grad.float(), conv.weight.grad, conv.bias.grad)
+    # the outputs differ by bf16 roundings; the gradients also by the few ReLU masks those roundings flip
+    for u, v, what, rel in zip(res["update_first"], res["aggregate_first"], ("out", "dX", "dW", "db"),
+                               (1e-2, 3e-2, 3e-2, 3e-2)):
+        assert (u - v).norm().item() <= rel * u.norm().item(), what
 
 
 def test_training_learns_and_gin_runs():
