@@ -33,6 +33,11 @@ class LayoutOpts(C.Structure):
                 ("reserved", C.c_int32 * 2)]
 
 
+class Epilogue(C.Structure):
+    _fields_ = [("bias", C.c_void_p), ("relu", C.c_int32), ("out_dtype", C.c_int32), ("self_weight", C.c_float),
+                ("reserved", C.c_int32 * 3)]
+
+
 def lib():
     """Load librof.so once.  Raises if it is missing: build it with `python -m artifact_amd.build`."""
     global _lib
@@ -69,7 +74,7 @@ def lib():
     L.rof_layout_workspace_bytes.argtypes = [vp, ci]
     L.rof_layout_free.argtypes = [vp]
     L.rof_aggregate.argtypes = [vp, vp, ci, i64, vp, i64, ci, ci, vp, C.c_size_t, vp]
-    L.rof_aggregate_epilogue.argtypes = [vp, vp, ci, i64, vp, ci, i64, ci, ci, vp, ci, vp, C.c_size_t, vp]
+    L.rof_aggregate_epilogue.argtypes = [vp, vp, ci, i64, vp, i64, ci, ci, C.POINTER(Epilogue), vp, C.c_size_t, vp]
     L.rof_aggregate_timed.argtypes = [vp, vp, ci, i64, vp, i64, ci, ci, vp, C.c_size_t, vp, ci, C.POINTER(C.c_float)]
     L.rof_set_xcd_run.argtypes = [ci, ci]
     L.rof_column_sums_workspace_bytes.argtypes = [i64, ci]

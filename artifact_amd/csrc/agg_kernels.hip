@@ -117,12 +117,30 @@ __global__ __launch_bounds__(256) void rof_colsum_partial_kernel(const XT *__res
     }
 }
 
-__global__ void rof_colsum_final_kernel(const float *__restrict__ partial, int blocks, int f, float *__restrict__ out) {
-    const int c = blockIdx.x * blockDim.x + threadIdx.x;
-    if (c >= f) return;
-    float acc = 0.f;
-    for (int b = 0; b < blocks; ++b) acc += partial[(int64_t)b * f + c];
-    out[c] = acc;
+__global__ __launch_bounds__(1024) void rof_colsum_final_kernel(const float *__restrict__ partial, int blocks, int f,
+                                                                 float *__restrict__ out) {
+    __shared__ float red[16][64];
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;   // 64 columns x 16 slices of the partial rows
+    const int c = blockIdx.x * 64 + tx;
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    if (c < f) {
+        int b = ty;
+        for (; b + 48 < blocks; b += 64) {
+            a0 += partial[(int64_t)b * f + c];
+            a1 += partial[(int64_t)(b + 16) * f + c];
+            a2 += partial[(int64_t)(b + 32) * f + c];
+            a3 += partial[(int64_t)(b + 48) * f + c];
+        }
+        for (; b < blocks; b += 16) a0 += partial[(int64_t)b * f + c];
+    }
+    red[ty][tx] = (a0 + a1) + (a2 + a3);
+    __syncthreads();
+    if (ty == 0 && c < f) {
+        float acc = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc += red[i][tx];
+        out[c] = acc;
+    }
 }
 
 int upload_phase(const rof_phase_host &h, rof_phase_dev &d, bool with_scale, hipStream_t st, int64_t *bytes) {
@@ -226,7 +244,7 @@ int rof_column_sums(const void *x, int x_dtype, int64_t ldx, int64_t n, int f, f
         hipLaunchKernelGGL(rof_colsum_partial_kernel<uint16_t>, dim3(blocks), dim3(256), 0, st, (const uint16_t *)x, ldx,
                            n, f, rows_per_block, partial);
     HIP_TRY(hipGetLastError());
-    hipLaunchKernelGGL(rof_colsum_final_kernel, dim3((f + 255) / 256), dim3(256), 0, st, partial, blocks, f, out);
+    hipLaunchKernelGGL(rof_colsum_final_kernel, dim3((f + 63) / 64), dim3(1024), 0, st, partial, blocks, f, out);
     HIP_TRY(hipGetLastError());
     return ROF_OK;
 }
@@ -297,7 +315,8 @@ void rof_layout_free(rof_layout *L) {
 
 static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64_t ldx, void *out, int64_t ldo,
                           int feat, int normalized, void *workspace, size_t workspace_bytes, void *stream,
-                          int launches, const float *bias = nullptr, int relu = 0, int out_dtype = ROF_F32) {
+                          int launches, const float *bias = nullptr, int relu = 0, int out_dtype = ROF_F32,
+                          float self_weight = 0.0f) {
     if (!L || !x || !out || feat < 1 || ldx < feat || ldo < feat) return ROF_ERR_ARG;
     if (x_dtype != ROF_F32 && x_dtype != ROF_BF16) return ROF_ERR_UNSUPPORTED;
     if (out_dtype != ROF_F32 && out_dtype != ROF_BF16) return ROF_ERR_UNSUPPORTED;
@@ -363,6 +382,7 @@ static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64
         a.vec_store = (ldo % 4 == 0) && (((uintptr_t)out) % (a.out_bf16 ? 8 : 16) == 0);
         a.bias = bias;
         a.relu = relu ? 1 : 0;
+        a.self_weight = self_weight;
         if ((rc = (x_dtype == ROF_F32 ? rofk::launch_rows_f32(a, 1, vec, off32, st) : rofk::launch_rows_bf16(a, 1, vec, off32, st)))) return rc;
     }
     return ROF_OK;
@@ -373,11 +393,13 @@ int rof_aggregate(const rof_layout *L, const void *x, int x_dtype, int64_t ldx, 
     return aggregate_impl(L, x, x_dtype, ldx, out, ldo, feat, normalized, workspace, workspace_bytes, stream, 3);
 }
 
-int rof_aggregate_epilogue(const rof_layout *L, const void *x, int x_dtype, int64_t ldx, void *out, int out_dtype,
-                           int64_t ldo, int feat, int normalized, const float *bias, int relu, void *workspace,
-                           size_t workspace_bytes, void *stream) {
-    return aggregate_impl(L, x, x_dtype, ldx, out, ldo, feat, normalized, workspace, workspace_bytes, stream, 3, bias,
-                          relu, out_dtype);
+int rof_aggregate_epilogue(const rof_layout *L, const void *x, int x_dtype, int64_t ldx, void *out, int64_t ldo,
+                           int feat, int normalized, const rof_epilogue *ep, void *workspace, size_t workspace_bytes,
+                           void *stream) {
+    if (!ep) return aggregate_impl(L, x, x_dtype, ldx, out, ldo, feat, normalized, workspace, workspace_bytes, stream, 3);
+    if (!(ep->self_weight == ep->self_weight)) return ROF_ERR_ARG;   // NaN
+    return aggregate_impl(L, x, x_dtype, ldx, out, ldo, feat, normalized, workspace, workspace_bytes, stream, 3,
+                          ep->bias, ep->relu, ep->out_dtype, ep->self_weight);
 }
 
 int rof_aggregate_timed(const rof_layout *L, const void *x, int x_dtype, int64_t ldx, float *out, int64_t ldo,

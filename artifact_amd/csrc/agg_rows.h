@@ -46,6 +46,7 @@ struct AggArgs {
     const float *bias;         // destination-row launch only: added to every output row (null: none)
     int32_t relu;              // destination-row launch only: clamp the output at zero
     int32_t out_bf16;          // destination-row launch only: store bf16 (round to nearest even)
+    float self_weight;         // destination-row launch only: + self_weight * x[out row] (0: none)
 };
 
 // fp32 -> bf16, round to nearest even, NaN -> quiet NaN (the conversion PyTorch's .to(bfloat16) performs)
@@ -310,7 +311,13 @@ __global__ __launch_bounds__(256, ROF_MIN_BLOCKS) void rof_rows_kernel(AggArgs a
             float r[VEC];
 #pragma unroll
             for (int k = 0; k < VEC; ++k) r[k] = acc[k] * s;
-            if (PHASE == 1) {   // epilogue of the layer: + bias, then ReLU (columns cstart .. cstart+VEC-1 exist)
+            if (PHASE == 1) {   // epilogue of the layer: + own row, + bias, then ReLU (columns cstart .. cstart+VEC-1 exist)
+                if (a.self_weight != 0.0f) {
+                    float own[VEC];
+                    RowLoad<XT, VEC>::load(reinterpret_cast<const XT *>(xb + (int64_t)a.task_out[t] * xld), own);
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) r[k] = fmaf(a.self_weight, own[k], r[k]);
+                }
                 if (a.bias) {
 #pragma unroll
                     for (int k = 0; k < VEC; ++k) r[k] = __fadd_rn(r[k], a.bias[cstart + k]);   // never fused into the scaling: same bits as a separate pass

@@ -221,10 +221,10 @@ class Layout:
         return dt, f, out, workspace
 
     def aggregate(self, x, normalized=True, out=None, feat_dim=None, workspace=None, bias=None, relu=False,
-                  out_dtype=None):
-        """out[v] = act(s(v) * sum_u w(u) x[u] + bias) through the plan; x may be a column-padded view.
-        bias (float32 [feat_dim] on the device) and relu are applied as each output row is stored;
-        out_dtype=torch.bfloat16 stores the fp32 sums rounded to bf16 (default: float32)."""
+                  out_dtype=None, self_weight=0.0):
+        """out[v] = act(s(v) * sum_u w(u) x[u] + self_weight * x[v] + bias) through the plan; x may be a
+        column-padded view.  bias (float32 [feat_dim] on the device), the node's own row and relu are applied as
+        each output row is stored; out_dtype=torch.bfloat16 stores the fp32 sums rounded to bf16."""
         import torch
 
         if out_dtype not in (None, torch.float32, torch.bfloat16):
@@ -236,11 +236,12 @@ class Layout:
             if (bias.dtype != torch.float32 or bias.device != x.device or bias.dim() != 1 or bias.numel() != f
                     or not bias.is_contiguous()):
                 raise ValueError("bias must be a contiguous float32 vector of feat_dim elements on the device of x")
+        ep = _lib.Epilogue(bias.data_ptr() if bias is not None else None, int(bool(relu)),
+                           ROF_BF16 if out.dtype == torch.bfloat16 else ROF_F32, float(self_weight))
         check(_lib.lib().rof_aggregate_epilogue(
-            self._h, C.c_void_p(x.data_ptr()), dt, x.stride(0), C.c_void_p(out.data_ptr()),
-            ROF_BF16 if out.dtype == torch.bfloat16 else ROF_F32, out.stride(0), f,
-            int(bool(normalized)), C.c_void_p(bias.data_ptr() if bias is not None else None), int(bool(relu)),
-            C.c_void_p(workspace.data_ptr()), workspace.numel() * workspace.element_size(), C.c_void_p(st)))
+            self._h, C.c_void_p(x.data_ptr()), dt, x.stride(0), C.c_void_p(out.data_ptr()), out.stride(0), f,
+            int(bool(normalized)), C.byref(ep), C.c_void_p(workspace.data_ptr()),
+            workspace.numel() * workspace.element_size(), C.c_void_p(st)))
         return out
 
     def aggregate_timed(self, x, iters, normalized=True, out=None, feat_dim=None, workspace=None):

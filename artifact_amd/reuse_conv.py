@@ -391,18 +391,21 @@ class ROF_GCNConv(torch.nn.Module):
 
 
 class _SumAggregate(torch.autograd.Function):
-    """Unnormalised neighbour sum through the reuse plan; the backward pass is the same sum on the
-    gradient because the graphs are symmetric (the assumption upstream makes for GCN as well)."""
+    """self_weight * x_v + unnormalised neighbour sum through the reuse plan, the own row added as the sum is
+    stored; the backward pass is the same operator on the gradient because the graphs are symmetric (the
+    assumption upstream makes for GCN as well)."""
 
     @staticmethod
-    def forward(ctx, x, family):
-        ctx.family = family
-        return family.get(x.shape[1]).aggregate(ROF._padded(x.contiguous()), normalized=False, feat_dim=x.shape[1])
+    def forward(ctx, x, family, self_weight):
+        ctx.family, ctx.self_weight = family, float(self_weight)
+        return family.get(x.shape[1]).aggregate(x.contiguous(), normalized=False, feat_dim=x.shape[1],
+                                                self_weight=ctx.self_weight)
 
     @staticmethod
     def backward(ctx, grad):
         g = grad.contiguous()
-        return ctx.family.get(g.shape[1]).aggregate(ROF._padded(g), normalized=False, feat_dim=g.shape[1]), None
+        return ctx.family.get(g.shape[1]).aggregate(g, normalized=False, feat_dim=g.shape[1],
+                                                    self_weight=ctx.self_weight), None, None
 
 
 class ROF_GINConv(torch.nn.Module):
@@ -415,5 +418,4 @@ class ROF_GINConv(torch.nn.Module):
         self.mlp = torch.nn.Linear(in_channels, out_channels)
 
     def forward(self, x, inputInfo):
-        agg = _SumAggregate.apply(x, _family(inputInfo, self.kernel_type, x.shape[0]))
-        return self.mlp((1.0 + self.eps) * x + agg)
+        return self.mlp(_SumAggregate.apply(x, _family(inputInfo, self.kernel_type, x.shape[0]), 1.0 + self.eps))

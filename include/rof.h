@@ -186,16 +186,27 @@ int rof_aggregate(const rof_layout *layout, const void *x, int x_dtype, int64_t 
                   int feat_dim, int normalized, void *workspace, size_t workspace_bytes, void *stream);
 
 /* rof_aggregate with the rest of the layer fused into the store of each output row:
- *     out[v,:] = act( aggregate(v) + bias )
+ *     out[v,:] = act( aggregate(v) + self_weight * x[v,:] + bias )
  * bias: device float32[feat_dim] or NULL (upstream adds it in a separate pass after the operator,
- * reuse_conv.py:147-150); relu != 0 clamps at zero (upstream's models apply F.relu to the layer output
- * as one more pass: activation=F.relu, ROF_evaluation/ROF_main.py:181-200).  Rows of nodes without in-edges
- * become act(bias).  out_dtype ROF_F32 or ROF_BF16: the sum is always accumulated in fp32; with ROF_BF16 the
- * finished row is rounded to nearest even and stored as bf16 (row stride ldo in elements), ready to be the
- * bf16 input of the next layer's GEMM or aggregation without a conversion pass.  With bias NULL, relu 0 and
- * ROF_F32 the call is rof_aggregate. */
-int rof_aggregate_epilogue(const rof_layout *layout, const void *x, int x_dtype, int64_t ldx, void *out, int out_dtype,
-                           int64_t ldo, int feat_dim, int normalized, const float *bias, int relu, void *workspace,
+ *   reuse_conv.py:147-150);
+ * relu != 0 clamps at zero (upstream's models apply F.relu to the layer output as one more pass:
+ *   activation=F.relu, ROF_evaluation/ROF_main.py:181-200);
+ * self_weight: the node's own row, e.g. 1 + eps of a GIN layer over the unnormalised sum of upstream's SAG
+ *   kernel (reuse_conv_kernel.cu:123-196); 0 = none;
+ * out_dtype ROF_F32 or ROF_BF16: the sum is always accumulated in fp32; with ROF_BF16 the finished row is
+ *   rounded to nearest even and stored as bf16 (row stride ldo in elements), ready to be the bf16 input of the
+ *   next layer's GEMM or aggregation without a conversion pass.
+ * Rows of nodes without in-edges become act(self_weight * x[v] + bias).  ep == NULL is rof_aggregate. */
+typedef struct {
+    const float *bias;
+    int32_t relu;
+    int32_t out_dtype;
+    float self_weight;
+    int32_t reserved[3];
+} rof_epilogue;
+
+int rof_aggregate_epilogue(const rof_layout *layout, const void *x, int x_dtype, int64_t ldx, void *out, int64_t ldo,
+                           int feat_dim, int normalized, const rof_epilogue *epilogue, void *workspace,
                            size_t workspace_bytes, void *stream);
 
 /* Timing helper for benchmarks: runs rof_aggregate `iters` times on `stream` between two HIP

@@ -268,3 +268,21 @@ def test_weight_gradient_in_row_slabs():
         gb = _weight_grad(x.to(torch.bfloat16), d.to(torch.bfloat16))
         wantb = x.to(torch.bfloat16).double().t() @ d.to(torch.bfloat16).double()
         assert gb.dtype == torch.float32 and (gb.double() - wantb).norm() <= 5e-3 * wantb.norm()
+
+
+@pytest.mark.parametrize("feat,bf16", [(3, False), (47, False), (64, False), (40, True)])
+def test_own_row_term_of_the_epilogue(oracle, feat, bf16):
+    """out = A x + w * x_v (a GIN layer's (1 + eps) x_v + sum) equals the plain sum plus a separate pass."""
+    indptr, indices, plan = _case("c3", 6, 2)
+    n = len(indptr) - 1
+    x = torch.from_numpy(features(n, feat, seed=23)).cuda()
+    if bf16:
+        x = x.to(torch.bfloat16)
+    lay = _layout(plan, n, 2, min_consumers=2)
+    plain = lay.aggregate(x, normalized=False).clone()
+    got = lay.aggregate(x, normalized=False, self_weight=1.25, relu=True)
+    want = torch.relu(plain.double() + 1.25 * x.double())
+    assert (got.double() - want).abs().max().item() <= 1e-5 * max(1.0, want.abs().max().item())
+    ref = oracle.closed_form(indptr, indices, x.float().cpu().numpy(), normalized=False) + 1.25 * x.double().cpu().numpy()
+    mag = oracle.closed_form(indptr, indices, np.abs(x.float().cpu().numpy()), normalized=False) + 1.25 * np.abs(x.float().cpu().numpy())
+    _close(got.cpu().numpy(), np.maximum(ref, 0), mag)

@@ -242,17 +242,17 @@ def test_gin_layer_sum_aggregation_and_gradient(oracle):
     ip, ix = make_workload("c3", 6)
     n = len(ip) - 1
     info = build_input_info(ip, ix, part_size=2, device=DEV, min_consumers=2)
-    gin = ROF_GINConv(64, 64, eps=0.0).to(DEV)
+    gin = ROF_GINConv(64, 64, eps=0.3).to(DEV)
     x = features(n, 64, seed=2003)
     xt = torch.from_numpy(x).to(DEV).requires_grad_(True)
     out = gin(xt, info)
     out.sum().backward()
     w = gin.mlp.weight.detach().cpu().numpy().astype(np.float64)
     b = gin.mlp.bias.detach().cpu().numpy().astype(np.float64)
-    agg = x + oracle.closed_form(ip, ix, x, normalized=False)
+    agg = 1.3 * x + oracle.closed_form(ip, ix, x, normalized=False)
     assert np.allclose(out.detach().cpu().numpy(), agg @ w.T + b, rtol=1e-4, atol=1e-4)
     gin_grad = np.ones((n, 64)) @ w                             # d/d(agg)
-    want = gin_grad + oracle.closed_form(ip, ix, gin_grad, normalized=False)
+    want = 1.3 * gin_grad + oracle.closed_form(ip, ix, gin_grad, normalized=False)
     assert np.allclose(xt.grad.cpu().numpy(), want, rtol=1e-4, atol=1e-4)
 
 
