@@ -22,7 +22,9 @@
 //     so the groups of one wavefront finish together;
 //   * column ids and weights are fetched coalesced, one per lane, and handed to the lane groups
 //     with ds_bpermute, so the only per-entry memory instruction is the row gather itself;
-//   * workgroups are renumbered so that each XCD (own L2) works on runs of consecutive tasks.
+//   * workgroups are renumbered so that each XCD (own L2) works on runs of consecutive tasks;
+//   * the store of a destination row can apply the rest of the layer -- the node's own row times a factor,
+//     a bias, ReLU, rounding to bf16 (rof_aggregate_epilogue) -- instead of separate passes over the output.
 // MFMA is not used: there is no dense contraction here, only gather + add, bounded by HBM.
 //
 // Reference semantics: ROF/reuse_conv/reuse_conv_kernel.cu:205-286 (GNNA), 396-601 (v1),

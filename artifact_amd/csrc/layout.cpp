@@ -4,8 +4,10 @@
 //   (2) the execution schedule for the gfx950 kernels: every destination row becomes one task whose
 //       entries are either feature-row ids or "virtual" ids >= N naming a partial-sum row; groups that
 //       are worth sharing become tasks of a first launch and segments of very long rows tasks of a second
-//       launch, both filling partial-sum rows that the last launch (one task per destination) reads.  Tasks are ordered long-to-short, short ones tile by tile, so that the lanes
-//       of a wavefront that share one launch slot do the same amount of work.
+//       launch, both filling partial-sum rows that the last launch (one task per destination) reads.
+//       Tasks are ordered long-to-short, short ones tile by tile, so that the lanes of a wavefront that
+//       share one launch slot do the same amount of work; inside a task the gathered rows are listed by
+//       descending id, which keeps consecutive gathers close in memory.
 #include <algorithm>
 #include <functional>
 #include <cstdint>

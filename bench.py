@@ -27,10 +27,10 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 
 # HBM-side bytes per destination-row launch measured offline with rocprofv3 (FETCH_SIZE x 2.0 + WRITE_SIZE, the
-# factors coming from a 1 GiB copy of known size; see profiles/rof_rows_kernel_c4_f47.md).  Counters cannot be
+# factors coming from a 1 GiB copy of known size).  Counters cannot be
 # read from inside this script, so the figure is carried here and reported only for the configuration it was
 # measured on: (workload, part size, width) with default layout options.
-PROFILED_TRAFFIC_BYTES = {("c4", 3, 47): 8.48e9}
+PROFILED_TRAFFIC_BYTES = {("c4", 3, 47): 8.56e9}
 
 DESCR = {
     "c1": "c1: R-MAT 2^14 nodes, avg deg 16, self loops, GCN sym-norm, F=32, fp32",
@@ -229,7 +229,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: every machine of this build has a single MI355X and the aggregation "
-                 "path has no multi-GPU part (sharding is described in DESIGN.md); run with --gpus 1")
+                 "path has no multi-GPU part; run with --gpus 1")
 
     import torch
 

@@ -164,8 +164,8 @@ def rsqrt_rn(deg):
 
 
 def closed_form(indptr, indices, x, deg=None, normalized=True):
-    """float64 D^-1/2 A D^-1/2 x (normalized) or A x, A taken row = destination (SURVEY fact F2:
-    out[v] = rs(deg v) * sum_{u in row v} rs(deg u) x[u], cu:254,270,276,282)."""
+    """float64 D^-1/2 A D^-1/2 x (normalized) or A x, A taken row = destination:
+    out[v] = rs(deg v) * sum_{u in row v} rs(deg u) x[u] (cu:254,270,276,282)."""
     import scipy.sparse as sp
 
     n = len(indptr) - 1
