@@ -1,6 +1,7 @@
 """The large workload (2.4M nodes, ~60M directed edges) at full size, checked through properties that
 do not need an oracle run of that size: exact integer sums, a float64 checksum of checksums, linearity,
-and agreement of the reuse path with the reuse-disabled path."""
+agreement of the reuse path with the reuse-disabled path, the fused store against separate passes, and the
+hub-pattern plan against the upstream plan."""
 import numpy as np
 import pytest
 
@@ -64,3 +65,48 @@ def test_full_size_properties(big):
         want = r[v] * (xh[nb] * r[nb, None]).sum(0) if len(nb) else np.zeros(47)
         mag = r[v] * (np.abs(xh[nb]) * r[nb, None]).sum(0) if len(nb) else np.zeros(47)
         assert (np.abs(ah[v] - want) <= 1e-6 + 1e-5 * np.abs(want) + 1e-5 * mag).all(), v
+
+
+def test_full_size_epilogue_and_bias_gradient(big):
+    """At full size: bias + ReLU stored by the kernel == two separate passes, bit for bit; the bf16 store ==
+    the float32 result rounded once; the own-row term; column sums against a float64 sum."""
+    from artifact_amd.layout import column_sums
+
+    ip, ix, n, reuse, plain = big
+    dev = "cuda"
+    g = torch.Generator(device=dev).manual_seed(9)
+    x = torch.randn((n, 48), device=dev, generator=g)[:, :47]
+    bias = torch.randn(47, device=dev, generator=g)
+    reuse.set_degrees(torch.from_numpy(np.diff(ip).astype(np.float32)).to(dev))
+    base = reuse.aggregate(x, feat_dim=47).clone()
+    fused = reuse.aggregate(x, feat_dim=47, bias=bias, relu=True).clone()
+    assert torch.equal(fused, torch.relu(base + bias))
+    half = reuse.aggregate(x, feat_dim=47, bias=bias, relu=True, out_dtype=torch.bfloat16)
+    assert torch.equal(half.view(torch.int16), fused.to(torch.bfloat16).view(torch.int16))
+    own = reuse.aggregate(x, feat_dim=47, self_weight=0.5)
+    assert torch.allclose(own, base + 0.5 * x, rtol=1e-6, atol=1e-6)
+    want = fused.double().sum(0)
+    got = column_sums(fused)
+    assert ((got.double() - want).abs() <= 1e-6 * fused.double().abs().sum(0)).all()
+
+
+def test_full_size_hub_pattern_plan(big):
+    """The alternative search at full size: its plan, read as v2 tensors, gives the same layer as upstream's plan
+    (so it covers every edge exactly once) and saves several times more gathers."""
+    ip, ix, n, reuse, plain = big
+    dev = "cuda"
+    plan = R.hub_pattern_plan(ip, ix, 16384, 8)
+    lay = Layout.from_v2(plan["uniqpart_column_index"], plan["uniqpart_pointers"], plan["part2Node_ptr"],
+                         plan["part2Node_col"], n, 8, min_consumers=3)
+    net = lambda s: len(ix) - s["gathered_rows"] - s["partial_reads"]
+    # stats also count the segment reads of long rows, which both layouts have: compare the savings net of those
+    assert net(lay.stats()) + lay.stats()["hub_segments"] > 3 * (net(reuse.stats()) + reuse.stats()["hub_segments"])
+    ones = torch.ones((n, 4), device=dev)
+    got = lay.aggregate(ones, normalized=False).cpu().numpy()
+    assert np.array_equal(got, np.repeat(np.diff(ip).astype(np.float32)[:, None], 4, axis=1))   # every edge once
+    g = torch.Generator(device=dev).manual_seed(10)
+    x = torch.randn((n, 48), device=dev, generator=g)[:, :47]
+    degt = torch.from_numpy(np.diff(ip).astype(np.float32)).to(dev)
+    lay.set_degrees(degt)
+    plain.set_degrees(degt)
+    assert torch.allclose(lay.aggregate(x, feat_dim=47), plain.aggregate(x, feat_dim=47), rtol=1e-5, atol=2e-6)
