@@ -41,7 +41,7 @@
 #include "rof_internal.h"
 
 namespace rofk {
-int g_xcd_run_a = 1, g_xcd_run_b = 64;
+int g_xcd_run_a = 1, g_xcd_run_b = 0;   // 0: each layout's own choice for the destination-row launch
 int g_lds_pad = 0;
 }  // namespace rofk
 
@@ -218,7 +218,7 @@ int rof_set_lds_pad(int bytes) {
 }
 
 int rof_set_xcd_run(int run_a, int run_b) {
-    if (run_a < 1 || run_b < 1 || run_a > 4096 || run_b > 4096) return ROF_ERR_ARG;
+    if (run_a < 1 || run_b < 0 || run_a > 4096 || run_b > 4096) return ROF_ERR_ARG;
     g_xcd_run_a = run_a;
     g_xcd_run_b = run_b;
     return ROF_OK;
@@ -379,7 +379,7 @@ static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64
         a.ldo = ldo;
         a.n_wave = L->db.n_wave;
         a.n_tasks = L->db.n_tasks;
-        a.xcd_run = g_xcd_run_b;
+        a.xcd_run = g_xcd_run_b > 0 ? g_xcd_run_b : L->xcd_run;
         a.out_bf16 = out_dtype == ROF_BF16;
         a.vec_store = (ldo % 4 == 0) && (((uintptr_t)out) % (a.out_bf16 ? 8 : 16) == 0);
         a.bias = bias;

@@ -19,7 +19,7 @@ STAT_NAMES = ("nodes", "edges", "groups", "materialised_groups", "gathered_rows"
               "hub_segments", "tasks_a", "tasks_b", "device_bytes", "part_size", "wave_tasks_a", "wave_tasks_b",
               "canonical", "gathered_rows_a")
 
-EXPORT_NAMES = ("group_ptr", "group_col", "group_dst_ptr", "group_dst", "res_ptr", "res_col", "canonical",
+EXPORT_NAMES = ("group_ptr", "group_col", "group_dst_ptr", "group_dst", "res_ptr", "res_col", "canonical", "xcd_run",
                 "uniqpart_column_index", "uniqpart_pointers", "part2Node_ptr", "part2Node_col",
                 "g_task_ptr", "g_task_nref", "g_task_out", "g_col", "s_task_ptr", "s_task_nref", "s_task_out", "s_col",
                 "b_task_ptr", "b_task_nref", "b_task_out", "b_col")
@@ -151,6 +151,7 @@ class Layout:
         check(_lib.lib().rof_layout_export(self._h, C.byref(h)))
         r = bag_take(h, EXPORT_NAMES, dtype=np.int32)
         r["canonical"] = bool(r["canonical"][0])
+        r["xcd_run"] = int(r["xcd_run"][0])
         return r
 
     def stats(self):

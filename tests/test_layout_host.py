@@ -114,6 +114,15 @@ def test_sharing_is_gated_by_the_bytes_it_saves():
     assert forced["materialised_groups"] == len(cnt)
 
 
+def test_xcd_run_follows_the_locality_of_the_graph():
+    """Block-structured graphs (rows gather from their own neighbourhood) keep long runs of workgroups on one
+    XCD; graphs without that locality use short runs."""
+    ip, ix = make_workload("c3", 4)                          # SBM: 24 of 26 neighbours inside the row's own block
+    assert Layout.from_csr(ip, ix).export()["xcd_run"] == 64
+    ip, ix = make_workload("c4", 3)                          # R-MAT, 300 000 nodes: 9 % of the neighbours are nearby
+    assert Layout.from_csr(ip, ix).export()["xcd_run"] == 16
+
+
 def test_long_tasks_come_first_and_short_tasks_are_sorted_inside_tiles():
     ip, ix = make_workload("c1", 1)
     n = len(ip) - 1
