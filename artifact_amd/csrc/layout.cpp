@@ -37,12 +37,14 @@ const int32_t kShortRow = 32;        // tasks up to this many entries share a wa
 // LDS -- was measured as well: no faster than segments on any workload, so it is not built in.)
 const int64_t kEntriesPerSplitUnit = 11000;   // hub_split ~ entries / this
 const int32_t kHubSplitMax = 8192;
-// Sharing groups costs one more launch (~4-6 us on MI355X).  Measured gain of sharing, net of that launch,
-// against the bytes it saves ((row gathers saved - partial-row reads added) x bytes per gathered row), on two
-// machines: 128 MB -> +5 .. +18 us, 75 MB -> -1 .. +7 us, 59 MB -> -5 .. +2.5 us, 47 MB -> -8 .. +2.6 us,
-// 4 MB -> -6 us.  Sharing repays its launch somewhere between 60 and 80 MB; plans that save less than the
-// figure below are executed with every group folded back into its consumers.
-const int64_t kMinSavedBytes = 100000000;
+// Sharing groups costs one more launch (~4-6 us on MI355X), and what it saves is cheap: the sources of a popular
+// group are themselves popular rows that sit in L2, while the partial rows that replace them are read a few
+// dozen times each.  Measured gain of sharing, net of that launch, against the bytes it saves ((row gathers saved
+// - partial-row reads added) x bytes per gathered row): 845 MB -> 0 .. +50 us of 10.8 ms, 283 MB -> -4 us of
+// 1.4 ms, 128 MB -> -10 .. +6 us, 59 MB -> -5 .. +2.5 us, 4 MB -> -6 us; 1.9 GB on a graph with planted reuse
+// -> +310 us of 0.73 ms.  Plans that save less than the figure below are executed with every group folded back
+// into its consumers.
+const int64_t kMinSavedBytes = 256000000;
 const int32_t kTileRows = 4096;      // short tasks are length-sorted inside tiles of this many rows
 
 bool ptr_ok(const int32_t *p, int64_t n, int64_t *total) {
@@ -151,6 +153,7 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     const bool disable = o && o->disable_reuse;
     const int32_t min_consumers = o ? o->min_consumers : 0;
     const int32_t entry_order = o ? o->entry_order : 0;
+    const int64_t tile_rows = (o && o->tile_rows > 0) ? o->tile_rows : kTileRows;
 
     // node -> groups it consumes (ascending group index)
     ivec ng_ptr((size_t)n + 1, 0), ng;
@@ -255,7 +258,7 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     L->partial_reads = reads;
     finalize_phase(tg, 1 << 30, L->g);
     finalize_phase(ts, 1 << 30, L->s);
-    finalize_phase(tb, kTileRows, L->b);
+    finalize_phase(tb, tile_rows, L->b);
     L->gathered_before_rows = (int64_t)tg.col.size();
     for (size_t t = 0; t < ts.out.size(); ++t) L->gathered_before_rows += (ts.ptr[t + 1] - ts.ptr[t]) - ts.nref[t];
     return ROF_OK;

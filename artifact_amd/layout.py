@@ -59,7 +59,8 @@ def lanes_per_row(feat_dim, bf16=False):
 ENTRY_ORDERS = {"descending": 0, "plan": 1, "ascending": 2}
 
 
-def _opts(min_consumers=0, disable_reuse=False, hub_split=0, segment=0, lanes_per_row=0, entry_order="descending"):
+def _opts(min_consumers=0, disable_reuse=False, hub_split=0, segment=0, lanes_per_row=0, entry_order="descending",
+          tile_rows=0):
     o = LayoutOpts()
     o.min_consumers = int(min_consumers)
     o.disable_reuse = int(bool(disable_reuse))
@@ -67,6 +68,7 @@ def _opts(min_consumers=0, disable_reuse=False, hub_split=0, segment=0, lanes_pe
     o.segment = int(segment)
     o.lanes_per_row = int(lanes_per_row)
     o.entry_order = ENTRY_ORDERS[entry_order]
+    o.tile_rows = int(tile_rows)
     return o
 
 

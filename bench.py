@@ -220,6 +220,7 @@ def main():
     ap.add_argument("--lds-pad", type=int, default=-1, help="launch tuning: unused LDS bytes per workgroup")
     ap.add_argument("--entry-order", default="descending", choices=["descending", "plan", "ascending"],
                     help="layout tuning: order of the gathered rows inside a task")
+    ap.add_argument("--tile-rows", type=int, default=0, help="layout tuning: destinations per length-sorted tile")
     ap.add_argument("--search", default="upstream", choices=["upstream", "hub"],
                     help="reuse search: upstream's greedy (bit-exact plan) or the hub-pattern search")
     ap.add_argument("--hubs", type=int, default=16384, help="--search hub: number of hub sources")
@@ -283,10 +284,10 @@ def main():
     t0 = time.time()
     reuse = Layout.from_v2(d["uniqpart_column_index"], d["uniqpart_pointers"], d["part2Node_ptr"], d["part2Node_col"],
                            n, ps, hub_split=args.hub_split, segment=args.segment, lanes_per_row=lpr,
-                           min_consumers=args.min_consumers, entry_order=args.entry_order)
+                           min_consumers=args.min_consumers, entry_order=args.entry_order, tile_rows=args.tile_rows)
     plain = Layout.from_v2(d["uniqpart_column_index"], d["uniqpart_pointers"], d["part2Node_ptr"], d["part2Node_col"],
                            n, ps, disable_reuse=True, hub_split=args.hub_split, segment=args.segment, lanes_per_row=lpr,
-                           entry_order=args.entry_order)
+                           entry_order=args.entry_order, tile_rows=args.tile_rows)
     t_layout = time.time() - t0
     # when the cost model folds every group back (the plan saves too little), also time the plan with its
     # profitable groups forced to be shared, so the cost of the reuse machinery stays visible
@@ -294,7 +295,7 @@ def main():
     if reuse.stats()["materialised_groups"] == 0 and len(d["index_picked"]) and not args.min_consumers:
         forced = Layout.from_v2(d["uniqpart_column_index"], d["uniqpart_pointers"], d["part2Node_ptr"],
                                 d["part2Node_col"], n, ps, hub_split=args.hub_split, segment=args.segment,
-                                lanes_per_row=lpr, min_consumers=3, entry_order=args.entry_order)
+                                lanes_per_row=lpr, min_consumers=3, entry_order=args.entry_order, tile_rows=args.tile_rows)
     for lay in (reuse, plain) + ((forced,) if forced else ()):
         lay.upload()
         if normalized:
@@ -487,7 +488,7 @@ def main():
     b_noreuse_model = e * (4 + feat * in_bytes) + n * (feat * 4 + 8)
     achieved_b = bytes_b / (ms_b * 1e-3) / 1e9
     default_opts = (not (args.hub_split or args.segment or args.min_consumers or args.fold_sources)
-                    and args.search == "upstream" and args.entry_order == "descending")
+                    and args.search == "upstream" and args.entry_order == "descending" and not args.tile_rows)
     traffic = PROFILED_TRAFFIC_BYTES.get((name, ps, feat)) if default_opts else None
 
     result = {

@@ -123,7 +123,8 @@ typedef struct {
     int32_t entry_order;     /* feature rows inside one task are gathered 0: by source id, descending      */
                              /* (default; measured 2-3 % faster than plan order and 20 % faster than a      */
                              /* random order on MI355X), 1: in the order the plan lists them, 2: ascending   */
-    int32_t reserved[2];
+    int32_t tile_rows;       /* short rows are sorted by length inside tiles of this many destinations; 0 = 4096 */
+    int32_t reserved[1];
 } rof_layout_opts;
 
 /* v2 tensors: replaces the plan arguments of reuse_forward_v2 / reuse_backward_v2

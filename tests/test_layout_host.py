@@ -104,13 +104,13 @@ def test_sharing_is_gated_by_the_bytes_it_saves():
     cnt = plan["intersect_count"][plan["index_picked"]].astype(np.int64)
     cnt = cnt[cnt >= 3]                                      # groups the per-group rule shares at ps = 3
     net = int(((cnt - 1) * 3 - cnt).sum())
-    assert net * 8 * 16 < 100_000_000 <= net * 16 * 16       # 128-byte rows: below the gate; 256-byte rows: above
-    narrow = _v2(plan, n, 3, lanes_per_row=8).stats()
-    wide = _v2(plan, n, 3, lanes_per_row=16).stats()
+    assert net * 32 * 16 < 256_000_000 <= net * 64 * 16      # 512-byte rows: below the gate; 1024-byte rows: above
+    narrow = _v2(plan, n, 3, lanes_per_row=32).stats()
+    wide = _v2(plan, n, 3, lanes_per_row=64).stats()
     assert narrow["materialised_groups"] == 0 and narrow["gathered_rows"] == len(ix)
     assert wide["materialised_groups"] == len(cnt)
     assert len(ix) - wide["gathered_rows"] - wide["partial_reads"] == net
-    forced = _v2(plan, n, 3, lanes_per_row=8, min_consumers=3).stats()   # an explicit threshold bypasses the gate
+    forced = _v2(plan, n, 3, lanes_per_row=32, min_consumers=3).stats()   # an explicit threshold bypasses the gate
     assert forced["materialised_groups"] == len(cnt)
 
 
