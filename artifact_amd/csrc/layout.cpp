@@ -25,7 +25,12 @@ namespace {
 
 typedef std::vector<int32_t> ivec;
 
-const int32_t kShortRow = 32;        // tasks up to this many entries share a wavefront
+// Tasks up to this many entries share a wavefront (one lane group each); longer ones get a wavefront of their
+// own.  Measured on MI355X at 5 rows per wavefront: 64 and 128 are 1 % faster than 32 and 256 is slower; at one
+// row per wavefront 64 equals 32 and 128 is 10 % slower.  A launch too small to fill the machine twice is bound
+// by its longest task instead and keeps the lower cut (16 384 rows: 18 us against 26).
+const int32_t kShortRow = 64, kShortRowSmall = 32;
+const int64_t kWavesToFill = 2 * 8192;   // two rounds of 256 CUs x 32 wavefronts
 // Default cut for long rows.  A wavefront works through a task G entries at a time (G = 64 / lanes per
 // row) with two gathers in flight, so a task of L entries is a serial chain of L / (2G) memory round
 // trips; the longest chain has to stay well below the duration of the launch, which grows with the number
@@ -37,14 +42,17 @@ const int32_t kShortRow = 32;        // tasks up to this many entries share a wa
 // LDS -- was measured as well: no faster than segments on any workload, so it is not built in.)
 const int64_t kEntriesPerSplitUnit = 11000;   // hub_split ~ entries / this
 const int32_t kHubSplitMax = 8192;
-// Sharing groups costs one more launch (~4-6 us on MI355X), and what it saves is cheap: the sources of a popular
-// group are themselves popular rows that sit in L2, while the partial rows that replace them are read a few
-// dozen times each.  Measured gain of sharing, net of that launch, against the bytes it saves ((row gathers saved
-// - partial-row reads added) x bytes per gathered row): 845 MB -> 0 .. +50 us of 10.8 ms, 283 MB -> -4 us of
-// 1.4 ms, 128 MB -> -10 .. +6 us, 59 MB -> -5 .. +2.5 us, 4 MB -> -6 us; 1.9 GB on a graph with planted reuse
-// -> +310 us of 0.73 ms.  Plans that save less than the figure below are executed with every group folded back
-// into its consumers.
+// Sharing groups costs one more launch (~4-6 us on MI355X), and on heavy-tailed graphs what it saves is cheap:
+// the sources of a popular group are themselves popular rows that sit in L2, while the partial rows that
+// replace them are read a few dozen times each.  Measured gain of the destination-row launch against the net
+// saving (row gathers saved - partial-row reads added), as a fraction of all gathers and in bytes:
+//   R-MAT, upstream plans: 1.1 % / 128 MB -> -0.7 .. +0.4 %;  2.4 % / 283 MB -> -1.5 %;  1.2 % / 845 MB -> 0.0 %
+//   R-MAT, hub-pattern plans: 3.3 % -> -0.9 %;  6.2 % -> -4.5 %
+//   planted reuse: 81 % / 1.9 GB -> +45 .. +100 %;  small graph, 4 MB -> -6 us of 18
+// A small saving is a saving on hub rows; only a plan that removes a sizeable part of all gathers is worth its
+// partial rows.  Plans below either figure are executed with every group folded back into its consumers.
 const int64_t kMinSavedBytes = 256000000;
+const int64_t kMinSavedShare = 10;   // net saving >= 1/10 of all gathers
 const int32_t kTileRows = 4096;      // short tasks are length-sorted inside tiles of this many rows
 
 bool ptr_ok(const int32_t *p, int64_t n, int64_t *total) {
@@ -90,34 +98,38 @@ struct TaskList {   // tasks in natural order, before sorting
     }
 };
 
-// Long tasks first (descending), then short tasks tile by tile, each tile descending.
-void order_tasks(const ivec &ptr, int64_t tile_rows, ivec &order, int32_t &n_wave) {
+// Long tasks first (descending), then short tasks tile by tile, each tile descending.  `groups`: short tasks
+// that share a wavefront.
+void order_tasks(const ivec &ptr, int64_t tile_rows, int32_t groups, ivec &order, int32_t &n_wave) {
     int64_t T = (int64_t)ptr.size() - 1;
     order.clear();
     order.reserve(T);
+    int64_t over = 0;
+    for (int64_t t = 0; t < T; ++t) over += ptr[t + 1] - ptr[t] > kShortRow;
+    const int32_t cut = over + (T - over + groups - 1) / groups >= kWavesToFill ? kShortRow : kShortRowSmall;
     ivec longs;
     for (int64_t t = 0; t < T; ++t)
-        if (ptr[t + 1] - ptr[t] > kShortRow) longs.push_back((int32_t)t);
+        if (ptr[t + 1] - ptr[t] > cut) longs.push_back((int32_t)t);
     std::stable_sort(longs.begin(), longs.end(),
                      [&ptr](int32_t x, int32_t y) { return ptr[x + 1] - ptr[x] > ptr[y + 1] - ptr[y]; });
     n_wave = (int32_t)longs.size();
     order = longs;
-    std::vector<ivec> bucket(kShortRow + 1);
+    std::vector<ivec> bucket(cut + 1);
     for (int64_t t0 = 0; t0 < T; t0 += tile_rows) {
         int64_t t1 = std::min(T, t0 + tile_rows);
         for (auto &b : bucket) b.clear();
         for (int64_t t = t0; t < t1; ++t) {
             int32_t len = ptr[t + 1] - ptr[t];
-            if (len <= kShortRow) bucket[len].push_back((int32_t)t);
+            if (len <= cut) bucket[len].push_back((int32_t)t);
         }
-        for (int32_t len = kShortRow; len >= 0; --len) order.insert(order.end(), bucket[len].begin(), bucket[len].end());
+        for (int32_t len = cut; len >= 0; --len) order.insert(order.end(), bucket[len].begin(), bucket[len].end());
     }
 }
 
-void finalize_phase(const TaskList &tl, int64_t tile_rows, rof_phase_host &ph) {
+void finalize_phase(const TaskList &tl, int64_t tile_rows, int32_t groups, rof_phase_host &ph) {
     int64_t T = (int64_t)tl.out.size();
     ivec order;
-    order_tasks(tl.ptr, tile_rows, order, ph.n_wave);
+    order_tasks(tl.ptr, tile_rows, groups, order, ph.n_wave);
     ph.n_tasks = (int32_t)T;
     ph.task_ptr.assign(T + 1, 0);
     ph.task_nref.resize(T);
@@ -181,7 +193,8 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
         int64_t cnt = L->group_dst_ptr[g + 1] - L->group_dst_ptr[g], len = L->group_ptr[g + 1] - L->group_ptr[g];
         if (worth(cnt, len)) saved += (cnt - 1) * len - cnt;
     }
-    const bool too_small = min_consumers == 0 && saved * lpr * 16 < kMinSavedBytes;   // a lane holds 16 bytes of a row
+    const bool too_small = min_consumers == 0 && (saved * lpr * 16 < kMinSavedBytes ||   // a lane holds 16 bytes of a row
+                                                  saved * kMinSavedShare < total);
     std::vector<int32_t> slot_of(G, -1);
     int64_t slots = 0;
     TaskList tg, ts, tb;
@@ -256,9 +269,9 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     L->n_segments = segments;
     L->gathered_rows = gathered;
     L->partial_reads = reads;
-    finalize_phase(tg, 1 << 30, L->g);
-    finalize_phase(ts, 1 << 30, L->s);
-    finalize_phase(tb, tile_rows, L->b);
+    finalize_phase(tg, 1 << 30, groups, L->g);
+    finalize_phase(ts, 1 << 30, groups, L->s);
+    finalize_phase(tb, tile_rows, groups, L->b);
     L->gathered_before_rows = (int64_t)tg.col.size();
     for (size_t t = 0; t < ts.out.size(); ++t) L->gathered_before_rows += (ts.ptr[t + 1] - ts.ptr[t]) - ts.nref[t];
     return ROF_OK;

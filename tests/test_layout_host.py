@@ -130,9 +130,14 @@ def test_long_tasks_come_first_and_short_tasks_are_sorted_inside_tiles():
     ex, st = lay.export(), lay.stats()
     lens = np.diff(ex["b_task_ptr"])
     nw = st["wave_tasks_b"]
-    assert (lens[:nw] > 32).all() and (lens[nw:] <= 32).all() and (np.diff(lens[:nw]) <= 0).all()
+    assert (lens[:nw] > 32).all() and (lens[nw:] <= 32).all() and (np.diff(lens[:nw]) <= 0).all()   # small launch: cut 32
     assert sorted(ex["b_task_out"].tolist()) == list(range(n))
     assert lens.max() <= 2048                                # longer rows were segmented
+    ip, ix = make_workload("c4", 2)                          # 600 000 rows fill the machine: cut 64
+    lay = Layout.from_csr(ip, ix, lanes_per_row=12)
+    ex, st = lay.export(), lay.stats()
+    lens, nw = np.diff(ex["b_task_ptr"]), st["wave_tasks_b"]
+    assert (lens[:nw] > 64).all() and (lens[nw:] <= 64).all() and lens[nw:].max() > 32
 
 
 def test_non_canonical_v2_input_is_still_executed_correctly(oracle):
