@@ -280,7 +280,15 @@ class ROF_GCNLayerFunc(torch.autograd.Function):
         saved, weight, out = ctx.saved_tensors
         g = grad_output.contiguous()
         if ctx.relu:
-            g = g * (out > 0)
+            f = g.shape[1]
+            if not ctx.bf16 and f % 4:
+                # the masked gradient is a new tensor anyway: give it 16-byte rows, which the backward
+                # aggregation gathers ~12 % faster than packed ones
+                masked = g.new_empty((g.shape[0], f + (-f) % 4))[:, :f]
+                torch.mul(g, out > 0, out=masked)
+                g = masked
+            else:
+                g = g * (out > 0)
         d_bias = column_sums(g) if ctx.has_bias and ctx.needs_input_grad[2] else None
         d_x = d_w = None
         half = torch.bfloat16
