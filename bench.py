@@ -30,7 +30,7 @@ HBM_PEAK_GBS = 8000.0
 # factors coming from a 1 GiB copy of known size).  Counters cannot be
 # read from inside this script, so the figure is carried here and reported only for the configuration it was
 # measured on: (workload, part size, width) with default layout options.
-PROFILED_TRAFFIC_BYTES = {("c4", 3, 47): 8.85e9}
+PROFILED_TRAFFIC_BYTES = {("c4", 3, 47): 8.85e9, ("c5", 3, 256): 48.1e9}
 
 DESCR = {
     "c1": "c1: R-MAT 2^14 nodes, avg deg 16, self loops, GCN sym-norm, F=32, fp32",
@@ -563,6 +563,20 @@ def main():
             result["cpu_baseline"]["torch_sparse_mm_GEdges_per_s"] = e / float(np.median(ts)) / 1e9
         except Exception as ex:  # the library leg is informative only
             result["cpu_baseline"]["torch_sparse_mm_error"] = str(ex)[:200]
+        try:   # one thread of scipy's CSR x dense, as a sanity line
+            import scipy.sparse as sp
+
+            rs = O.rsqrt_rn(np.diff(indptr).astype(np.float32))
+            rs[~np.isfinite(rs)] = 0.0
+            data = (rs[np.repeat(np.arange(n), np.diff(indptr))] * rs[indices]).astype(np.float32) if normalized \
+                else np.ones(e, dtype=np.float32)
+            a = sp.csr_matrix((data, indices, indptr), shape=(n, n))
+            xs = np.ascontiguousarray(x32)
+            t0 = time.time()
+            a @ xs
+            result["cpu_baseline"]["scipy_1_thread_GEdges_per_s"] = e / (time.time() - t0) / 1e9
+        except Exception as ex:
+            result["cpu_baseline"]["scipy_error"] = str(ex)[:200]
 
     print(json.dumps(result))
 
