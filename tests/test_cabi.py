@@ -49,6 +49,17 @@ def test_error_codes_and_messages():
     assert L.rof_aggregate(None, None, 0, 0, None, 0, 1, 1, None, 0, None) == -1
     assert L.rof_layout_workspace_bytes(None, 4) == 0
     assert L.rof_set_xcd_run(0, 1) == -1
+    assert L.rof_set_xcd_run(1, 0) == 0                      # 0 for the destination-row launch: per-layout choice
+    ep = _lib.Epilogue(None, 1, 0, 0.5)
+    assert L.rof_aggregate_epilogue(None, None, 0, 0, None, 0, 1, 1, C.byref(ep), None, 0, None) == -1
+    assert L.rof_column_sums(None, 0, 4, 10, 4, None, None, 0, None) == -1          # no output
+    out = (C.c_float * 4)()
+    assert L.rof_column_sums(None, 0, 4, 10, 4, out, None, 0, None) == -1            # rows but no matrix
+    assert L.rof_column_sums(out, 7, 4, 1, 4, out, out, 1 << 20, None) == -6         # unknown element type
+    assert L.rof_column_sums(out, 0, 4, 1, 4, out, out, 16, None) == -7              # workspace too small
+    assert L.rof_column_sums_workspace_bytes(1000, 47) == 2048 * 47 * 4 and L.rof_column_sums_workspace_bytes(0, 47) == 0
+    assert L.rof_plan_hub_patterns(None, None, 0, 0, 16, 8, C.byref(h)) == -1
+    assert C.sizeof(_lib.Epilogue) == 32 and C.sizeof(_lib.LayoutOpts) == 32         # the structs of include/rof.h
     with pytest.raises(_lib.RofError, match="invalid argument"):
         _lib.check(-1)
 
