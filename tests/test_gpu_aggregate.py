@@ -286,3 +286,37 @@ def test_own_row_term_of_the_epilogue(oracle, feat, bf16):
     ref = oracle.closed_form(indptr, indices, x.float().cpu().numpy(), normalized=False) + 1.25 * x.double().cpu().numpy()
     mag = oracle.closed_form(indptr, indices, np.abs(x.float().cpu().numpy()), normalized=False) + 1.25 * np.abs(x.float().cpu().numpy())
     _close(got.cpu().numpy(), np.maximum(ref, 0), mag)
+
+
+def test_aggregation_is_capturable_in_a_hip_graph(oracle):
+    """rof_aggregate_epilogue only enqueues kernels (no allocation, no synchronisation, no memset), so a layer's
+    aggregation can be captured once and replayed: three replays on fresh inputs, with eager work between them,
+    each equal to the eager result bit for bit."""
+    indptr, indices, plan = _case("c1", 1, 3)
+    n = len(indptr) - 1
+    feat = 32
+    lay = _layout(plan, n, 3, min_consumers=2)               # three launches: groups, segments, rows
+    lay.set_degrees(torch.from_numpy(np.diff(indptr).astype(np.float32)).cuda())
+    bias = torch.from_numpy(features(1, feat, seed=30)[0]).cuda()
+    x = torch.zeros((n, feat), device="cuda")
+    out = torch.empty((n, feat), device="cuda")
+    lay.aggregate(x, normalized=True, out=out, bias=bias, relu=True)          # uploads, sizes the workspace
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        lay.aggregate(x, normalized=True, out=out, bias=bias, relu=True)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        lay.aggregate(x, normalized=True, out=out, bias=bias, relu=True)
+    for trial in range(3):
+        fresh = torch.from_numpy(features(n, feat, seed=31 + trial)).cuda()
+        eager = lay.aggregate(fresh, normalized=True, bias=bias, relu=True).clone()   # eager work between replays
+        torch.cuda.synchronize()
+        x.copy_(fresh)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), trial
+    want = np.maximum(oracle.closed_form(indptr, indices, fresh.cpu().numpy(), np.diff(indptr).astype(np.float32))
+                      + bias.cpu().numpy(), 0)
+    assert np.allclose(out.cpu().numpy(), want, rtol=1e-5, atol=1e-5)
