@@ -134,7 +134,9 @@ __device__ __forceinline__ const char *row_ptr(int32_t c, const char *xb, uint32
         l = p ? pld : xld;
         b = p ? pb : xb;
     }
-    if (OFF32) return b + __umul24(r, l);
+    // HIP declares __umul24 as returning int: without the cast a byte offset of 2^31 or more would be
+    // sign-extended into a negative one
+    if (OFF32) return b + (uint32_t)__umul24(r, l);
     return b + (uint64_t)r * l;
 }
 

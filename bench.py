@@ -211,7 +211,8 @@ def main():
     ap.add_argument("--feat", type=int, default=0, help="override the aggregated width")
     ap.add_argument("--cache-dir", default="/tmp/rof_bench_cache")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--xcd-run", type=int, default=0)
+    ap.add_argument("--xcd-run", type=int, default=0, help="launch tuning: workgroups per XCD run, destination rows")
+    ap.add_argument("--xcd-run-partial", type=int, default=1, help="same for the partial-sum launches")
     ap.add_argument("--hub-split", type=int, default=0, help="layout tuning: rows longer than this are segmented")
     ap.add_argument("--segment", type=int, default=0, help="layout tuning: entries per segment")
     ap.add_argument("--min-consumers", type=int, default=0, help="layout tuning: share groups with >= this many consumers")
@@ -241,8 +242,8 @@ def main():
     L = _lib.lib()   # raises if the HIP library is missing
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
-    if args.xcd_run:
-        _lib.check(L.rof_set_xcd_run(1, args.xcd_run))
+    if args.xcd_run or args.xcd_run_partial != 1:
+        _lib.check(L.rof_set_xcd_run(args.xcd_run_partial, args.xcd_run))
     if args.lds_pad >= 0:
         _lib.check(L.rof_set_lds_pad(args.lds_pad))
     dev = torch.device("cuda:0")

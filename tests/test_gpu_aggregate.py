@@ -320,3 +320,37 @@ def test_aggregation_is_capturable_in_a_hip_graph(oracle):
     want = np.maximum(oracle.closed_form(indptr, indices, fresh.cpu().numpy(), np.diff(indptr).astype(np.float32))
                       + bias.cpu().numpy(), 0)
     assert np.allclose(out.cpu().numpy(), want, rtol=1e-5, atol=1e-5)
+
+
+def test_byte_offsets_between_2_and_4_gib():
+    """Regression: with the short address arithmetic (row id x row bytes in 32 bits) a feature matrix or a
+    partial-sum workspace between 2 GiB and 4 GiB puts byte offsets above 2^31, which must be taken as unsigned.
+    (1) 3 M rows of 192 floats (2.3 GB), gathered from the top of the matrix; (2) 2.56 M partial rows of 256
+    floats (2.6 GB): every entry of every row its own segment."""
+    dev = "cuda"
+    rng = np.random.default_rng(12)
+    # (1) the feature matrix
+    n, feat = 3_000_000, 192
+    dst = np.sort(rng.choice(n, 2000, replace=False))
+    nbr = np.sort(rng.integers(n - n // 10, n, (2000, 8)), axis=1)
+    deg = np.zeros(n, np.int64)
+    deg[dst] = 8
+    ip = np.r_[0, np.cumsum(deg)].astype(np.int32)
+    x = torch.randn((n, feat), device=dev)
+    got = Layout.from_csr(ip, nbr.ravel().astype(np.int32)).aggregate(x, normalized=False)
+    want = x[torch.from_numpy(nbr.ravel()).to(dev)].double().view(2000, 8, feat).sum(1)
+    assert torch.allclose(got[torch.from_numpy(dst).to(dev)].double(), want, rtol=1e-6, atol=1e-6)
+    assert float(got.abs().sum(1)[torch.from_numpy(np.setdiff1d(np.arange(0, n, 997), dst)).to(dev)].max()) == 0.0
+    del x, got, want
+    # (2) the partial-sum workspace
+    n, rows, per, feat = 100_000, 40_000, 64, 256
+    nbr = np.sort(rng.integers(0, n, (rows, per)), axis=1)
+    deg = np.zeros(n, np.int64)
+    deg[:rows] = per
+    ip = np.r_[0, np.cumsum(deg)].astype(np.int32)
+    lay = Layout.from_csr(ip, nbr.ravel().astype(np.int32), hub_split=32, segment=1, lanes_per_row=64)
+    assert lay.stats()["hub_segments"] == rows * per and lay.workspace_bytes(feat) > 2 ** 31
+    x = torch.randn((n, feat), device=dev)
+    got = lay.aggregate(x, normalized=False)
+    want = x[torch.from_numpy(nbr.ravel()).to(dev)].double().view(rows, per, feat).sum(1)
+    assert torch.allclose(got[:rows].double(), want, rtol=1e-5, atol=1e-5)
