@@ -31,17 +31,19 @@ typedef std::vector<int32_t> ivec;
 // by its longest task instead and keeps the lower cut (16 384 rows: 18 us against 26).
 const int32_t kShortRow = 64, kShortRowSmall = 32;
 const int64_t kWavesToFill = 2 * 8192;   // two rounds of 256 CUs x 32 wavefronts
-// Default cut for long rows.  A wavefront works through a task G entries at a time (G = 64 / lanes per
-// row) with two gathers in flight, so a task of L entries is a serial chain of L / (2G) memory round
-// trips; the longest chain has to stay well below the duration of the launch, which grows with the number
-// of entries and with the row size (~1/G).  Measured optima on MI355X: 1024 entries at 3.6 M entries with
-// G = 1, 5000-6000 at 60 M with G = 5, 8192 at 132 M with G = 2; beyond 8192 the tail always loses.
-// Cutting finer than needed costs too: every segment writes and re-reads one partial row (bigger for
-// small G), and the launch that runs the segments has few tasks, so segments are a quarter of the cut.
-// (Giving rows between one and four cuts a whole workgroup instead -- four wavefronts combined through
-// LDS -- was measured as well: no faster than segments on any workload, so it is not built in.)
-const int64_t kEntriesPerSplitUnit = 11000;   // hub_split ~ entries / this
-const int32_t kHubSplitMax = 8192;
+// Long rows.  Rows longer than a cut are gathered in segments that fill partial rows one launch earlier, and
+// the segment tasks of all rows run in the order of the highest source id they gather (entries inside a task are
+// listed by descending id): every wavefront in flight then works in the same narrow band of the feature matrix
+// and the launch sweeps the matrix once from top to bottom, so a row gathered for one destination is still in
+// L2 when the next destinations need it.  The effect is large -- rotating each row's list by a random offset,
+// which keeps every task monotone but puts the tasks out of phase, costs 25 % on the 2.4 M-node workload -- and
+// it is why the cut is low: measured optima with G rows per wavefront are cut / segment = 96-128 / 32 at G = 1
+// (-12 % against a cut of 1024), 256 / 64 at G = 2 (-18 % against 8192), 640-1024 / 160 at G = 5 (-7 % against
+// 5457), i.e. 128 G / 32 G.  Every segment writes and re-reads one partial row, which is what stops finer cuts.
+// (Giving long rows a whole workgroup instead -- four wavefronts combined through LDS -- was measured as well:
+// no faster than segments on any workload, so it is not built in.)
+// Beyond G = 5 nothing larger was measured to pay (16 384 rows at G = 8: 512 / 128 runs 18 us, 1024 / 256 20 us).
+const int32_t kCutPerGroup = 128, kCutMax = 640;
 // Sharing groups costs one more launch (~4-6 us on MI355X), and on heavy-tailed graphs what it saves is cheap:
 // the sources of a popular group are themselves popular rows that sit in L2, while the partial rows that
 // replace them are read a few dozen times each.  Measured gain of the destination-row launch against the net
@@ -99,8 +101,9 @@ struct TaskList {   // tasks in natural order, before sorting
 };
 
 // Long tasks first (descending), then short tasks tile by tile, each tile descending.  `groups`: short tasks
-// that share a wavefront.
-void order_tasks(const ivec &ptr, int64_t tile_rows, int32_t groups, ivec &order, int32_t &n_wave) {
+// that share a wavefront.  With `band` (one key per task: the highest source id it gathers) both kinds are
+// ordered by descending key instead.
+void order_tasks(const ivec &ptr, int64_t tile_rows, int32_t groups, const ivec *band, ivec &order, int32_t &n_wave) {
     int64_t T = (int64_t)ptr.size() - 1;
     order.clear();
     order.reserve(T);
@@ -110,6 +113,18 @@ void order_tasks(const ivec &ptr, int64_t tile_rows, int32_t groups, ivec &order
     ivec longs;
     for (int64_t t = 0; t < T; ++t)
         if (ptr[t + 1] - ptr[t] > cut) longs.push_back((int32_t)t);
+    if (band && cut == kShortRow) {   // a launch too small to fill the machine keeps the longest-first order
+        ivec shorts;
+        for (int64_t t = 0; t < T; ++t)
+            if (ptr[t + 1] - ptr[t] <= cut) shorts.push_back((int32_t)t);
+        auto higher = [band](int32_t x, int32_t y) { return (*band)[x] > (*band)[y]; };
+        std::stable_sort(longs.begin(), longs.end(), higher);
+        std::stable_sort(shorts.begin(), shorts.end(), higher);
+        n_wave = (int32_t)longs.size();
+        order = longs;
+        order.insert(order.end(), shorts.begin(), shorts.end());
+        return;
+    }
     std::stable_sort(longs.begin(), longs.end(),
                      [&ptr](int32_t x, int32_t y) { return ptr[x + 1] - ptr[x] > ptr[y + 1] - ptr[y]; });
     n_wave = (int32_t)longs.size();
@@ -126,10 +141,17 @@ void order_tasks(const ivec &ptr, int64_t tile_rows, int32_t groups, ivec &order
     }
 }
 
-void finalize_phase(const TaskList &tl, int64_t tile_rows, int32_t groups, rof_phase_host &ph) {
+void finalize_phase(const TaskList &tl, int64_t tile_rows, int32_t groups, bool by_band, rof_phase_host &ph) {
     int64_t T = (int64_t)tl.out.size();
-    ivec order;
-    order_tasks(tl.ptr, tile_rows, groups, order, ph.n_wave);
+    ivec order, band;
+    if (by_band) {
+        band.resize(T);
+        for (int64_t t = 0; t < T; ++t) {
+            const int32_t first = tl.ptr[t] + tl.nref[t];   // feature rows follow the partial-row references
+            band[t] = first < tl.ptr[t + 1] ? tl.col[first] : -1;
+        }
+    }
+    order_tasks(tl.ptr, tile_rows, groups, by_band ? &band : nullptr, order, ph.n_wave);
     ph.n_tasks = (int32_t)T;
     ph.task_ptr.assign(T + 1, 0);
     ph.task_nref.resize(T);
@@ -156,9 +178,7 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     if (lpr > 64) lpr = 64;
     const int32_t groups = std::max(1, 64 / lpr);
     const int64_t total = (int64_t)L->res_col.size() + (int64_t)L->group_dst.size();
-    const int64_t floor_split = std::max<int64_t>(64 * groups, 1024 / groups);
-    const int64_t auto_split = std::max<int64_t>(floor_split, std::min<int64_t>(kHubSplitMax, total / kEntriesPerSplitUnit));
-    const int32_t hub_split = (o && o->hub_split > 0) ? o->hub_split : (int32_t)auto_split;
+    const int32_t hub_split = (o && o->hub_split > 0) ? o->hub_split : std::min(kCutMax, kCutPerGroup * groups);
     const int32_t segment = (o && o->segment > 0) ? o->segment : std::max(16, hub_split / 4);
     L->hub_split = hub_split;
     L->segment = segment;
@@ -269,9 +289,9 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     L->n_segments = segments;
     L->gathered_rows = gathered;
     L->partial_reads = reads;
-    finalize_phase(tg, 1 << 30, groups, L->g);
-    finalize_phase(ts, 1 << 30, groups, L->s);
-    finalize_phase(tb, tile_rows, groups, L->b);
+    finalize_phase(tg, 1 << 30, groups, false, L->g);
+    finalize_phase(ts, 1 << 30, groups, entry_order == 0, L->s);   // the sweep needs the descending lists
+    finalize_phase(tb, tile_rows, groups, false, L->b);
     L->gathered_before_rows = (int64_t)tg.col.size();
     for (size_t t = 0; t < ts.out.size(); ++t) L->gathered_before_rows += (ts.ptr[t + 1] - ts.ptr[t]) - ts.nref[t];
     return ROF_OK;

@@ -114,12 +114,12 @@ typedef struct rof_layout rof_layout;
 typedef struct {
     int32_t min_consumers;   /* a group is materialised iff it has >= this many consumers; 0 = cost model; -1 = all */
     int32_t disable_reuse;   /* 1: expand every group back into its consumers' rows (the comparator)      */
-    int32_t hub_split;       /* rows with more entries than this are cut into segments; 0 = choose from    */
-                             /* lanes_per_row and the plan size                                            */
-    int32_t segment;         /* entries per segment; 0 = hub_split / 4                                     */
+    int32_t hub_split;       /* rows with more entries than this are gathered in segments one launch earlier;  */
+                             /* 0 = 128 x the rows a wavefront gathers at once (64 / lanes_per_row), at most 640 */
+    int32_t segment;         /* entries per segment; 0 = a quarter of hub_split                                */
     int32_t lanes_per_row;   /* lanes one gathered row occupies in the kernel that will use this layout:   */
                              /* smallest of 4,8,10,12,16,20,32,64 >= ceil(feat_dim / 4) (fp32) or / 8      */
-                             /* (bf16); 0 = 16.  Only steers the default hub_split.                         */
+                             /* (bf16); 0 = 16.  Steers the default hub_split and the sharing gate.        */
     int32_t entry_order;     /* feature rows inside one task are gathered 0: by source id, descending      */
                              /* (default; measured 2-3 % faster than plan order and 20 % faster than a      */
                              /* random order on MI355X), 1: in the order the plan lists them, 2: ascending   */
