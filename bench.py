@@ -26,11 +26,11 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 
-# HBM-side bytes per destination-row launch measured offline with rocprofv3 (FETCH_SIZE x 2.0 + WRITE_SIZE, the
-# factors coming from a 1 GiB copy of known size).  Counters cannot be
-# read from inside this script, so the figure is carried here and reported only for the configuration it was
+# HBM-side bytes per launch (partial-sum launch, destination-row launch) measured offline with rocprofv3
+# (FETCH_SIZE x 2.0 + WRITE_SIZE, the factors coming from a 1 GiB copy of known size).  Counters cannot be read
+# from inside this script, so the figures are carried here and reported only for the configurations they were
 # measured on: (workload, part size, width) with default layout options.
-PROFILED_TRAFFIC_BYTES = {("c4", 3, 47): 8.85e9, ("c5", 3, 256): 48.1e9}
+PROFILED_TRAFFIC_BYTES = {("c4", 3, 47): (1.75e9, 6.53e9), ("c5", 3, 256): (24.94e9, 23.56e9)}
 
 DESCR = {
     "c1": "c1: R-MAT 2^14 nodes, avg deg 16, self loops, GCN sym-norm, F=32, fp32",
@@ -490,7 +490,8 @@ def main():
     achieved_b = bytes_b / (ms_b * 1e-3) / 1e9
     default_opts = (not (args.hub_split or args.segment or args.min_consumers or args.fold_sources)
                     and args.search == "upstream" and args.entry_order == "descending" and not args.tile_rows)
-    traffic = PROFILED_TRAFFIC_BYTES.get((name, ps, feat)) if default_opts else None
+    traffic = PROFILED_TRAFFIC_BYTES.get((name, ps, feat), (None, None)) if default_opts else (None, None)
+    achieved_a = bytes_a / (ms_a * 1e-3) / 1e9 if ms_a > 0 else 0.0
 
     result = {
         "metric": "GEdges/s per aggregation layer (reuse plan), 1 MI355X",
@@ -510,7 +511,14 @@ def main():
         "roofline": {
             "bound": "hbm", "kernel": "rof_rows_kernel (destination-row launch)",
             "achieved": achieved_b, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved_b / HBM_PEAK_GBS,
-            "traffic": traffic, "bytes_per_launch": bytes_b, "ms_per_launch": ms_b,
+            "traffic": traffic[1], "bytes_per_launch": bytes_b, "ms_per_launch": ms_b,
+        },
+        # the launch before it (segments of long rows, swept in the order of their source ids): same kernel
+        # template, second in duration
+        "roofline_partial_launch": {
+            "bound": "hbm", "kernel": "rof_rows_kernel (partial-sum launch)",
+            "achieved": achieved_a, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved_a / HBM_PEAK_GBS,
+            "traffic": traffic[0], "bytes_per_launch": bytes_a, "ms_per_launch": ms_a,
         },
         "layer": {
             "event_ms": ev_ms, "event_ms_runs": ev_r, "per_call": spread, "launch1_ms": ms_a, "launch2_ms": ms_b,
