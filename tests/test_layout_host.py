@@ -114,6 +114,34 @@ def test_sharing_is_gated_by_the_bytes_it_saves():
     assert forced["materialised_groups"] == len(cnt)
 
 
+@pytest.mark.parametrize("lanes,cut,seg", [(64, 128, 32), (32, 256, 64), (12, 640, 160), (8, 640, 160)])
+def test_long_rows_are_cut_by_width_and_their_segments_swept_by_source_id(lanes, cut, seg):
+    """Default cut = 128 x rows per wavefront (at most 640), segments a quarter of it; the segment tasks come in
+    the order of the highest source id they gather (each task lists its sources by descending id), long tasks
+    before packed ones."""
+    ip, ix = make_workload("c4", 2)                          # 600 000 rows: enough segments to fill the machine
+    n = len(ip) - 1
+    lay = Layout.from_csr(ip, ix, lanes_per_row=lanes)
+    ex, st = lay.export(), lay.stats()
+    deg = np.diff(ip)
+    assert st["hub_segments"] == int(np.ceil(deg[deg > cut] / seg).sum())
+    b_len, b_ref = np.diff(ex["b_task_ptr"]), ex["b_task_nref"]
+    assert b_len[b_ref == 0].max() <= cut and (b_len[b_ref > 0] == b_ref[b_ref > 0]).all()
+    s_ptr, s_col = ex["s_task_ptr"], ex["s_col"]
+    s_len = np.diff(s_ptr)
+    assert s_len.max() == seg and (ex["s_task_nref"] == 0).all()
+    for t in range(0, len(s_len), 997):                      # sources inside a task: descending
+        assert (np.diff(s_col[s_ptr[t]:s_ptr[t + 1]]) < 0).all()
+    first = s_col[s_ptr[:-1]]
+    nw = st["wave_tasks_a"]
+    assert (np.diff(first[:nw]) <= 0).all() and (np.diff(first[nw:]) <= 0).all()
+    assert nw == int((s_len > 64).sum()) and (s_len[:nw] > 64).all()
+    # with the plan's own order inside tasks there is no sweep: segments come longest first
+    ex2 = Layout.from_csr(ip, ix, lanes_per_row=lanes, entry_order="plan").export()
+    first2 = ex2["s_col"][ex2["s_task_ptr"][:-1]]
+    assert not (np.diff(first2[:nw]) <= 0).all() or nw < 2 or not (np.diff(first2[nw:]) <= 0).all()
+
+
 def test_xcd_run_follows_the_locality_of_the_graph():
     """Block-structured graphs (rows gather from their own neighbourhood) keep long runs of workgroups on one
     XCD; graphs without that locality use short runs."""
