@@ -266,8 +266,13 @@ __global__ __launch_bounds__(256, ROF_MIN_BLOCKS) void rof_rows_kernel(AggArgs a
         constexpr bool kF32 = sizeof(XT) == 4;   // fp32 features: partial rows have the same element type
         if (wave_mode) {
             if (kF32) {
-                gather_sum<XT, VEC, LPR, true, true, OFF32>(xb, xld, pb, pld, a.nsplit, 0, a.col, a.w, beg, end, lane,
-                                                            sub, li, act, acc);
+                // only tasks that reference partial rows pay for the select between the two matrices
+                if (mid > beg)
+                    gather_sum<XT, VEC, LPR, true, true, OFF32>(xb, xld, pb, pld, a.nsplit, 0, a.col, a.w, beg, end,
+                                                                lane, sub, li, act, acc);
+                else
+                    gather_sum<XT, VEC, LPR, true, false, OFF32>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, beg, end, lane,
+                                                                 sub, li, act, acc);
             } else {
                 if (mid > beg)
                     gather_sum<float, VEC, LPR, true, false, OFF32>(pb, pld, nullptr, 0, 0, a.nsplit, a.col, a.w, beg,
@@ -292,8 +297,12 @@ __global__ __launch_bounds__(256, ROF_MIN_BLOCKS) void rof_rows_kernel(AggArgs a
             }
         } else {
             if (kF32) {
-                gather_sum<XT, VEC, LPR, false, true, OFF32>(xb, xld, pb, pld, a.nsplit, 0, a.col, a.w, beg, end, lane,
-                                                             sub, li, act, acc);
+                if (__any(mid > beg))
+                    gather_sum<XT, VEC, LPR, false, true, OFF32>(xb, xld, pb, pld, a.nsplit, 0, a.col, a.w, beg, end,
+                                                                 lane, sub, li, act, acc);
+                else
+                    gather_sum<XT, VEC, LPR, false, false, OFF32>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, beg, end, lane,
+                                                                  sub, li, act, acc);
             } else {
                 if (__any(mid > beg))
                     gather_sum<float, VEC, LPR, false, false, OFF32>(pb, pld, nullptr, 0, 0, a.nsplit, a.col, a.w, beg,
