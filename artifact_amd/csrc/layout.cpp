@@ -39,11 +39,15 @@ const int64_t kWavesToFill = 2 * 8192;   // two rounds of 256 CUs x 32 wavefront
 // which keeps every task monotone but puts the tasks out of phase, costs 25 % on the 2.4 M-node workload -- and
 // it is why the cut is low: measured optima with G rows per wavefront are cut / segment = 96-128 / 32 at G = 1
 // (-12 % against a cut of 1024), 256 / 64 at G = 2 (-18 % against 8192), 640-1024 / 160 at G = 5 (-7 % against
-// 5457), i.e. 128 G / 32 G.  Every segment writes and re-reads one partial row, which is what stops finer cuts.
+// 5457).  Every segment writes and re-reads one partial row (fp32, so twice a gathered row when those are bf16),
+// which is what stops finer cuts: at G = 2 the best cut is 128 / 32 for fp32 rows (-10 % against 256 / 64) and
+// 256 / 64 for bf16 rows; at G = 4 256-512; at G = 8 and 16 640-1024 (256 is 10-30 % slower there).
 // (Giving long rows a whole workgroup instead -- four wavefronts combined through LDS -- was measured as well:
 // no faster than segments on any workload, so it is not built in.)
-// Beyond G = 5 nothing larger was measured to pay (16 384 rows at G = 8: 512 / 128 runs 18 us, 1024 / 256 20 us).
-const int32_t kCutPerGroup = 128, kCutMax = 640;
+int32_t default_cut(int32_t groups, int32_t elem_bytes) {
+    const int32_t cut = groups <= 2 ? 128 : groups == 3 ? 256 : groups == 4 ? 384 : 640;
+    return std::min(640, elem_bytes == 2 ? 2 * cut : cut);
+}
 // Sharing groups costs one more launch (~4-6 us on MI355X), and on heavy-tailed graphs what it saves is cheap:
 // the sources of a popular group are themselves popular rows that sit in L2, while the partial rows that
 // replace them are read a few dozen times each.  Measured gain of the destination-row launch against the net
@@ -178,7 +182,7 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     if (lpr > 64) lpr = 64;
     const int32_t groups = std::max(1, 64 / lpr);
     const int64_t total = (int64_t)L->res_col.size() + (int64_t)L->group_dst.size();
-    const int32_t hub_split = (o && o->hub_split > 0) ? o->hub_split : std::min(kCutMax, kCutPerGroup * groups);
+    const int32_t hub_split = (o && o->hub_split > 0) ? o->hub_split : default_cut(groups, o ? o->elem_bytes : 4);
     const int32_t segment = (o && o->segment > 0) ? o->segment : std::max(16, hub_split / 4);
     L->hub_split = hub_split;
     L->segment = segment;

@@ -60,7 +60,7 @@ ENTRY_ORDERS = {"descending": 0, "plan": 1, "ascending": 2}
 
 
 def _opts(min_consumers=0, disable_reuse=False, hub_split=0, segment=0, lanes_per_row=0, entry_order="descending",
-          tile_rows=0):
+          tile_rows=0, elem_bytes=0):
     o = LayoutOpts()
     o.min_consumers = int(min_consumers)
     o.disable_reuse = int(bool(disable_reuse))
@@ -69,22 +69,30 @@ def _opts(min_consumers=0, disable_reuse=False, hub_split=0, segment=0, lanes_pe
     o.lanes_per_row = int(lanes_per_row)
     o.entry_order = ENTRY_ORDERS[entry_order]
     o.tile_rows = int(tile_rows)
+    o.elem_bytes = int(elem_bytes)
     return o
 
 
 class LayoutFamily:
-    """Layouts of one plan, one per lanes-per-row class: how finely long rows are segmented depends on
-    how many rows a wavefront gathers at once, i.e. on the feature width it will be used with."""
+    """Layouts of one plan, one per width class (lanes per row, element size): how finely long rows are cut
+    depends on how many rows a wavefront gathers at once and on how wide a partial-sum row is against a gathered
+    one, i.e. on the feature width and type the layout will be used with."""
 
     def __init__(self, build):
-        self._build = build            # callable(lanes_per_row) -> Layout
+        self._build = build            # callable(lanes_per_row[, elem_bytes]) -> Layout
         self._by_lpr = {}
+        try:
+            import inspect
+
+            self._two = len(inspect.signature(build).parameters) >= 2
+        except (TypeError, ValueError):
+            self._two = False
 
     def get(self, feat_dim, bf16=False):
-        lpr = lanes_per_row(feat_dim, bf16)
-        lay = self._by_lpr.get(lpr)
+        key = (lanes_per_row(feat_dim, bf16), 2 if bf16 else 4)
+        lay = self._by_lpr.get(key)
         if lay is None:
-            lay = self._by_lpr[lpr] = self._build(lpr)
+            lay = self._by_lpr[key] = self._build(*key) if self._two else self._build(key[0])
         return lay
 
     def close(self):

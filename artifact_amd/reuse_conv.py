@@ -82,8 +82,8 @@ class ROF_inputInfo:
             n, ps = len(z["row_pointers"]) - 1, int(z["partSize"])
             v2 = tuple(np.array(z[k]) for k in ("uniqpart_column_index", "uniqpart_pointers", "part2Node_ptr",
                                                  "part2Node_col"))
-            info.layouts["ROF_v2"] = LayoutFamily(lambda lpr: Layout.from_v2(*v2, n, ps, lanes_per_row=lpr,
-                                                                             **layout_opts))
+            info.layouts["ROF_v2"] = LayoutFamily(lambda lpr, eb: Layout.from_v2(
+                *v2, n, ps, lanes_per_row=lpr, elem_bytes=eb, **layout_opts))
         return info
 
     def __getstate__(self):
@@ -129,9 +129,9 @@ def build_input_info(indptr, indices, part_size=3, device="cuda", warps_per_bloc
                          t(plan["column_index_cache"]), t(plan["uniqpart_column_index"]), t(plan["uniqpart_pointers"]),
                          t(plan["part2Node_ptr"]), t(plan["part2Node_col"]))
     if torch.device(device).type == "cuda":
-        info.layouts["ROF_v2"] = LayoutFamily(lambda lpr: Layout.from_v2(
+        info.layouts["ROF_v2"] = LayoutFamily(lambda lpr, eb: Layout.from_v2(
             plan["uniqpart_column_index"], plan["uniqpart_pointers"], plan["part2Node_ptr"], plan["part2Node_col"], n,
-            part_size, lanes_per_row=lpr, **layout_opts))
+            part_size, lanes_per_row=lpr, elem_bytes=eb, **layout_opts))
     info.plan = plan
     return info
 

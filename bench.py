@@ -129,8 +129,9 @@ def model_step(name, d, n, ps, deg, dev, timed):
     from artifact_amd.layout import Layout, LayoutFamily
     from artifact_amd.reuse_conv import ROF_GCNConv, ROF_GINConv
 
-    fam = LayoutFamily(lambda lpr: Layout.from_v2(d["uniqpart_column_index"], d["uniqpart_pointers"],
-                                                  d["part2Node_ptr"], d["part2Node_col"], n, ps, lanes_per_row=lpr))
+    fam = LayoutFamily(lambda lpr, eb: Layout.from_v2(d["uniqpart_column_index"], d["uniqpart_pointers"],
+                                                      d["part2Node_ptr"], d["part2Node_col"], n, ps,
+                                                      lanes_per_row=lpr, elem_bytes=eb))
     dummy = torch.zeros(1, dtype=torch.int32, device=dev)   # the plan tensors are not read when a layout is attached
     info = types.SimpleNamespace(degrees=deg, layouts={"ROF_v2": fam}, partSize=ps, warpPerBlock=4,
                                  **{k: dummy for k in ("column_index", "part_pointers", "part2Node",
@@ -285,10 +286,10 @@ def main():
     t0 = time.time()
     reuse = Layout.from_v2(d["uniqpart_column_index"], d["uniqpart_pointers"], d["part2Node_ptr"], d["part2Node_col"],
                            n, ps, hub_split=args.hub_split, segment=args.segment, lanes_per_row=lpr,
-                           min_consumers=args.min_consumers, entry_order=args.entry_order, tile_rows=args.tile_rows)
+                           min_consumers=args.min_consumers, entry_order=args.entry_order, tile_rows=args.tile_rows, elem_bytes=in_bytes)
     plain = Layout.from_v2(d["uniqpart_column_index"], d["uniqpart_pointers"], d["part2Node_ptr"], d["part2Node_col"],
                            n, ps, disable_reuse=True, hub_split=args.hub_split, segment=args.segment, lanes_per_row=lpr,
-                           entry_order=args.entry_order, tile_rows=args.tile_rows)
+                           entry_order=args.entry_order, tile_rows=args.tile_rows, elem_bytes=in_bytes)
     t_layout = time.time() - t0
     # when the cost model folds every group back (the plan saves too little), also time the plan with its
     # profitable groups forced to be shared, so the cost of the reuse machinery stays visible
@@ -296,7 +297,7 @@ def main():
     if reuse.stats()["materialised_groups"] == 0 and len(d["index_picked"]) and not args.min_consumers:
         forced = Layout.from_v2(d["uniqpart_column_index"], d["uniqpart_pointers"], d["part2Node_ptr"],
                                 d["part2Node_col"], n, ps, hub_split=args.hub_split, segment=args.segment,
-                                lanes_per_row=lpr, min_consumers=3, entry_order=args.entry_order, tile_rows=args.tile_rows)
+                                lanes_per_row=lpr, min_consumers=3, entry_order=args.entry_order, tile_rows=args.tile_rows, elem_bytes=in_bytes)
     for lay in (reuse, plain) + ((forced,) if forced else ()):
         lay.upload()
         if normalized:

@@ -115,7 +115,8 @@ typedef struct {
     int32_t min_consumers;   /* a group is materialised iff it has >= this many consumers; 0 = cost model; -1 = all */
     int32_t disable_reuse;   /* 1: expand every group back into its consumers' rows (the comparator)      */
     int32_t hub_split;       /* rows with more entries than this are gathered in segments one launch earlier;  */
-                             /* 0 = 128 x the rows a wavefront gathers at once (64 / lanes_per_row), at most 640 */
+                             /* 0 = by the rows a wavefront gathers at once (G = 64 / lanes_per_row): 128 for   */
+                             /* G <= 2, 256 for 3, 384 for 4, 640 from 5 on; doubled for bfloat16 rows; <= 640  */
     int32_t segment;         /* entries per segment; 0 = a quarter of hub_split                                */
     int32_t lanes_per_row;   /* lanes one gathered row occupies in the kernel that will use this layout:   */
                              /* smallest of 4,8,10,12,16,20,32,64 >= ceil(feat_dim / 4) (fp32) or / 8      */
@@ -124,7 +125,9 @@ typedef struct {
                              /* (default; measured 2-3 % faster than plan order and 20 % faster than a      */
                              /* random order on MI355X), 1: in the order the plan lists them, 2: ascending   */
     int32_t tile_rows;       /* short rows are sorted by length inside tiles of this many destinations; 0 = 4096 */
-    int32_t reserved[1];
+    int32_t elem_bytes;      /* bytes per element of the rows that will be gathered: 4 (float32, also 0) or 2        */
+                             /* (bfloat16, whose partial-sum rows are twice as wide as its gathered rows).  Steers   */
+                             /* the default hub_split.                                                              */
 } rof_layout_opts;
 
 /* v2 tensors: replaces the plan arguments of reuse_forward_v2 / reuse_backward_v2

@@ -114,14 +114,16 @@ def test_sharing_is_gated_by_the_bytes_it_saves():
     assert forced["materialised_groups"] == len(cnt)
 
 
-@pytest.mark.parametrize("lanes,cut,seg", [(64, 128, 32), (32, 256, 64), (12, 640, 160), (8, 640, 160)])
-def test_long_rows_are_cut_by_width_and_their_segments_swept_by_source_id(lanes, cut, seg):
-    """Default cut = 128 x rows per wavefront (at most 640), segments a quarter of it; the segment tasks come in
-    the order of the highest source id they gather (each task lists its sources by descending id), long tasks
-    before packed ones."""
+@pytest.mark.parametrize("lanes,elem,cut,seg", [(64, 4, 128, 32), (32, 4, 128, 32), (32, 2, 256, 64), (16, 4, 384, 96),
+                                                (12, 4, 640, 160), (8, 0, 640, 160)])
+def test_long_rows_are_cut_by_width_and_their_segments_swept_by_source_id(lanes, elem, cut, seg):
+    """Default cut by the rows a wavefront gathers at once (128 up to two, 384 at four, 640 from five on; doubled
+    for bf16 rows, whose partial rows are twice as wide), segments a quarter of it; the segment tasks come in the
+    order of the highest source id they gather (each task lists its sources by descending id), long tasks before
+    packed ones."""
     ip, ix = make_workload("c4", 2)                          # 600 000 rows: enough segments to fill the machine
     n = len(ip) - 1
-    lay = Layout.from_csr(ip, ix, lanes_per_row=lanes)
+    lay = Layout.from_csr(ip, ix, lanes_per_row=lanes, elem_bytes=elem)
     ex, st = lay.export(), lay.stats()
     deg = np.diff(ip)
     assert st["hub_segments"] == int(np.ceil(deg[deg > cut] / seg).sum())
@@ -137,7 +139,7 @@ def test_long_rows_are_cut_by_width_and_their_segments_swept_by_source_id(lanes,
     assert (np.diff(first[:nw]) <= 0).all() and (np.diff(first[nw:]) <= 0).all()
     assert nw == int((s_len > 64).sum()) and (s_len[:nw] > 64).all()
     # with the plan's own order inside tasks there is no sweep: segments come longest first
-    ex2 = Layout.from_csr(ip, ix, lanes_per_row=lanes, entry_order="plan").export()
+    ex2 = Layout.from_csr(ip, ix, lanes_per_row=lanes, elem_bytes=elem, entry_order="plan").export()
     first2 = ex2["s_col"][ex2["s_task_ptr"][:-1]]
     assert not (np.diff(first2[:nw]) <= 0).all() or nw < 2 or not (np.diff(first2[nw:]) <= 0).all()
 
