@@ -241,9 +241,9 @@ int rof_device_copy(void *dst, const void *src, size_t nbytes, void *stream);
 
 /* Launch tuning: how many consecutive workgroups of the partial-sum launches / of the destination-row launch
  * stay on one XCD (each XCD has its own L2, so runs of neighbouring destination rows share gathered rows
- * there).  run_launch2 = 0 (the default) lets every layout use its own choice: 64 when at least half of the
- * neighbours lie within 8192 ids of their row (block-structured graphs), 16 otherwise.  Process-wide;
- * no upstream counterpart. */
+ * there).  run_launch2 = 0 (the default) lets every layout use its own choice: one tile of destinations per
+ * run when at least half of the neighbours lie within 8192 ids of their row (block-structured graphs), 16
+ * workgroups otherwise.  Process-wide; no upstream counterpart. */
 int rof_set_xcd_run(int run_launch1, int run_launch2);
 
 /* Launch tuning: request `bytes` (0..65536) of unused LDS per workgroup, which caps how many workgroups

@@ -145,10 +145,11 @@ def test_long_rows_are_cut_by_width_and_their_segments_swept_by_source_id(lanes,
 
 
 def test_xcd_run_follows_the_locality_of_the_graph():
-    """Block-structured graphs (rows gather from their own neighbourhood) keep long runs of workgroups on one
-    XCD; graphs without that locality use short runs."""
+    """Block-structured graphs (rows gather from their own neighbourhood) keep a whole tile of destinations on
+    one XCD; graphs without that locality use short runs."""
     ip, ix = make_workload("c3", 4)                          # SBM: 24 of 26 neighbours inside the row's own block
-    assert Layout.from_csr(ip, ix).export()["xcd_run"] == 64
+    assert Layout.from_csr(ip, ix).export()["xcd_run"] == 256               # 4096-row tile / (4 wavefronts x 4 rows)
+    assert Layout.from_csr(ip, ix, lanes_per_row=64).export()["xcd_run"] == 1024
     ip, ix = make_workload("c4", 3)                          # R-MAT, 300 000 nodes: 9 % of the neighbours are nearby
     assert Layout.from_csr(ip, ix).export()["xcd_run"] == 16
 
