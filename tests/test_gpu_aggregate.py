@@ -354,3 +354,37 @@ def test_byte_offsets_between_2_and_4_gib():
     got = lay.aggregate(x, normalized=False)
     want = x[torch.from_numpy(nbr.ravel()).to(dev)].double().view(rows, per, feat).sum(1)
     assert torch.allclose(got[:rows].double(), want, rtol=1e-5, atol=1e-5)
+
+
+def test_byte_offsets_above_4_gib_and_row_ids_above_2_pow_24():
+    """The long address arithmetic (64-bit multiply per row): (1) a feature matrix of 4.6 GB gathered from its
+    top, bottom and middle; (2) 17 M nodes, so that row ids need more than 24 bits, with bf16 rows."""
+    dev = "cuda"
+    rng = np.random.default_rng(13)
+    n, feat = 6_000_000, 192
+    dst = np.sort(rng.choice(n, 3000, replace=False))
+    nbr = np.concatenate([rng.integers(n - n // 20, n, (3000, 3)), rng.integers(0, n // 20, (3000, 2)),
+                          rng.integers(n // 2, n // 2 + n // 20, (3000, 3))], axis=1)
+    nbr.sort(axis=1)
+    deg = np.zeros(n, np.int64)
+    deg[dst] = 8
+    ip = np.r_[0, np.cumsum(deg)].astype(np.int32)
+    x = torch.randn((n, feat), device=dev)
+    assert x.numel() * 4 > 2 ** 32
+    got = Layout.from_csr(ip, nbr.ravel().astype(np.int32)).aggregate(x, normalized=False)
+    want = x[torch.from_numpy(nbr.ravel()).to(dev)].double().view(3000, 8, feat).sum(1)
+    assert torch.allclose(got[torch.from_numpy(dst).to(dev)].double(), want, rtol=1e-6, atol=1e-6)
+    del x, got, want
+    torch.cuda.empty_cache()
+    n, feat = 17_000_000, 16
+    dst = np.sort(rng.choice(n, 3000, replace=False))
+    nbr = np.sort(np.concatenate([rng.integers(2 ** 24, n, (3000, 5)), rng.integers(0, n, (3000, 3))], axis=1), axis=1)
+    deg = np.zeros(n, np.int64)
+    deg[dst] = 8
+    ip = np.r_[0, np.cumsum(deg)].astype(np.int32)
+    for dtype in (torch.float32, torch.bfloat16):
+        x = torch.randn((n, feat), device=dev).to(dtype)
+        got = Layout.from_csr(ip, nbr.ravel().astype(np.int32)).aggregate(x, normalized=False)
+        want = x[torch.from_numpy(nbr.ravel()).to(dev)].double().view(3000, 8, feat).sum(1)
+        assert torch.allclose(got[torch.from_numpy(dst).to(dev)].double(), want, rtol=1e-6, atol=1e-6), dtype
+        del x, got, want
