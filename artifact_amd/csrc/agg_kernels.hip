@@ -325,6 +325,10 @@ static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64
     if (((uintptr_t)out) % (out_dtype == ROF_F32 ? 4 : 2)) return ROF_ERR_ARG;
     if (!L->uploaded || (normalized && !L->weights_set)) return ROF_ERR_STATE;
     if ((int64_t)L->n * ldx >= ((int64_t)1 << 40) || (int64_t)L->n * ldo >= ((int64_t)1 << 40)) return ROF_ERR_UNSUPPORTED;
+    if (ldx >= ((int64_t)1 << 28) || feat >= (1 << 24)) return ROF_ERR_UNSUPPORTED;   // the kernel keeps row bytes in 32 bits
+    int device = -1;
+    HIP_TRY(hipGetDevice(&device));
+    if (device != L->device) return ROF_ERR_STATE;   // the schedule lives on the device it was uploaded to
     const size_t need = rof_layout_workspace_bytes(L, feat);
     if (need && (!workspace || workspace_bytes < need)) return ROF_ERR_WORKSPACE;
     if (need && ((uintptr_t)workspace & 15)) return ROF_ERR_ARG;
