@@ -588,6 +588,30 @@ def main():
         except Exception as ex:
             result["cpu_baseline"]["scipy_error"] = str(ex)[:200]
 
+        # the host half of the path: upstream's own plan builder (compiled from its sources into oracle/_ref,
+        # when that build is present) beside this library's, same graph, same threads, results compared
+        try:
+            from artifact_amd.graphgen import make_workload
+
+            from artifact_amd import reuse_search_ext as RS
+
+            ip_s, ix_s = make_workload("c2", 1)
+            t0 = time.time()
+            mine = RS.build_plan(ip_s, ix_s, 3)
+            t_mine = time.time() - t0
+            pb = {"sample": f"R-MAT {len(ip_s) - 1} nodes, {len(ix_s)} edges, part size 3 (half of c2)",
+                  "threads": threads, "this_library_s": t_mine, "upstream_s": None}
+            if O.ref_module() is not None:
+                t0 = time.time()
+                theirs = O.ref_plan(ip_s, ix_s, 3)
+                pb["upstream_s"] = time.time() - t0
+                pb["speedup"] = pb["upstream_s"] / t_mine
+                pb["identical"] = all(np.array_equal(mine[k], theirs[k]) for k in theirs
+                                      if k in mine and isinstance(theirs[k], np.ndarray))
+            result["cpu_baseline"]["plan_builder"] = pb
+        except Exception as ex:
+            result["cpu_baseline"]["plan_builder_error"] = str(ex)[:200]
+
     print(json.dumps(result))
 
 
