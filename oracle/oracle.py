@@ -159,8 +159,9 @@ def ref_plan(indptr_dst, indices_src, part_size, indptr_src=None, indices_dst=No
 
 # --------------------------------------------------------------------------- aggregation
 def rsqrt_rn(deg):
-    """Correctly rounded fp32 1/sqrt, the value of __frsqrt_rn (cu:254)."""
-    return (1.0 / np.sqrt(np.asarray(deg, dtype=np.float64))).astype(np.float32)
+    """Correctly rounded fp32 1/sqrt, the value of __frsqrt_rn (cu:254); +inf for a degree of 0, as on the device."""
+    with np.errstate(divide="ignore"):
+        return (1.0 / np.sqrt(np.asarray(deg, dtype=np.float64))).astype(np.float32)
 
 
 def closed_form(indptr, indices, x, deg=None, normalized=True):
