@@ -163,6 +163,41 @@ def test_training_learns_and_gin_runs():
     assert out.shape == (n, 4) and all(p.grad is not None for p in gin.parameters())
 
 
+@pytest.mark.parametrize("fused", [False, True])
+def test_loss_curve_follows_a_dense_float64_model(fused):
+    """Forty Adam steps of the two-layer GCN (no dropout) against the same model written with a dense float64
+    adjacency and trained by the same optimizer from the same parameters: the loss curves must stay together
+    (fp32 round-off only), and so must the trained weights."""
+    ip, ix = make_workload("c1", 4)                                      # 1024 nodes
+    n = len(ip) - 1
+    info = build_input_info(ip, ix, 3, device=DEV, min_consumers=2)
+    x = features(n, 20, seed=61)
+    y = synthetic_labels(ip, ix, x, 6, seed=62)
+    torch.manual_seed(3)
+    model = ROF_GCN(20, 24, 6, 1, F.relu, 0.0, add_self_loops=False, reuse_size=info.reuse_size,
+                    kernel_type="ROF_v2", fuse_epilogue=fused).to(DEV)
+    params = [(l.weight.detach().cpu().double().clone().requires_grad_(True),
+               l.bias.detach().cpu().double().clone().requires_grad_(True)) for l in model.layers]
+    xt, yt = torch.from_numpy(x).to(DEV), torch.from_numpy(y).to(DEV)
+    mask = torch.ones(n, dtype=torch.bool, device=DEV)
+    losses, _, _ = train(model, xt, info, yt, mask, mask, epochs=40, lr=1e-2, weight_decay=5e-4)
+    a, xd, yd = _dense_norm_adj(ip, ix), torch.from_numpy(x).double(), torch.from_numpy(y)
+    opt = torch.optim.Adam([t for wb in params for t in wb], lr=1e-2, weight_decay=5e-4)
+    want = []
+    for _ in range(40):
+        opt.zero_grad()
+        (w1, b1), (w2, b2) = params
+        loss = F.cross_entropy(a @ (torch.relu(a @ (xd @ w1) + b1) @ w2) + b2, yd)
+        loss.backward()
+        opt.step()
+        want.append(float(loss.detach()))
+    assert want[-1] < 0.9 * want[0]                                      # the reference itself learns
+    assert np.allclose(losses, want, rtol=2e-4, atol=1e-5), np.abs(np.array(losses) - np.array(want)).max()
+    for layer, (w, b) in zip(model.layers, params):
+        assert torch.allclose(layer.weight.detach().cpu().double(), w.detach(), rtol=0, atol=2e-4)
+        assert torch.allclose(layer.bias.detach().cpu().double(), b.detach(), rtol=0, atol=2e-4)
+
+
 def test_plan_container_round_trips_through_disk(tmp_path):
     ip, ix = make_workload("c1", 4)
     n = len(ip) - 1
