@@ -19,7 +19,7 @@ SYMBOLS = (
     "rof_part_intersect_count", "rof_part_intersect_lists", "rof_greedy_max_reuse", "rof_reorganize",
     "rof_transpose_csr", "rof_plan_build", "rof_layout_from_v2", "rof_layout_from_v1", "rof_layout_from_parts",
     "rof_layout_export", "rof_layout_stats", "rof_layout_upload", "rof_layout_set_degrees",
-    "rof_plan_hub_patterns", "rof_column_sums", "rof_column_sums_workspace_bytes", "rof_layout_workspace_bytes", "rof_layout_free", "rof_aggregate", "rof_aggregate_epilogue", "rof_aggregate_timed", "rof_set_xcd_run", "rof_aggregate_launch_times", "rof_device_copy", "rof_set_lds_pad",
+    "rof_plan_hub_patterns", "rof_plan_dynamic_greedy", "rof_column_sums", "rof_column_sums_workspace_bytes", "rof_layout_workspace_bytes", "rof_layout_free", "rof_aggregate", "rof_aggregate_epilogue", "rof_aggregate_timed", "rof_set_xcd_run", "rof_aggregate_launch_times", "rof_device_copy", "rof_set_lds_pad",
 )
 
 
@@ -63,6 +63,7 @@ def lib():
     L.rof_transpose_csr.argtypes = [vp, vp, u32, u64, pp]
     L.rof_plan_build.argtypes = [vp, vp, vp, vp, u32, u64, ci, ci, pp]
     L.rof_plan_hub_patterns.argtypes = [vp, vp, u32, u64, u32, ci, pp]
+    L.rof_plan_dynamic_greedy.argtypes = [vp, vp, vp, vp, u32, u64, ci, pp]
     L.rof_layout_from_v2.argtypes = [vp, vp, vp, vp, i64, i32, ci, vp, pp]
     L.rof_layout_from_v1.argtypes = [vp, vp, vp, i64, vp, vp, vp, i64, i32, ci, vp, pp]
     L.rof_layout_from_parts.argtypes = [vp, vp, vp, i64, i32, ci, vp, pp]

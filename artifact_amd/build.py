@@ -17,7 +17,7 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "librof.so")
 
-HOST_SOURCES = ["plan_builder.cpp", "hub_patterns.cpp", "layout.cpp"]
+HOST_SOURCES = ["plan_builder.cpp", "hub_patterns.cpp", "dynamic_greedy.cpp", "layout.cpp"]
 HIP_SOURCES = ["agg_kernels.hip", "agg_rows_f32.hip", "agg_rows_bf16.hip"]
 
 # packed fp32 instructions stay off: the compiler must not form v_pk_{add,mul,fma}_f32

@@ -103,13 +103,15 @@ def build_input_info(indptr, indices, part_size=3, device="cuda", warps_per_bloc
     ROF_main.py:71-178: plan on the CPU, arrays cast to int32, degrees = diff(indptr) as float32.
     `layout_opts` (min_consumers, disable_reuse, hub_split, segment) go to the device layout.
     search="hub_patterns" (not upstream) fills the v2 tensors from reuse_search_ext.hub_pattern_plan with
-    `hubs` hubs in blocks of `part_size`; the GNNA / v1 tensors then describe the graph without reuse."""
+    `hubs` hubs in blocks of `part_size`, search="dynamic_greedy" from reuse_search_ext.dynamic_greedy_plan; the
+    GNNA / v1 tensors then describe the graph without reuse."""
     indptr = np.asarray(indptr)
     indices = np.asarray(indices)
-    if search not in ("upstream", "hub_patterns"):
-        raise ValueError("search must be 'upstream' or 'hub_patterns'")
-    if plan is None and search == "hub_patterns":
-        plan = reuse_search_ext.hub_pattern_plan(indptr, indices, hubs, part_size)
+    if search not in ("upstream", "hub_patterns", "dynamic_greedy"):
+        raise ValueError("search must be 'upstream', 'hub_patterns' or 'dynamic_greedy'")
+    if plan is None and search != "upstream":
+        plan = (reuse_search_ext.hub_pattern_plan(indptr, indices, hubs, part_size) if search == "hub_patterns"
+                else reuse_search_ext.dynamic_greedy_plan(indptr, indices, part_size))
         empty = np.zeros(0, np.uint32)
         ptr, p2n, _ = reuse_search_ext.py_split_part(empty, empty, indptr, part_size)
         plan.update(new_indices_src=np.asarray(indices), part_ptr=ptr, part2Node=p2n,

@@ -184,6 +184,27 @@ def hub_pattern_plan(indptr_dst, indices_src, hubs=16384, block=8):
     return plan
 
 
+def dynamic_greedy_plan(indptr_dst, indices_src, part_size, indptr_src=None, indices_dst=None):
+    """The dynamic greedy that upstream sketches and leaves unfinished (reuse_search_ext.h:305-321; see
+    rof_plan_dynamic_greedy in include/rof.h): the candidate part with the longest current intersection list is
+    picked, conflicting candidates lose its destinations and stay in the race.  Returns the four v2 arrays (format
+    of py_reorganize_indices_uniquely, reuse_search_ext.cc:214-257) plus "index_picked" (part indices in pick
+    order), "shared_parts", "candidates" and "part_size"; omit the out-neighbour CSR for a symmetric graph."""
+    ipd, isrc = u32(indptr_dst), u32(indices_src)
+    ips = None if indptr_src is None else u32(indptr_src)
+    idst = None if indices_dst is None else u32(indices_dst)
+    h = C.c_void_p()
+    check(_lib.lib().rof_plan_dynamic_greedy(ptr(ipd), ptr(isrc), None if ips is None else ips.ctypes.data,
+                                             None if idst is None else ptr(idst), len(ipd) - 1, len(isrc),
+                                             int(part_size), C.byref(h)))
+    plan = bag_take(h, ("uniqpart_column_index", "uniqpart_pointers", "part2Node_ptr", "part2Node_col",
+                        "index_picked", "shared_parts", "candidates"))
+    plan["shared_parts"] = int(plan["shared_parts"][0])
+    plan["candidates"] = int(plan["candidates"][0])
+    plan["part_size"] = int(part_size)
+    return plan
+
+
 def reuse_statistics(plan, part_size, num_edges):
     """The four reuse figures the upstream scripts print (ROF_evaluation/cuda/small-main.py:176-188)."""
     cnt = plan["intersect_count"][plan["index_picked"]].astype(np.int64)

@@ -224,8 +224,9 @@ def main():
     ap.add_argument("--entry-order", default="descending", choices=["descending", "plan", "ascending"],
                     help="layout tuning: order of the gathered rows inside a task")
     ap.add_argument("--tile-rows", type=int, default=0, help="layout tuning: destinations per length-sorted tile")
-    ap.add_argument("--search", default="upstream", choices=["upstream", "hub"],
-                    help="reuse search: upstream's greedy (bit-exact plan) or the hub-pattern search")
+    ap.add_argument("--search", default="upstream", choices=["upstream", "hub", "dynamic"],
+                    help="reuse search: upstream's greedy (bit-exact plan), the hub-pattern search, or the dynamic "
+                         "greedy that upstream sketches")
     ap.add_argument("--hubs", type=int, default=16384, help="--search hub: number of hub sources")
     ap.add_argument("--block", type=int, default=8, help="--search hub: hubs per block (= part size of the plan)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -268,6 +269,16 @@ def main():
         d["index_picked"] = np.arange(hp["shared_parts"], dtype=np.uint32)
         ps = args.block
         log(f"[bench] hub-pattern plan: {t_plan:.1f}s, {hp['shared_parts']} shared parts")
+    if args.search == "dynamic":
+        from artifact_amd import reuse_search_ext as R
+
+        t0 = time.time()
+        dp = R.dynamic_greedy_plan(indptr, indices, ps)
+        t_plan = time.time() - t0
+        for k in ("uniqpart_column_index", "uniqpart_pointers", "part2Node_ptr", "part2Node_col", "index_picked"):
+            d[k] = dp[k]
+        log(f"[bench] dynamic greedy plan: {t_plan:.1f}s, {dp['shared_parts']} shared parts of {dp['candidates']} "
+            f"candidates")
     deg = torch.from_numpy(np.diff(indptr).astype(np.float32)).to(dev)
 
     # features: N(0,1) fp32 (uniform(-1,1) -> bf16 for c5), rows padded to a multiple of 4 (8) elements

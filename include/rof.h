@@ -90,6 +90,17 @@ int rof_plan_build(const uint32_t *indptr_dst, const uint32_t *indices_src, cons
                    const uint32_t *indices_dst, uint32_t n, uint64_t e, int part_size, int discard_remainder_part,
                    rof_bag **out);
 
+/* A different reuse search, off by default: the "dynamic greedy" sketched and left unfinished in the comment at
+ * reuse_search_ext.h:305-321.  Candidates are the full parts with >= 2 destinations in their intersection list
+ * (h:152-228; equal source tuples count once); the candidate with the longest current list is picked, and every
+ * candidate that shares a source with it loses the picked part's destinations (ties: lower part index).  A source
+ * may thus sit in many shared parts, never in two parts of one destination.  Pass indptr_src/indices_dst = NULL
+ * for a symmetric graph.  The plan comes out in upstream's v2 format (h:537-636):
+ * bag: "uniqpart_column_index", "uniqpart_pointers"[U+1], "part2Node_ptr"[U+1], "part2Node_col",
+ *      "index_picked"[shared parts] (part indices in pick order), "shared_parts"[1], "candidates"[1]. */
+int rof_plan_dynamic_greedy(const uint32_t *indptr_dst, const uint32_t *indices_src, const uint32_t *indptr_src,
+                            const uint32_t *indices_dst, uint32_t n, uint64_t e, int part_size, rof_bag **out);
+
 /* A different reuse search, off by default: "hub patterns".  No counterpart in upstream, whose comment block at
  * reuse_search_ext.h:305-406 sketches a stronger search than its one-part-per-source greedy and leaves it
  * unfinished.  The `hubs` most frequent sources are tied into blocks of `block` (2..16) by popularity rank;

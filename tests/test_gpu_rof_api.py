@@ -194,13 +194,14 @@ def test_first_layer_without_input_gradient_skips_nothing_it_needs(oracle):
         assert np.allclose(conv.bias.grad.cpu().numpy(), coef.sum(0), rtol=1e-4, atol=1e-3), order
 
 
+@pytest.mark.parametrize("search,ps", [("hub_patterns", 8), ("dynamic_greedy", 3)])
 @pytest.mark.parametrize("kernel_type", ["GNNA", "ROF_v1", "ROF_v2"])
-def test_hub_pattern_plan_through_the_operator_api(oracle, kernel_type):
-    """The plan of the hub-pattern search travels in upstream's v2 tensors; all three kernel types give the
-    closed form on it (v1 / GNNA see the same graph without reuse)."""
+def test_plans_of_the_other_searches_through_the_operator_api(oracle, kernel_type, search, ps):
+    """The plans of the hub-pattern search and of the dynamic greedy travel in upstream's v2 tensors; all three
+    kernel types give the closed form on them (v1 / GNNA see the same graph without reuse)."""
     ip, ix = make_workload("c4", 5)
     n = len(ip) - 1
-    info = build_input_info(ip, ix, part_size=8, device=DEV, search="hub_patterns", hubs=4096, min_consumers=3)
+    info = build_input_info(ip, ix, part_size=ps, device=DEV, search=search, hubs=4096, min_consumers=3)
     assert info.layouts["ROF_v2"].get(40).stats()["materialised_groups"] > 100
     x, w = features(n, 24, seed=51), glorot(24, 40, seed=52)
     conv = ROF_GCNConv(24, 40, add_self_loops=False, kernel_type=kernel_type, reuse_size=info.reuse_size).to(DEV)
