@@ -96,14 +96,16 @@ extern "C" int rof_plan_dynamic_greedy(const uint32_t *indptr_dst, const uint32_
             delete bag;
             return rc;
         }
-        const u32 *lptr = lists.get("ptr");
         int64_t ldata_len = 0;
-        const u32 *ldata0 = lists.get("data", &ldata_len);
+        const u32 *lptr0 = lists.get("ptr"), *ldata0 = lists.get("data", &ldata_len);
+        const vec lptr(lptr0, lptr0 + (size_t)C + 1);
         vec ldata(ldata0, ldata0 + (ldata_len > 0 ? ldata_len : 0));
+        rof_bag_free(lists.b);   // the copies above are what is worked on
+        lists.b = nullptr;
         vec live(C);
         for (u32 c = 0; c < C; ++c) live[c] = lptr[c + 1] - lptr[c];
         // 64-bit signature of each list (one hashed bit per destination): two lists whose signatures do not
-        // meet have no destination in common, which settles nine out of ten comparisons without reading a list
+        // meet have no destination in common, which settles more than half of the comparisons without reading a list
         auto bit_of = [](u32 d) { return (u64)1 << ((d * 0x9E3779B1u) >> 26); };
         std::vector<u64> sig(C, 0);
 #pragma omp parallel for schedule(dynamic, 4096)
