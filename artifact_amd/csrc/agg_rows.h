@@ -80,6 +80,9 @@ struct RowLoad;
 // address, so packed rows (e.g. 47 floats = 188 bytes) are gathered with the same instruction as padded ones
 typedef float rof_f4 __attribute__((ext_vector_type(4), aligned(4)));
 typedef unsigned int rof_u4 __attribute__((ext_vector_type(4), aligned(4)));
+// naturally aligned vectors for the output stores
+typedef float rof_f4s __attribute__((ext_vector_type(4)));
+typedef unsigned int rof_u2 __attribute__((ext_vector_type(2)));
 
 template <>
 struct RowLoad<float, 4> {
@@ -214,8 +217,9 @@ __device__ __forceinline__ void gather_sum(const char *xb, uint32_t xld, const c
     }
 }
 
-// PHASE 0: the partial-sum launches (no scaling); PHASE 1: the destination-row launch.  Same code; the
-// parameter only gives them distinct kernel names in profiles.
+// PHASE 0: the partial-sum launches (no scaling, no epilogue); PHASE 1: the destination-row launch; PHASE 2: the
+// same with the output rows written as streaming stores.  (A run-time switch between the two kinds of store does
+// not survive the optimiser, which merges the two stores into an ordinary one.)
 template <typename XT, int VEC, int LPR, int PHASE, bool OFF32>
 __global__ __launch_bounds__(256, ROF_MIN_BLOCKS) void rof_rows_kernel(AggArgs a) {
     constexpr int G = 64 / LPR;
@@ -322,7 +326,7 @@ __global__ __launch_bounds__(256, ROF_MIN_BLOCKS) void rof_rows_kernel(AggArgs a
             float r[VEC];
 #pragma unroll
             for (int k = 0; k < VEC; ++k) r[k] = acc[k] * s;
-            if (PHASE == 1) {   // epilogue of the layer: + own row, + bias, then ReLU (columns cstart .. cstart+VEC-1 exist)
+            if (PHASE >= 1) {   // epilogue of the layer: + own row, + bias, then ReLU (columns cstart .. cstart+VEC-1 exist)
                 if (a.self_weight != 0.0f) {
                     float own[VEC];
                     RowLoad<XT, VEC>::load(reinterpret_cast<const XT *>(xb + (int64_t)a.task_out[t] * xld), own);
@@ -338,14 +342,20 @@ __global__ __launch_bounds__(256, ROF_MIN_BLOCKS) void rof_rows_kernel(AggArgs a
                     for (int k = 0; k < VEC; ++k) r[k] = fmaxf(r[k], 0.0f);
                 }
             }
-            if (PHASE == 1 && a.out_bf16) {
+            // A large output is not read again before the caches have turned over, so its rows are written as
+            // streaming stores (`nt`): they then do not push feature rows out of L2 and the Infinity Cache.  Whole
+            // 16-byte pieces only: element-wise streaming stores of packed rows are far slower than ordinary ones.
+            constexpr bool stream = PHASE == 2;
+            if (PHASE >= 1 && a.out_bf16) {
                 uint16_t *o = reinterpret_cast<uint16_t *>(a.out) + at;
                 if (VEC >= 4 && a.vec_store && skip == 0) {
 #pragma unroll
-                    for (int k = 0; k < VEC; k += 4)
-                        *reinterpret_cast<uint2 *>(o + k) =
-                            make_uint2(rof_bf16_bits(r[k]) | (rof_bf16_bits(r[k + 1]) << 16),
-                                       rof_bf16_bits(r[k + 2]) | (rof_bf16_bits(r[k + 3]) << 16));
+                    for (int k = 0; k < VEC; k += 4) {
+                        const rof_u2 t = {rof_bf16_bits(r[k]) | (rof_bf16_bits(r[k + 1]) << 16),
+                                          rof_bf16_bits(r[k + 2]) | (rof_bf16_bits(r[k + 3]) << 16)};
+                        if (stream) __builtin_nontemporal_store(t, reinterpret_cast<rof_u2 *>(o + k));
+                        else *reinterpret_cast<rof_u2 *>(o + k) = t;
+                    }
                 } else {
 #pragma unroll
                     for (int k = 0; k < VEC; ++k)
@@ -355,8 +365,11 @@ __global__ __launch_bounds__(256, ROF_MIN_BLOCKS) void rof_rows_kernel(AggArgs a
                 float *o = reinterpret_cast<float *>(a.out) + at;
                 if (VEC >= 4 && a.vec_store && skip == 0) {
 #pragma unroll
-                    for (int k = 0; k < VEC; k += 4)
-                        *reinterpret_cast<float4 *>(o + k) = make_float4(r[k], r[k + 1], r[k + 2], r[k + 3]);
+                    for (int k = 0; k < VEC; k += 4) {
+                        const rof_f4s t = {r[k], r[k + 1], r[k + 2], r[k + 3]};
+                        if (stream) __builtin_nontemporal_store(t, reinterpret_cast<rof_f4s *>(o + k));
+                        else *reinterpret_cast<rof_f4s *>(o + k) = t;
+                    }
                 } else {
 #pragma unroll
                     for (int k = 0; k < VEC; ++k)
@@ -409,7 +422,8 @@ int launch_lpr(const AggArgs &a0, int lpr, hipStream_t st) {
     return ROF_OK;
 }
 
-// Instantiated in agg_rows_f32.hip / agg_rows_bf16.hip.  phase 0: partial-sum launches, 1: destination rows.
+// Instantiated in agg_rows_f32.hip / agg_rows_bf16.hip.  phase 0: partial-sum launches, 1: destination rows,
+// 2: destination rows with streaming stores.
 // off32: every byte offset into the feature matrix and into the partial-sum workspace fits 32 bits and
 // every row id fits 24 bits, so the kernels may use the short address arithmetic.
 int launch_rows_f32(const AggArgs &a, int phase, int vec, bool off32, hipStream_t st);

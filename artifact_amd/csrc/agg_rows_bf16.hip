@@ -13,7 +13,8 @@ static int launch_bf16(const AggArgs &a, int vec, bool off32, hipStream_t st) {
 }
 
 int launch_rows_bf16(const AggArgs &a, int phase, int vec, bool off32, hipStream_t st) {
-    return phase == 0 ? launch_bf16<0>(a, vec, off32, st) : launch_bf16<1>(a, vec, off32, st);
+    if (phase == 0) return launch_bf16<0>(a, vec, off32, st);
+    return phase == 1 ? launch_bf16<1>(a, vec, off32, st) : launch_bf16<2>(a, vec, off32, st);
 }
 
 }  // namespace rofk

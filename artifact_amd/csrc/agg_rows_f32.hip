@@ -12,7 +12,8 @@ static int launch_f32(const AggArgs &a, int vec, bool off32, hipStream_t st) {
 }
 
 int launch_rows_f32(const AggArgs &a, int phase, int vec, bool off32, hipStream_t st) {
-    return phase == 0 ? launch_f32<0>(a, vec, off32, st) : launch_f32<1>(a, vec, off32, st);
+    if (phase == 0) return launch_f32<0>(a, vec, off32, st);
+    return phase == 1 ? launch_f32<1>(a, vec, off32, st) : launch_f32<2>(a, vec, off32, st);
 }
 
 }  // namespace rofk
