@@ -35,7 +35,7 @@ class LayoutOpts(C.Structure):
 
 class Epilogue(C.Structure):
     _fields_ = [("bias", C.c_void_p), ("relu", C.c_int32), ("out_dtype", C.c_int32), ("self_weight", C.c_float),
-                ("reserved", C.c_int32 * 3)]
+                ("pad_columns", C.c_int32), ("reserved", C.c_int32 * 2)]
 
 
 def lib():
@@ -76,14 +76,15 @@ def lib():
     L.rof_layout_free.argtypes = [vp]
     L.rof_aggregate.argtypes = [vp, vp, ci, i64, vp, i64, ci, ci, vp, C.c_size_t, vp]
     L.rof_aggregate_epilogue.argtypes = [vp, vp, ci, i64, vp, i64, ci, ci, C.POINTER(Epilogue), vp, C.c_size_t, vp]
-    L.rof_aggregate_timed.argtypes = [vp, vp, ci, i64, vp, i64, ci, ci, vp, C.c_size_t, vp, ci, C.POINTER(C.c_float)]
+    L.rof_aggregate_timed.argtypes = [vp, vp, ci, i64, vp, i64, ci, ci, C.POINTER(Epilogue), vp, C.c_size_t, vp, ci,
+                                      C.POINTER(C.c_float)]
     L.rof_set_xcd_run.argtypes = [ci, ci]
     L.rof_column_sums_workspace_bytes.argtypes = [i64, ci]
     L.rof_column_sums_workspace_bytes.restype = C.c_size_t
     L.rof_column_sums.argtypes = [vp, ci, i64, i64, ci, vp, vp, C.c_size_t, vp]
     L.rof_set_lds_pad.argtypes = [ci]
     L.rof_device_copy.argtypes = [vp, vp, C.c_size_t, vp]
-    L.rof_aggregate_launch_times.argtypes = [vp, vp, ci, i64, vp, i64, ci, ci, vp, C.c_size_t, vp, ci,
+    L.rof_aggregate_launch_times.argtypes = [vp, vp, ci, i64, vp, i64, ci, ci, C.POINTER(Epilogue), vp, C.c_size_t, vp, ci,
                                              C.POINTER(C.c_float * 2)]
     _lib = L
     return L

@@ -324,7 +324,7 @@ void rof_layout_free(rof_layout *L) {
 static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64_t ldx, void *out, int64_t ldo,
                           int feat, int normalized, void *workspace, size_t workspace_bytes, void *stream,
                           int launches, const float *bias = nullptr, int relu = 0, int out_dtype = ROF_F32,
-                          float self_weight = 0.0f) {
+                          float self_weight = 0.0f, int pad_columns = 0) {
     if (!L || !x || !out || feat < 1 || ldx < feat || ldo < feat) return ROF_ERR_ARG;
     if (x_dtype != ROF_F32 && x_dtype != ROF_BF16) return ROF_ERR_UNSUPPORTED;
     if (out_dtype != ROF_F32 && out_dtype != ROF_BF16) return ROF_ERR_UNSUPPORTED;
@@ -345,6 +345,11 @@ static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64
     // 16-byte gathers need rows that start on a 4-byte boundary and hold at least one full vector
     const bool dword_rows = (((uintptr_t)x) % 4 == 0) && ((ldx * esz) % 4 == 0);
     const int vec = (dword_rows && feat >= wide) ? wide : 1;
+    if (pad_columns && vec > 1 && feat % wide) {   // the caller lets the rows be taken as whole vectors
+        const int padded = (int)round_up(feat, wide);
+        if (ldx < padded || ldo < padded) return ROF_ERR_ARG;
+        feat = padded;   // the workspace rows are round_up(feat, 8) floats wide either way
+    }
     const int64_t ldp = round_up(feat, 8);
     const int64_t rows_x = L->n, rows_p = L->n_slots;
     const bool off32 = rows_x < (1 << 24) && rows_p < (1 << 24) && ldx * esz < (1 << 24) && ldp * 4 < (1 << 24) &&
@@ -412,12 +417,21 @@ int rof_aggregate_epilogue(const rof_layout *L, const void *x, int x_dtype, int6
     if (!ep) return aggregate_impl(L, x, x_dtype, ldx, out, ldo, feat, normalized, workspace, workspace_bytes, stream, 3);
     if (!(ep->self_weight == ep->self_weight)) return ROF_ERR_ARG;   // NaN
     return aggregate_impl(L, x, x_dtype, ldx, out, ldo, feat, normalized, workspace, workspace_bytes, stream, 3,
-                          ep->bias, ep->relu, ep->out_dtype, ep->self_weight);
+                          ep->bias, ep->relu, ep->out_dtype, ep->self_weight, ep->pad_columns);
 }
 
-int rof_aggregate_timed(const rof_layout *L, const void *x, int x_dtype, int64_t ldx, float *out, int64_t ldo,
-                        int feat, int normalized, void *workspace, size_t workspace_bytes, void *stream, int iters,
-                        float *ms_per_call) {
+static int aggregate_with(const rof_layout *L, const void *x, int x_dtype, int64_t ldx, void *out, int64_t ldo, int feat,
+                          int normalized, const rof_epilogue *ep, void *workspace, size_t workspace_bytes, void *stream,
+                          int launches) {
+    if (!ep) return aggregate_impl(L, x, x_dtype, ldx, out, ldo, feat, normalized, workspace, workspace_bytes, stream, launches);
+    if (!(ep->self_weight == ep->self_weight)) return ROF_ERR_ARG;   // NaN
+    return aggregate_impl(L, x, x_dtype, ldx, out, ldo, feat, normalized, workspace, workspace_bytes, stream, launches,
+                          ep->bias, ep->relu, ep->out_dtype, ep->self_weight, ep->pad_columns);
+}
+
+int rof_aggregate_timed(const rof_layout *L, const void *x, int x_dtype, int64_t ldx, void *out, int64_t ldo,
+                        int feat, int normalized, const rof_epilogue *ep, void *workspace, size_t workspace_bytes,
+                        void *stream, int iters, float *ms_per_call) {
     if (!ms_per_call || iters < 1) return ROF_ERR_ARG;
     hipStream_t st = (hipStream_t)stream;
     hipEvent_t e0, e1;
@@ -426,7 +440,7 @@ int rof_aggregate_timed(const rof_layout *L, const void *x, int x_dtype, int64_t
     int rc = ROF_OK;
     HIP_TRY(hipEventRecord(e0, st));
     for (int i = 0; i < iters && rc == ROF_OK; ++i)
-        rc = rof_aggregate(L, x, x_dtype, ldx, out, ldo, feat, normalized, workspace, workspace_bytes, st);
+        rc = aggregate_with(L, x, x_dtype, ldx, out, ldo, feat, normalized, ep, workspace, workspace_bytes, st, 3);
     HIP_TRY(hipEventRecord(e1, st));
     HIP_TRY(hipEventSynchronize(e1));
     float ms = 0.f;
@@ -437,9 +451,9 @@ int rof_aggregate_timed(const rof_layout *L, const void *x, int x_dtype, int64_t
     return rc;
 }
 
-int rof_aggregate_launch_times(const rof_layout *L, const void *x, int x_dtype, int64_t ldx, float *out, int64_t ldo,
-                               int feat, int normalized, void *workspace, size_t workspace_bytes, void *stream,
-                               int iters, float ms_launch[2]) {
+int rof_aggregate_launch_times(const rof_layout *L, const void *x, int x_dtype, int64_t ldx, void *out, int64_t ldo,
+                               int feat, int normalized, const rof_epilogue *ep, void *workspace,
+                               size_t workspace_bytes, void *stream, int iters, float ms_launch[2]) {
     if (!ms_launch || iters < 1 || !L) return ROF_ERR_ARG;
     hipStream_t st = (hipStream_t)stream;
     // each iteration times [launch 1 + launch 2] and then [launch 2 alone]; launch 2 alone is a
@@ -449,13 +463,13 @@ int rof_aggregate_launch_times(const rof_layout *L, const void *x, int x_dtype, 
     HIP_TRY(hipEventCreate(&e1));
     HIP_TRY(hipEventCreate(&e2));
     double both = 0.0, second = 0.0;
-    int rc = rof_aggregate(L, x, x_dtype, ldx, out, ldo, feat, normalized, workspace, workspace_bytes, st);
+    int rc = aggregate_with(L, x, x_dtype, ldx, out, ldo, feat, normalized, ep, workspace, workspace_bytes, st, 3);
     for (int i = 0; i < iters && rc == ROF_OK; ++i) {
         HIP_TRY(hipEventRecord(e0, st));
-        rc = rof_aggregate(L, x, x_dtype, ldx, out, ldo, feat, normalized, workspace, workspace_bytes, st);
+        rc = aggregate_with(L, x, x_dtype, ldx, out, ldo, feat, normalized, ep, workspace, workspace_bytes, st, 3);
         HIP_TRY(hipEventRecord(e1, st));
         if (rc == ROF_OK)
-            rc = aggregate_impl(L, x, x_dtype, ldx, out, ldo, feat, normalized, workspace, workspace_bytes, st, 2);
+            rc = aggregate_with(L, x, x_dtype, ldx, out, ldo, feat, normalized, ep, workspace, workspace_bytes, st, 2);
         HIP_TRY(hipEventRecord(e2, st));
         HIP_TRY(hipEventSynchronize(e2));
         float a = 0.f, b = 0.f;

@@ -232,30 +232,59 @@ class Layout:
         return dt, f, out, workspace
 
     def aggregate(self, x, normalized=True, out=None, feat_dim=None, workspace=None, bias=None, relu=False,
-                  out_dtype=None, self_weight=0.0):
+                  out_dtype=None, self_weight=0.0, pad_columns=False):
         """out[v] = act(s(v) * sum_u w(u) x[u] + self_weight * x[v] + bias) through the plan; x may be a
         column-padded view.  bias (float32 [feat_dim] on the device), the node's own row and relu are applied as
-        each output row is stored; out_dtype=torch.bfloat16 stores the fp32 sums rounded to bf16."""
+        each output row is stored; out_dtype=torch.bfloat16 stores the fp32 sums rounded to bf16.
+        pad_columns=True: x is a view into rows that are allocated up to the next multiple of 4 columns (8 for
+        bfloat16) and the kernel may work on whole 16-byte pieces; an output allocated here then has rows of that
+        width and the first feat_dim columns are returned as a view (see rof_epilogue in include/rof.h)."""
         import torch
 
         if out_dtype not in (None, torch.float32, torch.bfloat16):
             raise RofError("out_dtype must be float32 or bfloat16")
+        pad = 0
+        if pad_columns:
+            f0 = x.shape[1] if feat_dim is None else int(feat_dim)
+            wide = 8 if x.dtype == torch.bfloat16 else 4
+            padded = -(-f0 // wide) * wide
+            if padded != f0 and f0 >= wide and x.stride(0) >= padded:
+                pad = padded
+                if out is None:
+                    out = torch.empty((self.num_nodes, padded), dtype=out_dtype or torch.float32,
+                                      device=x.device)[:, :f0]
+                if out.stride(0) < padded:
+                    raise RofError("pad_columns needs output rows allocated up to the padded width")
+                if bias is not None:
+                    bias = torch.cat([bias, bias.new_zeros(padded - f0)])
         dt, f, out, workspace = self._args(x, out, feat_dim, workspace, out_dtype)
         st = torch.cuda.current_stream().cuda_stream
         self.upload(st)
         if bias is not None:
-            if (bias.dtype != torch.float32 or bias.device != x.device or bias.dim() != 1 or bias.numel() != f
-                    or not bias.is_contiguous()):
+            if (bias.dtype != torch.float32 or bias.device != x.device or bias.dim() != 1
+                    or bias.numel() != (pad or f) or not bias.is_contiguous()):
                 raise ValueError("bias must be a contiguous float32 vector of feat_dim elements on the device of x")
         ep = _lib.Epilogue(bias.data_ptr() if bias is not None else None, int(bool(relu)),
-                           ROF_BF16 if out.dtype == torch.bfloat16 else ROF_F32, float(self_weight))
+                           ROF_BF16 if out.dtype == torch.bfloat16 else ROF_F32, float(self_weight), int(bool(pad)))
         check(_lib.lib().rof_aggregate_epilogue(
             self._h, C.c_void_p(x.data_ptr()), dt, x.stride(0), C.c_void_p(out.data_ptr()), out.stride(0), f,
             int(bool(normalized)), C.byref(ep), C.c_void_p(workspace.data_ptr()),
             workspace.numel() * workspace.element_size(), C.c_void_p(st)))
         return out
 
-    def aggregate_timed(self, x, iters, normalized=True, out=None, feat_dim=None, workspace=None):
+    def _plain_epilogue(self, x, out, f, pad_columns):
+        """Epilogue argument of the timing helpers: none, or just the permission to work on whole vectors."""
+        import torch
+
+        if not pad_columns:
+            return None
+        wide = 8 if x.dtype == torch.bfloat16 else 4
+        padded = -(-f // wide) * wide
+        if x.stride(0) < padded or out.stride(0) < padded:
+            raise RofError("pad_columns needs input and output rows allocated up to the padded width")
+        return C.byref(_lib.Epilogue(None, 0, ROF_F32, 0.0, 1))
+
+    def aggregate_timed(self, x, iters, normalized=True, out=None, feat_dim=None, workspace=None, pad_columns=False):
         """Mean milliseconds per aggregation over `iters` back-to-back calls, measured with HIP events
         recorded on the stream the kernels run on."""
         import torch
@@ -266,12 +295,13 @@ class Layout:
         ms = C.c_float()
         check(_lib.lib().rof_aggregate_timed(self._h, C.c_void_p(x.data_ptr()), dt, x.stride(0),
                                              C.c_void_p(out.data_ptr()), out.stride(0), f, int(bool(normalized)),
+                                             self._plain_epilogue(x, out, f, pad_columns),
                                              C.c_void_p(workspace.data_ptr()),
                                              workspace.numel() * workspace.element_size(), C.c_void_p(st), int(iters),
                                              C.byref(ms)))
         return float(ms.value), out
 
-    def launch_times(self, x, iters, normalized=True, out=None, feat_dim=None, workspace=None):
+    def launch_times(self, x, iters, normalized=True, out=None, feat_dim=None, workspace=None, pad_columns=False):
         """(ms of the partial-sum launch, ms of the destination-row launch), HIP-event means over `iters`."""
         import torch
 
@@ -281,7 +311,8 @@ class Layout:
         ms = (C.c_float * 2)()
         check(_lib.lib().rof_aggregate_launch_times(self._h, C.c_void_p(x.data_ptr()), dt, x.stride(0),
                                                     C.c_void_p(out.data_ptr()), out.stride(0), f,
-                                                    int(bool(normalized)), C.c_void_p(workspace.data_ptr()),
+                                                    int(bool(normalized)), self._plain_epilogue(x, out, f, pad_columns),
+                                                    C.c_void_p(workspace.data_ptr()),
                                                     workspace.numel() * workspace.element_size(), C.c_void_p(st),
                                                     int(iters), C.byref(ms)))
         return float(ms[0]), float(ms[1])

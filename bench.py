@@ -215,6 +215,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--xcd-run", type=int, default=0, help="launch tuning: workgroups per XCD run, destination rows")
     ap.add_argument("--xcd-run-partial", type=int, default=1, help="same for the partial-sum launches")
+    ap.add_argument("--packed-output", action="store_true",
+                    help="store the output as packed [N, feat] rows instead of rows of the input's stride")
     ap.add_argument("--hub-split", type=int, default=0, help="layout tuning: rows longer than this are segmented")
     ap.add_argument("--segment", type=int, default=0, help="layout tuning: entries per segment")
     ap.add_argument("--min-consumers", type=int, default=0, help="layout tuning: share groups with >= this many consumers")
@@ -314,15 +316,19 @@ def main():
         lay.upload()
         if normalized:
             lay.set_degrees(deg)
-    out = torch.empty((n, feat), dtype=torch.float32, device=dev)
-    out_plain = torch.empty_like(out)
+    # output rows as wide as the input rows (47 floats live in rows of 48) unless --packed-output: the kernel may
+    # then store whole 16-byte pieces (rof_epilogue.pad_columns); columns 0 .. feat-1 are the same either way
+    pad = (not args.packed_output) and ld != feat
+    ldo = ld if pad else feat
+    out = torch.empty((n, ldo), dtype=torch.float32, device=dev)[:, :feat]
+    out_plain = torch.empty((n, ldo), dtype=torch.float32, device=dev)[:, :feat]
 
     # ---- warm-up: W steps, and at least ~0.3 s of work so the clocks have settled
     t0 = time.perf_counter()
     done = 0
     while done < args.warmup or time.perf_counter() - t0 < 0.3:
-        reuse.aggregate(x, normalized, out=out, feat_dim=feat)
-        plain.aggregate(x, normalized, out=out_plain, feat_dim=feat)
+        reuse.aggregate(x, normalized, out=out, feat_dim=feat, pad_columns=pad)
+        plain.aggregate(x, normalized, out=out_plain, feat_dim=feat, pad_columns=pad)
         done += 1
         if done % 8 == 0:
             torch.cuda.synchronize()
@@ -331,7 +337,7 @@ def main():
     # ---- timed region: exactly K steps between synchronisations
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        reuse.aggregate(x, normalized, out=out, feat_dim=feat)
+        reuse.aggregate(x, normalized, out=out, feat_dim=feat, pad_columns=pad)
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
 
@@ -340,22 +346,22 @@ def main():
     per = max(5, args.steps // 4)
     ev_r, ev_p = [], []
     for _ in range(4):
-        ev_r.append(reuse.aggregate_timed(x, per, normalized, out=out, feat_dim=feat)[0])
-        ev_p.append(plain.aggregate_timed(x, per, normalized, out=out_plain, feat_dim=feat)[0])
+        ev_r.append(reuse.aggregate_timed(x, per, normalized, out=out, feat_dim=feat, pad_columns=pad)[0])
+        ev_p.append(plain.aggregate_timed(x, per, normalized, out=out_plain, feat_dim=feat, pad_columns=pad)[0])
     ev_ms, plain_ms = float(np.median(ev_r)), float(np.median(ev_p))
     # per-call spread the way the upstream micro-benchmark samples it (10 warm-ups + 100 timed runs,
     # ROF_evaluation/cuda/small-main.py:364-390), one HIP-event pair per call
-    singles = sorted(reuse.aggregate_timed(x, 1, normalized, out=out, feat_dim=feat)[0] for _ in range(100))
+    singles = sorted(reuse.aggregate_timed(x, 1, normalized, out=out, feat_dim=feat, pad_columns=pad)[0] for _ in range(100))
     spread = {"runs": 100, "median_ms": float(np.median(singles)), "p10_ms": float(np.percentile(singles, 10)),
               "p90_ms": float(np.percentile(singles, 90))}
     forced_info = None
     if forced is not None:
-        out_f = torch.empty_like(out)
-        forced.aggregate(x, normalized, out=out_f, feat_dim=feat)
+        out_f = torch.empty((n, ldo), dtype=torch.float32, device=dev)[:, :feat]
+        forced.aggregate(x, normalized, out=out_f, feat_dim=feat, pad_columns=pad)
         ev_f, ev_p2 = [], []
         for _ in range(4):
-            ev_f.append(forced.aggregate_timed(x, per, normalized, out=out_f, feat_dim=feat)[0])
-            ev_p2.append(plain.aggregate_timed(x, per, normalized, out=out_plain, feat_dim=feat)[0])
+            ev_f.append(forced.aggregate_timed(x, per, normalized, out=out_f, feat_dim=feat, pad_columns=pad)[0])
+            ev_p2.append(plain.aggregate_timed(x, per, normalized, out=out_plain, feat_dim=feat, pad_columns=pad)[0])
         fs = forced.stats()
         forced_info = {"min_consumers": 3, "event_ms": float(np.median(ev_f)),
                        "speedup_vs_reuse_disabled": float(np.median(ev_p2) / np.median(ev_f)),
@@ -363,8 +369,8 @@ def main():
                        "saved_gathers_frac": 1.0 - fs["gathered_rows"] / max(1, e),
                        "max_abs_diff_vs_reuse_disabled": float((out_f - out_plain).abs().max())}
         del out_f
-    ms_a, ms_b = reuse.launch_times(x, max(5, args.steps // 2), normalized, out=out, feat_dim=feat)
-    pms_a, pms_b = plain.launch_times(x, max(5, args.steps // 2), normalized, out=out_plain, feat_dim=feat)
+    ms_a, ms_b = reuse.launch_times(x, max(5, args.steps // 2), normalized, out=out, feat_dim=feat, pad_columns=pad)
+    pms_a, pms_b = plain.launch_times(x, max(5, args.steps // 2), normalized, out=out_plain, feat_dim=feat, pad_columns=pad)
     torch.cuda.synchronize()
     max_diff = float((out - out_plain).abs().max())
 
@@ -519,7 +525,7 @@ def main():
         "vs_baseline": None,
         "dtype": "bf16->f32" if bf16 else "f32",
         "data": "synthetic",
-        "config": {"workload": DESCR[name], "nodes": n, "edges": e, "feat": feat, "row_stride": ld,
+        "config": {"workload": DESCR[name], "nodes": n, "edges": e, "feat": feat, "row_stride": ld, "out_row_stride": ldo,
                    "part_size": ps, "normalized": normalized, "search": args.search},
         "roofline": {
             "bound": "hbm", "kernel": "rof_rows_kernel (destination-row launch)",

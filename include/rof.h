@@ -211,31 +211,37 @@ int rof_aggregate(const rof_layout *layout, const void *x, int x_dtype, int64_t 
  * out_dtype ROF_F32 or ROF_BF16: the sum is always accumulated in fp32; with ROF_BF16 the finished row is
  *   rounded to nearest even and stored as bf16 (row stride ldo in elements), ready to be the bf16 input of the
  *   next layer's GEMM or aggregation without a conversion pass.
+ * pad_columns != 0: the caller allows the library to treat the rows as round_up(feat_dim, 4) (8 for bf16
+ *   features) columns wide: ldx and ldo are at least that, the extra columns of x are readable, `bias` (if any) has
+ *   that many elements, and the extra columns of `out` receive the aggregate of the extra columns of x.  Every
+ *   lane then stores whole 16-byte pieces, and a large output qualifies for streaming stores (2.4 M x 47 floats
+ *   in rows of 48: 1.24 ms against 1.32 ms).  Columns 0 .. feat_dim-1 are the same either way.
  * Rows of nodes without in-edges become act(self_weight * x[v] + bias).  ep == NULL is rof_aggregate. */
 typedef struct {
     const float *bias;
     int32_t relu;
     int32_t out_dtype;
     float self_weight;
-    int32_t reserved[3];
+    int32_t pad_columns;
+    int32_t reserved[2];
 } rof_epilogue;
 
 int rof_aggregate_epilogue(const rof_layout *layout, const void *x, int x_dtype, int64_t ldx, void *out, int64_t ldo,
                            int feat_dim, int normalized, const rof_epilogue *epilogue, void *workspace,
                            size_t workspace_bytes, void *stream);
 
-/* Timing helper for benchmarks: runs rof_aggregate `iters` times on `stream` between two HIP
+/* Timing helper for benchmarks: runs rof_aggregate_epilogue (rof_aggregate when epilogue == NULL) `iters` times on `stream` between two HIP
  * events recorded on that same stream and returns the mean milliseconds per call. */
-int rof_aggregate_timed(const rof_layout *layout, const void *x, int x_dtype, int64_t ldx, float *out, int64_t ldo,
-                        int feat_dim, int normalized, void *workspace, size_t workspace_bytes, void *stream,
-                        int iters, float *ms_per_call);
+int rof_aggregate_timed(const rof_layout *layout, const void *x, int x_dtype, int64_t ldx, void *out, int64_t ldo,
+                        int feat_dim, int normalized, const rof_epilogue *epilogue, void *workspace,
+                        size_t workspace_bytes, void *stream, int iters, float *ms_per_call);
 
 /* Per-launch timing for the roofline report: ms_launch[1] = mean duration of the destination-row
  * launch alone (HIP events on `stream` around it), ms_launch[0] = mean duration of the whole call minus
  * that, i.e. the partial-sum launch.  No upstream counterpart. */
-int rof_aggregate_launch_times(const rof_layout *layout, const void *x, int x_dtype, int64_t ldx, float *out,
-                               int64_t ldo, int feat_dim, int normalized, void *workspace, size_t workspace_bytes,
-                               void *stream, int iters, float ms_launch[2]);
+int rof_aggregate_launch_times(const rof_layout *layout, const void *x, int x_dtype, int64_t ldx, void *out,
+                               int64_t ldo, int feat_dim, int normalized, const rof_epilogue *epilogue,
+                               void *workspace, size_t workspace_bytes, void *stream, int iters, float ms_launch[2]);
 
 /* Column sums of a row-major device matrix: out[c] = sum_r x[r, c], x float32 or bfloat16 [n, f] with row
  * stride ldx (elements), out float32[f].  This is the bias gradient of a layer (upstream leaves it to autograd's

@@ -14,6 +14,7 @@ torch = pytest.importorskip("torch")
 from artifact_amd import reuse_search_ext as R            # noqa: E402
 from artifact_amd.graphgen import features, make_workload  # noqa: E402
 from artifact_amd.layout import Layout                     # noqa: E402
+from artifact_amd._lib import RofError                     # noqa: E402
 
 
 def _case(name, scale_down, ps):
@@ -388,3 +389,28 @@ def test_byte_offsets_above_4_gib_and_row_ids_above_2_pow_24():
         want = x[torch.from_numpy(nbr.ravel()).to(dev)].double().view(3000, 8, feat).sum(1)
         assert torch.allclose(got[torch.from_numpy(dst).to(dev)].double(), want, rtol=1e-6, atol=1e-6), dtype
         del x, got, want
+
+
+@pytest.mark.parametrize("feat,bf16_in,bf16_out", [(47, False, False), (5, False, False), (101, False, True),
+                                                    (41, True, False), (13, True, True), (48, False, False)])
+def test_rows_taken_as_whole_vectors_give_the_same_columns(oracle, feat, bf16_in, bf16_out):
+    """pad_columns lets the kernel read and write the rows up to the next multiple of 4 (8) columns; the first
+    feat columns must come out bit for bit as without it, whatever the padding of x holds."""
+    indptr, indices, plan = _case("c1", 2, 3)
+    n = len(indptr) - 1
+    wide = 8 if bf16_in else 4
+    ld = -(-feat // wide) * wide
+    lay = _layout(plan, n, 3, min_consumers=2, hub_split=40)
+    lay.set_degrees(torch.from_numpy(np.diff(indptr).astype(np.float32)).cuda())
+    buf = torch.randn((n, ld), device="cuda")                      # the padding columns hold arbitrary values
+    buf = buf.to(torch.bfloat16) if bf16_in else buf
+    x = buf[:, :feat]
+    bias = torch.randn(feat, device="cuda")
+    kw = dict(normalized=True, bias=bias, relu=True, self_weight=0.5, out_dtype=torch.bfloat16 if bf16_out else None)
+    want = lay.aggregate(x, **kw)
+    got = lay.aggregate(x, pad_columns=True, **kw)
+    assert got.shape == (n, feat) and torch.equal(got, want)
+    if feat % wide:
+        assert got.stride(0) == ld                                 # rows of the padded width, returned as a view
+        with pytest.raises(RofError):
+            lay.aggregate(x, pad_columns=True, out=torch.empty((n, feat), device="cuda", dtype=want.dtype), **kw)
