@@ -159,7 +159,7 @@ def _backward(family, d_output, X, W, degrees):
     f = d_output.shape[1]
     layout = family.get(f)
     layout.set_degrees(degrees)
-    d_input_prime = layout.aggregate(_padded(d_output), normalized=True, feat_dim=f)
+    d_input_prime = layout.aggregate(_padded(d_output), normalized=True, feat_dim=f, pad_columns=True)   # an intermediate: rows of the padded stride
     d_input = torch.mm(d_input_prime, W.transpose(0, 1))
     d_weight = _weight_grad(X, d_input_prime)
     return [d_input, d_weight], layout

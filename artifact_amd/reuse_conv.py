@@ -312,7 +312,7 @@ class ROF_GCNLayerFunc(torch.autograd.Function):
         elif ctx.needs_input_grad[0] or ctx.needs_input_grad[1]:
             lay = ctx.fam.get(g.shape[1], ctx.bf16)
             lay.set_degrees(ctx.deg)
-            dt = lay.aggregate(g, normalized=True, feat_dim=g.shape[1], out_dtype=gdt)
+            dt = lay.aggregate(g, normalized=True, feat_dim=g.shape[1], out_dtype=gdt, pad_columns=True)   # internal: rows may keep the padded stride
             if ctx.needs_input_grad[0]:
                 d_x = torch.mm(dt, wb.transpose(0, 1)).to(ctx.x_dtype)
             if ctx.needs_input_grad[1]:

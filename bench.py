@@ -30,7 +30,7 @@ HBM_PEAK_GBS = 8000.0
 # (FETCH_SIZE x 2.0 + WRITE_SIZE, the factors coming from a 1 GiB copy of known size).  Counters cannot be read
 # from inside this script, so the figures are carried here and reported only for the configurations they were
 # measured on: (workload, part size, width) with default layout options.
-PROFILED_TRAFFIC_BYTES = {("c4", 3, 47): (1.75e9, 6.53e9), ("c5", 3, 256): (24.94e9, 23.56e9),
+PROFILED_TRAFFIC_BYTES = {("c4", 3, 47): (1.76e9, 6.12e9), ("c5", 3, 256): (24.94e9, 23.56e9),
                           ("c3", 3, 64): (None, 1.19e9)}
 
 DESCR = {
@@ -509,7 +509,8 @@ def main():
     achieved_b = bytes_b / (ms_b * 1e-3) / 1e9
     default_opts = (not (args.hub_split or args.segment or args.min_consumers or args.fold_sources)
                     and args.search == "upstream" and args.entry_order == "descending" and not args.tile_rows)
-    traffic = PROFILED_TRAFFIC_BYTES.get((name, ps, feat), (None, None)) if default_opts else (None, None)
+    traffic = (PROFILED_TRAFFIC_BYTES.get((name, ps, feat), (None, None)) if default_opts and not args.packed_output
+               else (None, None))
     achieved_a = bytes_a / (ms_a * 1e-3) / 1e9 if ms_a > 0 else 0.0
 
     result = {
