@@ -162,8 +162,9 @@ __device__ __forceinline__ void gather_sum(const char *xb, uint32_t xld, const c
         int32_t mycol = bias;               // past the end: row 0 of the source, weight 0
         float myw = 0.0f;
         if (!idle && mine < end) {
-            mycol = col[mine];
-            myw = w ? w[mine] : 1.0f;
+            // read once per launch: streaming loads, so that they do not push feature rows out of the caches
+            mycol = __builtin_nontemporal_load(col + mine);
+            myw = w ? __builtin_nontemporal_load(w + mine) : 1.0f;
         }
 #pragma unroll
         for (int j0 = 0; j0 < LPR; j0 += U) {
