@@ -147,7 +147,7 @@ __device__ __forceinline__ const char *row_ptr(int32_t c, const char *xb, uint32
 // the task (beg/end wave-uniform) and take every G-th entry; otherwise each lane group owns its
 // task.  ST is the element type of the source rows.  Blocks of U entries that are complete for every
 // lane group run without any per-entry predicate; ragged ends are predicated entry by entry.
-template <typename ST, int VEC, int LPR, bool WAVE, bool DUAL, bool OFF32>
+template <typename ST, int VEC, int LPR, bool WAVE, bool DUAL, bool OFF32, bool STREAM_IDS>
 __device__ __forceinline__ void gather_sum(const char *xb, uint32_t xld, const char *pb, uint32_t pld, int32_t nsplit,
                                            int32_t bias, const int32_t *__restrict__ col,
                                            const float *__restrict__ w, int32_t beg, int32_t end, int lane, int sub,
@@ -162,9 +162,16 @@ __device__ __forceinline__ void gather_sum(const char *xb, uint32_t xld, const c
         int32_t mycol = bias;               // past the end: row 0 of the source, weight 0
         float myw = 0.0f;
         if (!idle && mine < end) {
-            // read once per launch: streaming loads, so that they do not push feature rows out of the caches
-            mycol = __builtin_nontemporal_load(col + mine);
-            myw = w ? __builtin_nontemporal_load(w + mine) : 1.0f;
+            if constexpr (STREAM_IDS) {
+                // read once per launch, and the launch is a large one (see PHASE 2): streaming loads, so that they
+                // do not push feature rows out of the caches.  Small graphs keep their index arrays cached from one
+                // layer to the next and are better off with ordinary loads.
+                mycol = __builtin_nontemporal_load(col + mine);
+                myw = w ? __builtin_nontemporal_load(w + mine) : 1.0f;
+            } else {
+                mycol = col[mine];
+                myw = w ? w[mine] : 1.0f;
+            }
         }
 #pragma unroll
         for (int j0 = 0; j0 < LPR; j0 += U) {
@@ -219,7 +226,8 @@ __device__ __forceinline__ void gather_sum(const char *xb, uint32_t xld, const c
 }
 
 // PHASE 0: the partial-sum launches (no scaling, no epilogue); PHASE 1: the destination-row launch; PHASE 2: the
-// same with the output rows written as streaming stores.  (A run-time switch between the two kinds of store does
+// same with the output rows written as streaming stores and the index arrays read as streaming loads (large outputs,
+// hence large graphs).  (A run-time switch between the two kinds of store does
 // not survive the optimiser, which merges the two stores into an ordinary one.)
 template <typename XT, int VEC, int LPR, int PHASE, bool OFF32>
 __global__ __launch_bounds__(256, ROF_MIN_BLOCKS) void rof_rows_kernel(AggArgs a) {
@@ -273,16 +281,16 @@ __global__ __launch_bounds__(256, ROF_MIN_BLOCKS) void rof_rows_kernel(AggArgs a
             if (kF32) {
                 // only tasks that reference partial rows pay for the select between the two matrices
                 if (mid > beg)
-                    gather_sum<XT, VEC, LPR, true, true, OFF32>(xb, xld, pb, pld, a.nsplit, 0, a.col, a.w, beg, end,
+                    gather_sum<XT, VEC, LPR, true, true, OFF32, PHASE == 2>(xb, xld, pb, pld, a.nsplit, 0, a.col, a.w, beg, end,
                                                                 lane, sub, li, act, acc);
                 else
-                    gather_sum<XT, VEC, LPR, true, false, OFF32>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, beg, end, lane,
+                    gather_sum<XT, VEC, LPR, true, false, OFF32, PHASE == 2>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, beg, end, lane,
                                                                  sub, li, act, acc);
             } else {
                 if (mid > beg)
-                    gather_sum<float, VEC, LPR, true, false, OFF32>(pb, pld, nullptr, 0, 0, a.nsplit, a.col, a.w, beg,
+                    gather_sum<float, VEC, LPR, true, false, OFF32, PHASE == 2>(pb, pld, nullptr, 0, 0, a.nsplit, a.col, a.w, beg,
                                                                     mid, lane, sub, li, act, acc);
-                gather_sum<XT, VEC, LPR, true, false, OFF32>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, mid, end, lane, sub,
+                gather_sum<XT, VEC, LPR, true, false, OFF32, PHASE == 2>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, mid, end, lane, sub,
                                                              li, act, acc);
             }
             if ((G & (G - 1)) == 0) {   // power-of-two group count: butterfly
@@ -303,16 +311,16 @@ __global__ __launch_bounds__(256, ROF_MIN_BLOCKS) void rof_rows_kernel(AggArgs a
         } else {
             if (kF32) {
                 if (__any(mid > beg))
-                    gather_sum<XT, VEC, LPR, false, true, OFF32>(xb, xld, pb, pld, a.nsplit, 0, a.col, a.w, beg, end,
+                    gather_sum<XT, VEC, LPR, false, true, OFF32, PHASE == 2>(xb, xld, pb, pld, a.nsplit, 0, a.col, a.w, beg, end,
                                                                  lane, sub, li, act, acc);
                 else
-                    gather_sum<XT, VEC, LPR, false, false, OFF32>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, beg, end, lane,
+                    gather_sum<XT, VEC, LPR, false, false, OFF32, PHASE == 2>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, beg, end, lane,
                                                                   sub, li, act, acc);
             } else {
                 if (__any(mid > beg))
-                    gather_sum<float, VEC, LPR, false, false, OFF32>(pb, pld, nullptr, 0, 0, a.nsplit, a.col, a.w, beg,
+                    gather_sum<float, VEC, LPR, false, false, OFF32, PHASE == 2>(pb, pld, nullptr, 0, 0, a.nsplit, a.col, a.w, beg,
                                                                      mid, lane, sub, li, act, acc);
-                gather_sum<XT, VEC, LPR, false, false, OFF32>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, mid, end, lane, sub,
+                gather_sum<XT, VEC, LPR, false, false, OFF32, PHASE == 2>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, mid, end, lane, sub,
                                                               li, act, acc);
             }
         }
