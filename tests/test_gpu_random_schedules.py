@@ -1,6 +1,7 @@
 """Randomised parity of the aggregation through the C ABI: random graphs (empty rows, hubs), random plans
 (upstream's builder or none), random schedule options (cut, segment length, lanes per row, entry order, tile
-size), random widths, strides, input and output types and epilogues, each against the float64 closed form
+size), random widths, strides (with and without permission to use the padding), input and output types and
+epilogues, each against the float64 closed form
     out[v] = relu( rs(deg v) * sum_u rs(deg u) x[u]  +  self_weight * x[v]  +  bias )
 (reuse_conv_kernel.cu:254,276 for the normalisation; reuse_conv.py:147-150 for the bias).  The schedule may
 re-bracket the sum in any way, so every case must meet the same bar: fp32 rel 1e-5 (+ the summation bound),
@@ -73,22 +74,24 @@ def test_random_schedules_match_the_closed_form(oracle, block):
         bias = rng.standard_normal(feat).astype(np.float32) if rng.random() < 0.5 else None
         relu = rng.random() < 0.5
         self_weight = float(rng.choice([0.0, 0.0, 0.7, -1.25]))
+        pad = bool(rng.random() < 0.4)                         # rows taken as whole vectors where the stride allows it
         what = (f"seed {seed}: n {n} edges {len(ix)} ps {ps} plan {use_plan} {opts} feat {feat} ld {ld} "
                 f"bf16 in {bf16_in} out {bf16_out} normalized {normalized} bias {bias is not None} relu {relu} "
-                f"self {self_weight} stats {lay.stats()}")
+                f"self {self_weight} pad {pad} stats {lay.stats()}")
         print(what, flush=True)
 
         x = rng.standard_normal((n, feat)).astype(np.float32)
         if bf16_in:
             x = bf16_round(x)
         deg = rng.integers(1, 50, n).astype(np.float32)        # the degrees are an input of their own (cu:254)
-        base = torch.zeros((n, ld), dtype=torch.bfloat16 if bf16_in else torch.float32, device="cuda")
+        base = torch.full((n, ld), 3.0, dtype=torch.bfloat16 if bf16_in else torch.float32, device="cuda")   # padding: junk
         base[:, :feat] = torch.from_numpy(x).cuda()
         xt = base[:, :feat]
         if normalized:
             lay.set_degrees(torch.from_numpy(deg).cuda())
         got = lay.aggregate(xt, normalized=normalized, bias=None if bias is None else torch.from_numpy(bias).cuda(),
-                            relu=relu, out_dtype=torch.bfloat16 if bf16_out else None, self_weight=self_weight)
+                            relu=relu, out_dtype=torch.bfloat16 if bf16_out else None, self_weight=self_weight,
+                            pad_columns=pad)
         assert got.dtype == (torch.bfloat16 if bf16_out else torch.float32) and got.shape == (n, feat)
         got = got.float().cpu().numpy().astype(np.float64)
 
