@@ -34,6 +34,8 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
+#include <atomic>
+#include <mutex>
 #include <new>
 
 #include "agg_rows.h"
@@ -190,6 +192,37 @@ void free_phase(rof_phase_dev &d) {
 
 inline int64_t round_up(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
 
+// Partial-sum rows of rof_aggregate_noalloc: device memory that belongs to the library's code object, so a
+// caller that may not allocate (HIP graph capture, a serving loop) does not have to bring a workspace.  Each
+// GPU the library runs on holds its own copy, at its own address, until the process ends.  In host code the
+// array's name is only a handle for hipGetSymbolAddress; the address it returns for the current device is what
+// kernels and copies are given.
+constexpr size_t kScratchBytes = ROF_NOALLOC_WORKSPACE_BYTES;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+constexpr int kMaxDevices = 64;
+std::atomic<void *> g_scratch_ptr[kMaxDevices];
+std::mutex g_scratch_mu;
+
+// Address of `scratch` on the current device, looked up once per device.
+int scratch_of_current_device(void **out) {
+    int dev = -1;
+    HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return ROF_ERR_UNSUPPORTED;
+    void *p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        std::lock_guard<std::mutex> lock(g_scratch_mu);
+        p = g_scratch_ptr[dev].load(std::memory_order_relaxed);
+        if (!p) {
+            HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+            if (!p) return ROF_ERR_DEVICE;
+            g_scratch_ptr[dev].store(p, std::memory_order_release);
+        }
+    }
+    *out = p;
+    return ROF_OK;
+}
+
 }  // namespace
 
 void rof_set_device_error(const char *what, const char *text) {
@@ -283,7 +316,8 @@ int rof_layout_upload(rof_layout *L, void *stream) {
     }
     HIP_TRY(hipStreamSynchronize(st));   // the host vectors may be released after this call
     L->uploaded = true;
-    return ROF_OK;
+    void *unused = nullptr;   // set-up is also where this device's copy of the static scratch gets its address
+    return scratch_of_current_device(&unused);
 }
 
 int rof_layout_set_degrees(rof_layout *L, const float *deg, void *stream) {
@@ -418,6 +452,23 @@ int rof_aggregate_epilogue(const rof_layout *L, const void *x, int x_dtype, int6
     if (!(ep->self_weight == ep->self_weight)) return ROF_ERR_ARG;   // NaN
     return aggregate_impl(L, x, x_dtype, ldx, out, ldo, feat, normalized, workspace, workspace_bytes, stream, 3,
                           ep->bias, ep->relu, ep->out_dtype, ep->self_weight, ep->pad_columns);
+}
+
+int rof_aggregate_noalloc(const rof_layout *L, const void *x, int x_dtype, int64_t ldx, void *out, int64_t ldo,
+                          int feat, int normalized, const rof_epilogue *ep, void *stream) {
+    if (!L || feat < 1) return ROF_ERR_ARG;
+    const size_t need = rof_layout_workspace_bytes(L, feat);
+    if (need > kScratchBytes) {
+        rof_set_device_error("rof_aggregate_noalloc",
+                             "the layout's partial-sum rows exceed ROF_NOALLOC_WORKSPACE_BYTES; use rof_aggregate "
+                             "with a caller-allocated workspace");
+        return ROF_ERR_WORKSPACE;
+    }
+    void *ws = nullptr;
+    int rc = scratch_of_current_device(&ws);
+    if (rc) return rc;
+    // every partial row a launch reads was written earlier in the same call, so nothing has to be cleared
+    return rof_aggregate_epilogue(L, x, x_dtype, ldx, out, ldo, feat, normalized, ep, ws, kScratchBytes, stream);
 }
 
 static int aggregate_with(const rof_layout *L, const void *x, int x_dtype, int64_t ldx, void *out, int64_t ldo, int feat,

@@ -14,6 +14,7 @@ from . import _lib
 from ._lib import LayoutOpts, RofError, bag_take, check, i32, ptr
 
 ROF_F32, ROF_BF16 = 0, 1
+NOALLOC_WORKSPACE_BYTES = 64 << 20   # ROF_NOALLOC_WORKSPACE_BYTES of include/rof.h
 
 STAT_NAMES = ("nodes", "edges", "groups", "materialised_groups", "gathered_rows", "partial_reads", "partial_rows",
               "hub_segments", "tasks_a", "tasks_b", "device_bytes", "part_size", "wave_tasks_a", "wave_tasks_b",
@@ -270,6 +271,30 @@ class Layout:
             self._h, C.c_void_p(x.data_ptr()), dt, x.stride(0), C.c_void_p(out.data_ptr()), out.stride(0), f,
             int(bool(normalized)), C.byref(ep), C.c_void_p(workspace.data_ptr()),
             workspace.numel() * workspace.element_size(), C.c_void_p(st)))
+        return out
+
+    def aggregate_noalloc(self, x, out, normalized=True, feat_dim=None, bias=None, relu=False, self_weight=0.0):
+        """`aggregate` into a caller-provided `out` through rof_aggregate_noalloc: the partial-sum rows live in the
+        library's static device array (NOALLOC_WORKSPACE_BYTES per GPU), and neither the library nor this wrapper
+        allocates device memory.  Raises when the layout needs more than that, or was not uploaded yet (uploading
+        allocates).  Calls that overlap on one GPU share the array and must be serialised by the caller."""
+        import torch
+
+        if out is None:
+            raise RofError("aggregate_noalloc needs an output tensor: it allocates nothing")
+        dt, f, out, _ = self._args(x, out, feat_dim, out, out.dtype)   # no workspace tensor is created
+        if bias is not None and (bias.dtype != torch.float32 or bias.device != x.device or bias.dim() != 1
+                                 or bias.numel() != f or not bias.is_contiguous()):
+            raise ValueError("bias must be a contiguous float32 vector of feat_dim elements on the device of x")
+        ep = _lib.Epilogue(bias.data_ptr() if bias is not None else None, int(bool(relu)),
+                           ROF_BF16 if out.dtype == torch.bfloat16 else ROF_F32, float(self_weight), 0)
+        L = _lib.lib()
+        rc = L.rof_aggregate_noalloc(self._h, C.c_void_p(x.data_ptr()), dt, x.stride(0), C.c_void_p(out.data_ptr()),
+                                     out.stride(0), f, int(bool(normalized)), C.byref(ep),
+                                     C.c_void_p(torch.cuda.current_stream().cuda_stream))
+        if rc == -7:
+            raise RofError("librof: " + L.rof_last_device_error().decode() + " (status -7)")
+        check(rc)
         return out
 
     def _plain_epilogue(self, x, out, f, pad_columns):

@@ -230,6 +230,22 @@ int rof_aggregate_epilogue(const rof_layout *layout, const void *x, int x_dtype,
                            int feat_dim, int normalized, const rof_epilogue *epilogue, void *workspace,
                            size_t workspace_bytes, void *stream);
 
+/* rof_aggregate_epilogue for callers that cannot allocate device memory or bring a workspace: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in upstream (whose
+ * operators allocate their output and intermediates on every call, reuse_conv_kernel.cu:302-303).  The partial-sum rows live in a static device array of
+ * ROF_NOALLOC_WORKSPACE_BYTES inside the library, one copy per GPU, held until the process ends; the call itself
+ * allocates and frees nothing.  Its address on a device is looked up once, by rof_layout_upload or by the first
+ * call on that device (so make that first call outside a graph capture).
+ * Returns ROF_ERR_WORKSPACE (rof_last_device_error() names the limit) when
+ * rof_layout_workspace_bytes(layout, feat_dim) exceeds ROF_NOALLOC_WORKSPACE_BYTES: use rof_aggregate_epilogue
+ * with a workspace of your own then.  All calls on one GPU share the array: calls that overlap in time on one
+ * GPU (different streams or threads) race and must be serialised by the caller.  Nothing in the array has to be
+ * cleared between calls, because every partial row is written before it is read within one call.
+ * x, out, epilogue (may be NULL) and the result are exactly those of rof_aggregate_epilogue. */
+#define ROF_NOALLOC_WORKSPACE_BYTES ((size_t)64 << 20)
+int rof_aggregate_noalloc(const rof_layout *layout, const void *x, int x_dtype, int64_t ldx, void *out, int64_t ldo,
+                          int feat_dim, int normalized, const rof_epilogue *epilogue, void *stream);
+
 /* Timing helper for benchmarks: runs rof_aggregate_epilogue (rof_aggregate when epilogue == NULL) `iters` times on `stream` between two HIP
  * events recorded on that same stream and returns the mean milliseconds per call. */
 int rof_aggregate_timed(const rof_layout *layout, const void *x, int x_dtype, int64_t ldx, void *out, int64_t ldo,
