@@ -110,24 +110,6 @@ def _update(x, weight):
     return torch.mm(x, wpad), f
 
 
-def _padded(t):
-    """Packed rows are gathered in place: the kernels read 16 bytes at any 4-byte boundary."""
-    return t
-
-
-def _restrided(t):
-    """Copy of `t` whose row stride is a multiple of four floats (rows then start on 16-byte boundaries and
-    straddle fewer cache lines).  Not used on the operator path; kept for measurements."""
-    f = t.shape[1]
-    pad = (-f) % 4
-    if pad == 0:
-        return t
-    buf = t.new_empty(t.shape[0], f + pad)
-    buf[:, :f].copy_(t)
-    buf[:, f:].zero_()
-    return buf
-
-
 def _weight_grad(x, d):
     """x^T @ d in float32 for tall operands ([N, in]^T [N, out], N in the millions): the product has only
     in * out outputs, far too few tiles to fill the GPU, and a single GEMM call runs at a tenth of the memory
@@ -159,7 +141,9 @@ def _backward(family, d_output, X, W, degrees):
     f = d_output.shape[1]
     layout = family.get(f)
     layout.set_degrees(degrees)
-    d_input_prime = layout.aggregate(_padded(d_output), normalized=True, feat_dim=f, pad_columns=True)   # an intermediate: rows of the padded stride
+    # the packed gradient is gathered in place (16-byte loads at any 4-byte boundary); the result is an
+    # intermediate and keeps rows of the padded stride
+    d_input_prime = layout.aggregate(d_output, normalized=True, feat_dim=f, pad_columns=True)
     d_input = torch.mm(d_input_prime, W.transpose(0, 1))
     d_weight = _weight_grad(X, d_input_prime)
     return [d_input, d_weight], layout
@@ -170,7 +154,7 @@ def SAG(input, row_pointers, column_index, degrees, part_pointers, part2Node, pa
     _check(input=input, row_pointers=row_pointers, column_index=column_index, degrees=degrees,
            part_pointers=part_pointers, part2Node=part2Node)
     fam = _layout_parts(column_index, part_pointers, part2Node, input.shape[0], partSize)
-    return fam.get(input.shape[1]).aggregate(_padded(input), normalized=False, feat_dim=input.shape[1])
+    return fam.get(input.shape[1]).aggregate(input, normalized=False, feat_dim=input.shape[1])
 
 
 def GNNA_forward(input, weight, column_index, degrees, part_pointers, part2Node, partSize, dimWorker, warpPerBlock):

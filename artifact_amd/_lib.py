@@ -10,7 +10,7 @@ import os
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.environ.get("ROF_LIBRARY") or os.path.join(_HERE, "librof.so")   # override: experiments only
+LIB_PATH = os.path.join(_HERE, "librof.so")
 _lib = None
 
 # every symbol include/rof.h declares (checked by the CPU test-suite against the header text)

@@ -40,6 +40,7 @@
 
 #include "agg_rows.h"
 #include "rof.h"
+#include "rof_bench.h"
 #include "rof_internal.h"
 
 namespace rofk {
@@ -58,8 +59,10 @@ thread_local char g_dev_err[256] = "";
 
 // An output of this size or more is written with streaming stores: it would not survive in the 256 MB Infinity
 // Cache until its consumer runs anyway, and written normally it evicts the feature rows the gathers re-read.
-// Measured on MI355X (outputs of 268 MB): block-structured graph -9 %, R-MAT 2^18 x 256 floats -2.5 %; only rows
-// stored in whole 16-byte pieces qualify (packed 47-float rows written element by element: +17 % when streamed).
+// Measured on MI355X (outputs of 268 MB): block-structured graph -9 %, R-MAT 2^18 x 256 floats -2.5 %; packed
+// 47-float rows (2.4 M of them, stored as 16-byte pieces at dword alignment) -1.8 %.  Rows whose pieces cannot be
+// stored whole (scalar instantiation, bf16 rows of odd stride) keep ordinary stores: streamed element by element
+// they were 17 % slower.
 constexpr int64_t kStreamOutBytes = 128 << 20;
 
 // rsqrt of the in-degree, correctly rounded like __frsqrt_rn (reuse_conv_kernel.cu:254,276)
@@ -430,11 +433,12 @@ static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64
         a.n_tasks = L->db.n_tasks;
         a.xcd_run = g_xcd_run_b > 0 ? g_xcd_run_b : L->xcd_run;
         a.out_bf16 = out_dtype == ROF_BF16;
-        a.vec_store = (ldo % 4 == 0) && (((uintptr_t)out) % (a.out_bf16 ? 8 : 16) == 0);
+        a.vec_store = ((uintptr_t)out) % 4 == 0;   // pieces of a row are stored whole wherever they start on a dword
         a.bias = bias;
         a.relu = relu ? 1 : 0;
         a.self_weight = self_weight;
-        const int phase = ((int64_t)L->n * feat * (a.out_bf16 ? 2 : 4) >= kStreamOutBytes && a.vec_store && vec > 1 && feat % vec == 0) ? 2 : 1;
+        const int phase = ((int64_t)L->n * feat * (a.out_bf16 ? 2 : 4) >= kStreamOutBytes && a.vec_store && vec > 1 &&
+                           (!a.out_bf16 || ldo % 2 == 0)) ? 2 : 1;
         if ((rc = (x_dtype == ROF_F32 ? rofk::launch_rows_f32(a, phase, vec, off32, st) : rofk::launch_rows_bf16(a, phase, vec, off32, st)))) return rc;
     }
     return ROF_OK;
@@ -480,24 +484,36 @@ static int aggregate_with(const rof_layout *L, const void *x, int x_dtype, int64
                           ep->bias, ep->relu, ep->out_dtype, ep->self_weight, ep->pad_columns);
 }
 
+namespace {
+// HIP events that are destroyed on every exit path
+struct EventSet {
+    hipEvent_t ev[3] = {nullptr, nullptr, nullptr};
+    int n = 0;
+    int create(int count) {
+        for (; n < count; ++n) HIP_TRY(hipEventCreate(&ev[n]));
+        return ROF_OK;
+    }
+    ~EventSet() {
+        for (int i = 0; i < n; ++i) (void)hipEventDestroy(ev[i]);
+    }
+};
+}  // namespace
+
 int rof_aggregate_timed(const rof_layout *L, const void *x, int x_dtype, int64_t ldx, void *out, int64_t ldo,
                         int feat, int normalized, const rof_epilogue *ep, void *workspace, size_t workspace_bytes,
                         void *stream, int iters, float *ms_per_call) {
     if (!ms_per_call || iters < 1) return ROF_ERR_ARG;
     hipStream_t st = (hipStream_t)stream;
-    hipEvent_t e0, e1;
-    HIP_TRY(hipEventCreate(&e0));
-    HIP_TRY(hipEventCreate(&e1));
-    int rc = ROF_OK;
-    HIP_TRY(hipEventRecord(e0, st));
+    EventSet e;
+    int rc = e.create(2);
+    if (rc) return rc;
+    HIP_TRY(hipEventRecord(e.ev[0], st));
     for (int i = 0; i < iters && rc == ROF_OK; ++i)
         rc = aggregate_with(L, x, x_dtype, ldx, out, ldo, feat, normalized, ep, workspace, workspace_bytes, st, 3);
-    HIP_TRY(hipEventRecord(e1, st));
-    HIP_TRY(hipEventSynchronize(e1));
+    HIP_TRY(hipEventRecord(e.ev[1], st));
+    HIP_TRY(hipEventSynchronize(e.ev[1]));
     float ms = 0.f;
-    HIP_TRY(hipEventElapsedTime(&ms, e0, e1));
-    (void)hipEventDestroy(e0);
-    (void)hipEventDestroy(e1);
+    HIP_TRY(hipEventElapsedTime(&ms, e.ev[0], e.ev[1]));
     *ms_per_call = ms / iters;
     return rc;
 }
@@ -509,29 +525,25 @@ int rof_aggregate_launch_times(const rof_layout *L, const void *x, int x_dtype, 
     hipStream_t st = (hipStream_t)stream;
     // each iteration times [launch 1 + launch 2] and then [launch 2 alone]; launch 2 alone is a
     // complete run because launch 1's rows are still in the workspace
-    hipEvent_t e0, e1, e2;
-    HIP_TRY(hipEventCreate(&e0));
-    HIP_TRY(hipEventCreate(&e1));
-    HIP_TRY(hipEventCreate(&e2));
+    EventSet e;
+    int rc = e.create(3);
+    if (rc) return rc;
     double both = 0.0, second = 0.0;
-    int rc = aggregate_with(L, x, x_dtype, ldx, out, ldo, feat, normalized, ep, workspace, workspace_bytes, st, 3);
+    rc = aggregate_with(L, x, x_dtype, ldx, out, ldo, feat, normalized, ep, workspace, workspace_bytes, st, 3);
     for (int i = 0; i < iters && rc == ROF_OK; ++i) {
-        HIP_TRY(hipEventRecord(e0, st));
+        HIP_TRY(hipEventRecord(e.ev[0], st));
         rc = aggregate_with(L, x, x_dtype, ldx, out, ldo, feat, normalized, ep, workspace, workspace_bytes, st, 3);
-        HIP_TRY(hipEventRecord(e1, st));
+        HIP_TRY(hipEventRecord(e.ev[1], st));
         if (rc == ROF_OK)
             rc = aggregate_with(L, x, x_dtype, ldx, out, ldo, feat, normalized, ep, workspace, workspace_bytes, st, 2);
-        HIP_TRY(hipEventRecord(e2, st));
-        HIP_TRY(hipEventSynchronize(e2));
+        HIP_TRY(hipEventRecord(e.ev[2], st));
+        HIP_TRY(hipEventSynchronize(e.ev[2]));
         float a = 0.f, b = 0.f;
-        HIP_TRY(hipEventElapsedTime(&a, e0, e1));
-        HIP_TRY(hipEventElapsedTime(&b, e1, e2));
+        HIP_TRY(hipEventElapsedTime(&a, e.ev[0], e.ev[1]));
+        HIP_TRY(hipEventElapsedTime(&b, e.ev[1], e.ev[2]));
         both += a;
         second += b;
     }
-    (void)hipEventDestroy(e0);
-    (void)hipEventDestroy(e1);
-    (void)hipEventDestroy(e2);
     ms_launch[1] = (float)(second / iters);
     ms_launch[0] = (float)((both - second) / iters);
     return rc;

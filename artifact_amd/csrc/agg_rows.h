@@ -22,7 +22,8 @@
 
 namespace rofk {
 
-// process-wide launch tuning (rof_set_xcd_run, rof_set_lds_pad); defined in agg_kernels.hip
+// process-wide launch tuning of the benchmark interface (rof_set_xcd_run, rof_set_lds_pad in rof_bench.h);
+// defined in agg_kernels.hip
 extern int g_xcd_run_a, g_xcd_run_b;
 extern int g_lds_pad;   // bytes of unused LDS requested per workgroup: caps the workgroups resident per CU
 
@@ -42,7 +43,7 @@ struct AggArgs {
     int32_t n_wave, n_tasks;
     int32_t n_blocks;          // logical workgroups
     int32_t xcd_run;           // consecutive logical workgroups kept on one XCD
-    int32_t vec_store;         // output rows allow aligned 16-byte stores
+    int32_t vec_store;         // output rows start on 4-byte boundaries: whole-vector stores
     const float *bias;         // destination-row launch only: added to every output row (null: none)
     int32_t relu;              // destination-row launch only: clamp the output at zero
     int32_t out_bf16;          // destination-row launch only: store bf16 (round to nearest even)
@@ -59,30 +60,19 @@ __device__ __forceinline__ uint32_t rof_bf16_bits(float f) {
 // Row gathers a lane group keeps in flight.  Measured on MI355X with all eight wave slots per SIMD
 // occupied: 2 beats 4 by ~10 % on the miss-dominated workloads (more outstanding gathers per CU slow the
 // L1/L2 miss path down) and loses ~2 % where gathers hit in L2; 8 loses everywhere.
-#ifndef ROF_UNROLL
-#define ROF_UNROLL 2
-#endif
-#ifndef ROF_MIN_BLOCKS
-#define ROF_MIN_BLOCKS 1
-#endif
+constexpr int kGathersInFlight = 2;
 constexpr int kWavesPerBlock = 4;
 constexpr int kXcds = 8;
 
 template <typename XT, int VEC>
 struct RowLoad;
 
-#ifdef ROF_NT_LOADS
-#define ROF_LD16(T, p) __builtin_nontemporal_load(reinterpret_cast<const T *>(p))
-#else
 #define ROF_LD16(T, p) (*reinterpret_cast<const T *>(p))
-#endif
 // 16-byte vectors that only promise 4-byte alignment: gfx950 executes global_load_dwordx4 at any dword
 // address, so packed rows (e.g. 47 floats = 188 bytes) are gathered with the same instruction as padded ones
 typedef float rof_f4 __attribute__((ext_vector_type(4), aligned(4)));
 typedef unsigned int rof_u4 __attribute__((ext_vector_type(4), aligned(4)));
-// naturally aligned vectors for the output stores
-typedef float rof_f4s __attribute__((ext_vector_type(4)));
-typedef unsigned int rof_u2 __attribute__((ext_vector_type(2)));
+typedef unsigned int rof_u2s __attribute__((ext_vector_type(2), aligned(4)));
 
 template <>
 struct RowLoad<float, 4> {
@@ -153,7 +143,7 @@ __device__ __forceinline__ void gather_sum(const char *xb, uint32_t xld, const c
                                            const float *__restrict__ w, int32_t beg, int32_t end, int lane, int sub,
                                            int li, bool act, float (&acc)[VEC]) {
     constexpr int G = 64 / LPR;             // lane groups per wavefront; lanes >= G*LPR stay idle
-    constexpr int U = LPR >= ROF_UNROLL ? ROF_UNROLL : LPR;   // row gathers in flight per lane group
+    constexpr int U = LPR >= kGathersInFlight ? kGathersInFlight : LPR;   // row gathers in flight per lane group
     constexpr int CH = WAVE ? G * LPR : LPR;   // entries fetched per step by the wave / by the lane group
     static_assert(LPR % U == 0, "the unroll factor must divide the lanes per row");
     const bool idle = (G * LPR < 64) && lane >= G * LPR;
@@ -230,7 +220,7 @@ __device__ __forceinline__ void gather_sum(const char *xb, uint32_t xld, const c
 // hence large graphs).  (A run-time switch between the two kinds of store does
 // not survive the optimiser, which merges the two stores into an ordinary one.)
 template <typename XT, int VEC, int LPR, int PHASE, bool OFF32>
-__global__ __launch_bounds__(256, ROF_MIN_BLOCKS) void rof_rows_kernel(AggArgs a) {
+__global__ __launch_bounds__(256) void rof_rows_kernel(AggArgs a) {
     constexpr int G = 64 / LPR;
     // XCD-aware renumbering: the hardware deals workgroup ids round-robin to the 8 XCDs; give each
     // XCD runs of `xcd_run` consecutive logical workgroups instead of every 8th one.
@@ -352,18 +342,22 @@ __global__ __launch_bounds__(256, ROF_MIN_BLOCKS) void rof_rows_kernel(AggArgs a
                 }
             }
             // A large output is not read again before the caches have turned over, so its rows are written as
-            // streaming stores (`nt`): they then do not push feature rows out of L2 and the Infinity Cache.  Whole
-            // 16-byte pieces only: element-wise streaming stores of packed rows are far slower than ordinary ones.
+            // streaming stores (`nt`): they then do not push feature rows out of L2 and the Infinity Cache.
+            // Every lane stores whole 16-byte pieces (8-byte for bf16 output) wherever the piece starts on a 4-byte
+            // boundary -- gfx950 executes global_store_dwordx4 at any dword address, like the loads -- so packed rows
+            // (47 floats = 188 bytes) are written as one contiguous burst per row.  The lane that was shifted back
+            // to stay inside the row rewrites `skip` elements of its neighbour's piece with the same bits (both
+            // lanes sum the same entries in the same order).
             constexpr bool stream = PHASE == 2;
             if (PHASE >= 1 && a.out_bf16) {
                 uint16_t *o = reinterpret_cast<uint16_t *>(a.out) + at;
-                if (VEC >= 4 && a.vec_store && skip == 0) {
+                if (VEC >= 4 && a.vec_store && (at & 1) == 0) {
 #pragma unroll
                     for (int k = 0; k < VEC; k += 4) {
-                        const rof_u2 t = {rof_bf16_bits(r[k]) | (rof_bf16_bits(r[k + 1]) << 16),
-                                          rof_bf16_bits(r[k + 2]) | (rof_bf16_bits(r[k + 3]) << 16)};
-                        if (stream) __builtin_nontemporal_store(t, reinterpret_cast<rof_u2 *>(o + k));
-                        else *reinterpret_cast<rof_u2 *>(o + k) = t;
+                        const rof_u2s t = {rof_bf16_bits(r[k]) | (rof_bf16_bits(r[k + 1]) << 16),
+                                           rof_bf16_bits(r[k + 2]) | (rof_bf16_bits(r[k + 3]) << 16)};
+                        if (stream) __builtin_nontemporal_store(t, reinterpret_cast<rof_u2s *>(o + k));
+                        else *reinterpret_cast<rof_u2s *>(o + k) = t;
                     }
                 } else {
 #pragma unroll
@@ -372,12 +366,12 @@ __global__ __launch_bounds__(256, ROF_MIN_BLOCKS) void rof_rows_kernel(AggArgs a
                 }
             } else {
                 float *o = reinterpret_cast<float *>(a.out) + at;
-                if (VEC >= 4 && a.vec_store && skip == 0) {
+                if (VEC >= 4 && a.vec_store) {
 #pragma unroll
                     for (int k = 0; k < VEC; k += 4) {
-                        const rof_f4s t = {r[k], r[k + 1], r[k + 2], r[k + 3]};
-                        if (stream) __builtin_nontemporal_store(t, reinterpret_cast<rof_f4s *>(o + k));
-                        else *reinterpret_cast<rof_f4s *>(o + k) = t;
+                        const rof_f4 t = {r[k], r[k + 1], r[k + 2], r[k + 3]};
+                        if (stream) __builtin_nontemporal_store(t, reinterpret_cast<rof_f4 *>(o + k));
+                        else *reinterpret_cast<rof_f4 *>(o + k) = t;
                     }
                 } else {
 #pragma unroll

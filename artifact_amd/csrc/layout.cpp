@@ -10,6 +10,7 @@
 //       descending id, which keeps consecutive gathers close in memory.
 #include <algorithm>
 #include <functional>
+#include <memory>
 #include <cstdint>
 #include <cstdlib>
 #include <cstring>
@@ -304,8 +305,8 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     return ROF_OK;
 }
 
-rof_layout *new_layout(int32_t n, int ps) {
-    rof_layout *L = new (std::nothrow) rof_layout;
+std::unique_ptr<rof_layout> new_layout(int32_t n, int ps) {
+    std::unique_ptr<rof_layout> L(new (std::nothrow) rof_layout);
     if (!L) return nullptr;
     L->n = n;
     L->part_size = ps;
@@ -345,13 +346,12 @@ void canonical_from_unique(rof_layout *L, const int32_t *src, const int32_t *spt
     }
 }
 
-int finish(rof_layout *L, const rof_layout_opts *opts, rof_layout **out) {
-    int st = build_schedule(L, opts);
-    if (st) {
-        delete L;
-        return st;
-    }
-    *out = L;
+// Takes ownership: the layout is released on every path that does not hand it to the caller, including
+// an allocation failure thrown while the schedule is built.
+int finish(std::unique_ptr<rof_layout> L, const rof_layout_opts *opts, rof_layout **out) {
+    int st = build_schedule(L.get(), opts);
+    if (st) return st;
+    *out = L.release();
     return ROF_OK;
 }
 
@@ -367,9 +367,9 @@ int rof_layout_from_v2(const int32_t *ucol, const int32_t *uptr, const int32_t *
     if ((ne && !ucol) || (nd && !dcol)) return ROF_ERR_ARG;
     if (!ids_ok(ucol, ne, n) || !ids_ok(dcol, nd, n)) return ROF_ERR_RANGE;
     try {
-        rof_layout *L = new_layout(n, part_size);
+        std::unique_ptr<rof_layout> L = new_layout(n, part_size);
         if (!L) return ROF_ERR_ALLOC;
-        canonical_from_unique(L, ucol, uptr, dptr, dcol, U);
+        canonical_from_unique(L.get(), ucol, uptr, dptr, dcol, U);
         int64_t G = (int64_t)L->group_ptr.size() - 1;
         bool groups_first = true;
         for (int64_t w = 0; w < U && groups_first; ++w) {
@@ -377,7 +377,7 @@ int rof_layout_from_v2(const int32_t *ucol, const int32_t *uptr, const int32_t *
             if ((w < G) != (cnt >= 2) || cnt == 0) groups_first = false;
         }
         L->canonical = groups_first && v2_is_canonical(uptr, dptr, dcol, U, part_size, G);
-        return finish(L, opts, out);
+        return finish(std::move(L), opts, out);
     } catch (const std::bad_alloc &) {
         return ROF_ERR_ALLOC;
     }
@@ -394,7 +394,7 @@ int rof_layout_from_v1(const int32_t *col, const int32_t *pptr, const int32_t *p
     if (!ids_ok(col, ne, n) || !ids_ok(ccol, nc, n) || !ids_ok(p2n, parts, n)) return ROF_ERR_RANGE;
     if (!ids_ok(flag, parts, cache_num + 1)) return ROF_ERR_RANGE;
     try {
-        rof_layout *L = new_layout(n, part_size);
+        std::unique_ptr<rof_layout> L = new_layout(n, part_size);
         if (!L) return ROF_ERR_ALLOC;
         // groups = cache rows (reuse_conv_kernel.cu:431-440); consumers = nodes of the flagged parts
         // (cu:523-531), which come in ascending node order because part2Node is non-decreasing
@@ -431,7 +431,7 @@ int rof_layout_from_v1(const int32_t *col, const int32_t *pptr, const int32_t *p
         for (int64_t g = 0; g < cache_num; ++g)
             if (L->group_dst_ptr[g + 1] - L->group_dst_ptr[g] < 2) ok = false;
         L->canonical = ok;
-        return finish(L, opts, out);
+        return finish(std::move(L), opts, out);
     } catch (const std::bad_alloc &) {
         return ROF_ERR_ALLOC;
     }
@@ -445,7 +445,7 @@ int rof_layout_from_parts(const int32_t *col, const int32_t *pptr, const int32_t
     if (ne && !col) return ROF_ERR_ARG;
     if (!ids_ok(col, ne, n) || !ids_ok(p2n, parts, n)) return ROF_ERR_RANGE;
     try {
-        rof_layout *L = new_layout(n, part_size);
+        std::unique_ptr<rof_layout> L = new_layout(n, part_size);
         if (!L) return ROF_ERR_ALLOC;
         L->group_ptr.assign(1, 0);
         L->group_dst_ptr.assign(1, 0);
@@ -461,7 +461,7 @@ int rof_layout_from_parts(const int32_t *col, const int32_t *pptr, const int32_t
         }
         L->e_orig = ne;
         L->canonical = true;
-        return finish(L, opts, out);
+        return finish(std::move(L), opts, out);
     } catch (const std::bad_alloc &) {
         return ROF_ERR_ALLOC;
     }

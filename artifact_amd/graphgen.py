@@ -54,19 +54,43 @@ def _rmat_pairs(rng, scale, m, a, b, c):
     return u, v
 
 
-def rmat_csr(num_nodes, avg_degree, seed, a=0.57, b=0.19, c=0.19, self_loops=False):
+def rmat_csr(num_nodes, avg_degree, seed, a=0.57, b=0.19, c=0.19, self_loops=False, distinct_pairs=False):
     """R-MAT(a,b,c,d) graph on `num_nodes` ids inside a 2^ceil(log2 N) id space.
 
     Draws N*avg_degree/2 undirected pairs; pairs with an endpoint >= N are dropped and
     the draw is topped up until that many in-range pairs exist (matters only when N is
-    not a power of two).
+    not a power of two).  With `distinct_pairs` the draw goes on until that many *distinct*
+    undirected pairs (no self pairs) remain after de-duplication, so the stored graph has
+    exactly N*avg_degree directed edges (the 2.4 M-node workload is specified by its edge
+    count after symmetrisation, the power-of-two ones by the number of pairs drawn).
     """
     rng = np.random.Generator(np.random.PCG64(seed))
     scale = int(np.ceil(np.log2(num_nodes)))
     want = int(num_nodes * avg_degree // 2)
+    oversample = 1 if (1 << scale) == num_nodes else 1.6
+    if distinct_pairs:
+        n = np.int64(num_nodes)
+        keys = np.empty(0, dtype=np.int64)      # distinct pairs so far, as min*N+max, ascending
+        yield_ = 0.7 / oversample               # distinct new pairs per draw, re-estimated after every batch
+        while len(keys) < want:
+            short = want - len(keys)
+            # large batches aim 3 % below the target so that only a small last batch has to be trimmed
+            m = max(4096, int((short * 0.97 if short > 100000 else short * 1.5) / yield_))
+            u, v = _rmat_pairs(rng, scale, m, a, b, c)
+            ok = (u < num_nodes) & (v < num_nodes) & (u != v)
+            k = np.minimum(u[ok], v[ok]) * n + np.maximum(u[ok], v[ok])
+            del u, v, ok
+            fresh = np.setdiff1d(k, keys)       # sorted, distinct
+            yield_ = max(len(fresh), 1) / m
+            if len(fresh) > short:              # overshoot: keep the pairs that were drawn first
+                f2, first = np.unique(k, return_index=True)
+                first = first[np.isin(f2, fresh, assume_unique=True)]
+                fresh = fresh[np.argsort(first, kind="stable")[:short]]
+            keys = np.union1d(keys, fresh)
+        return csr_from_pairs(keys // n, keys % n, num_nodes, self_loops)
     us, vs, have = [], [], 0
     while have < want:
-        m = max(1024, int((want - have) * 1.05 * (1 if (1 << scale) == num_nodes else 1.6)))
+        m = max(1024, int((want - have) * 1.05 * oversample))
         u, v = _rmat_pairs(rng, scale, m, a, b, c)
         ok = (u < num_nodes) & (v < num_nodes)
         u, v = u[ok][: want - have], v[ok][: want - have]
@@ -137,7 +161,9 @@ WORKLOADS = {
     "c2": dict(kind="rmat", num_nodes=1 << 18, avg_degree=14, self_loops=True, seed=1002, dims=(128, 256, 40)),
     "c3": dict(kind="sbm", num_blocks=256, block_size=4096, deg_in=24, deg_out=2, self_loops=False, seed=1003,
                dims=(64, 64)),
-    "c4": dict(kind="rmat", num_nodes=2_400_000, avg_degree=26, self_loops=False, seed=1004, dims=(100, 47)),
+    # specified by its edge count after symmetrisation (~62 M directed): the draw is topped up after de-duplication
+    "c4": dict(kind="rmat", num_nodes=2_400_000, avg_degree=26, self_loops=False, seed=1004, dims=(100, 47),
+               distinct_pairs=True),
     "c5": dict(kind="rmat", num_nodes=1 << 22, avg_degree=32, self_loops=True, seed=1005, dims=(256, 256)),
     # planted reuse (see planted_reuse_csr): 2^20 nodes, 12 shared anchors + ~4 random neighbours per member
     "hr": dict(kind="planted", num_nodes=1 << 20, set_size=12, members_per_set=64, extra_degree=4, seed=1006,
@@ -151,7 +177,8 @@ def make_workload(name, scale_down=0):
     w = dict(WORKLOADS[name])
     if w["kind"] == "rmat":
         n = max(64, w["num_nodes"] >> scale_down)
-        return rmat_csr(n, w["avg_degree"], w["seed"], self_loops=w["self_loops"])
+        return rmat_csr(n, w["avg_degree"], w["seed"], self_loops=w["self_loops"],
+                        distinct_pairs=w.get("distinct_pairs", False))
     if w["kind"] == "planted":
         n = max(512, w["num_nodes"] >> scale_down)
         return planted_reuse_csr(n, w["set_size"], w["members_per_set"], w["extra_degree"], w["seed"])

@@ -347,9 +347,9 @@ class ROF_GCNConv(torch.nn.Module):
         else:
             self.register_parameter("bias", None)
         self.reuse_size = kwargs.get("reuse_size", 0)
-        # scratch of the v1 kernels; a Parameter upstream, so it is kept one here (state_dict parity)
-        self.part_result_cache = torch.nn.Parameter(torch.empty(max(self.reuse_size, 0), out_channels + 1),
-                                                    requires_grad=False)
+        # scratch of the v1 kernels; a plain Parameter upstream (reuse_conv.py:113), so it is one here: it shows
+        # up in state_dict() and in parameters() (an optimizer skips it, it never receives a gradient)
+        self.part_result_cache = torch.nn.Parameter(torch.empty(max(self.reuse_size, 0), out_channels + 1))
         self.dimWorker = kwargs.get("dimWorker", 0)
         if self.dimWorker == 0:
             self.dimWorker = 32 if out_channels > 32 else out_channels   # reuse_conv.py:115-120
@@ -365,6 +365,12 @@ class ROF_GCNConv(torch.nn.Module):
         if kwargs.get("compute_dtype", None) not in (None, "bf16", torch.bfloat16, "fp32", torch.float32):
             raise ValueError("compute_dtype must be None or 'bf16'")
         self.out_bf16 = self.bf16 and kwargs.get("out_dtype", None) in ("bf16", torch.bfloat16)
+        if self.kernel_type == "ROF_v1" and not self.bf16 and (self.aggregate_first or "fuse_epilogue" in kwargs):
+            # only upstream's literal sequence fills the caller's part_result_cache, so that is what ROF_v1 runs
+            import warnings
+
+            warnings.warn("ROF_GCNConv(kernel_type='ROF_v1') always runs upstream's sequence (update, aggregate, "
+                          "bias pass): `order` and `fuse_epilogue` have no effect; use kernel_type='ROF_v2' for them")
         self.reset_parameters()
 
     def reset_parameters(self):

@@ -4,18 +4,28 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4] [--part-size 3]
 
 A step is one aggregation layer: out = D^-1/2 A D^-1/2 (XW) evaluated through the reuse plan on a
-feature matrix that is already resident in HBM (the dense update X*W is not part of the step).
-The default workload is the 2.4M-node R-MAT graph with aggregated width 47.  Prints one JSON line:
-GEdges/s (original edge count / time), the HBM roofline of the destination-row launch measured with
-HIP events on the launch stream, the same kernels with reuse disabled, and a CPU baseline (the
-oracle's destination-parallel SpMM) timed on this machine's host cores.
+feature matrix that is already resident in HBM (the dense update X*W is not part of the step), with
+the operands laid out as the operator API lays them out: the update's rows in a stride that is a
+multiple of four floats, the output a packed [N, F] tensor.  The default workload is the 2.4M-node
+R-MAT graph with aggregated width 47.  Prints one JSON line: GEdges/s (original edge count / time);
+the HBM roofline of the destination-row launch -- its duration measured with HIP events on the launch
+stream, its HBM-side bytes measured by running this same script under `rocprofv3 --pmc` in child
+processes (FETCH_SIZE, WRITE_SIZE, TCC hits/misses; scaled by a copy of known size) before this
+process touches the GPU; the same kernels with reuse disabled; part sizes 2..5; and a CPU baseline
+(the oracle's destination-parallel SpMM) timed on this machine's host cores.
 """
 from __future__ import annotations
 
 import argparse
+import collections
+import csv
+import glob
 import json
 import os
+import shutil
+import subprocess
 import sys
+import tempfile
 import time
 
 import numpy as np
@@ -26,18 +36,18 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 
-# HBM-side bytes per launch (partial-sum launch, destination-row launch) measured offline with rocprofv3
-# (FETCH_SIZE x 2.0 + WRITE_SIZE, the factors coming from a 1 GiB copy of known size).  Counters cannot be read
-# from inside this script, so the figures are carried here and reported only for the configurations they were
-# measured on: (workload, part size, width) with default layout options.
-PROFILED_TRAFFIC_BYTES = {("c4", 3, 47): (1.76e9, 6.12e9), ("c5", 3, 256): (24.93e9, 23.75e9),
-                          ("c3", 3, 64): (None, 1.31e9)}
+# HBM-side bytes per launch (partial-sum launch, destination-row launch) and TCC hit rates from the committed
+# rocprofv3 summaries under profiles/ (FETCH_SIZE x its copy-calibrated factor + WRITE_SIZE).  Used only when the
+# live counter runs are switched off or fail, and only for the configurations they were measured on:
+# (workload, part size, width, packed output) with default layout options; the JSON then says "offline profile".
+PROFILED_TRAFFIC = {}
+COPY_BYTES = 1 << 30   # size of the calibration copy the counter runs include
 
 DESCR = {
     "c1": "c1: R-MAT 2^14 nodes, avg deg 16, self loops, GCN sym-norm, F=32, fp32",
     "c2": "c2: R-MAT 2^18 nodes, avg deg 14, self loops, GCN sym-norm, F=256, fp32",
     "c3": "c3: SBM 2^20 nodes (256 blocks), deg 24+2, GIN sum aggregation, F=64, fp32",
-    "c4": "c4: R-MAT 2.4M nodes, ~60M directed edges, GCN sym-norm, aggregated width 47, fp32",
+    "c4": "c4: R-MAT 2.4M nodes, 62.4M directed edges, GCN sym-norm, aggregated width 47, fp32",
     "c5": "c5: R-MAT 2^22 nodes, avg deg 32, self loops, GCN sym-norm, F=256, bf16 in / fp32 accumulate",
     "hr": "hr: planted-reuse graph 2^20 nodes (12 shared anchors + ~4 random neighbours per node), GCN, F=64, fp32",
 }
@@ -203,6 +213,174 @@ def model_step(name, d, n, ps, deg, dev, timed):
     return res
 
 
+def build_layouts(d, n, ps, lpr, in_bytes, args, want_forced=True):
+    """(reuse, reuse-disabled, forced-sharing or None) layouts of one plan, not yet uploaded."""
+    from artifact_amd.layout import Layout
+
+    v2 = (d["uniqpart_column_index"], d["uniqpart_pointers"], d["part2Node_ptr"], d["part2Node_col"], n, ps)
+    common = dict(hub_split=args.hub_split, segment=args.segment, lanes_per_row=lpr, entry_order=args.entry_order,
+                  tile_rows=args.tile_rows, elem_bytes=in_bytes)
+    reuse = Layout.from_v2(*v2, min_consumers=args.min_consumers, **common)
+    plain = Layout.from_v2(*v2, disable_reuse=True, **common)
+    # when the cost model folds every group back (the plan saves too little), also time the plan with its
+    # profitable groups forced to be shared, so the cost of the reuse machinery stays visible
+    forced = None
+    if want_forced and reuse.stats()["materialised_groups"] == 0 and len(d["index_picked"]) and not args.min_consumers:
+        forced = Layout.from_v2(*v2, min_consumers=3, **common)
+    return reuse, plain, forced
+
+
+def make_features(name, n, feat, bf16, dev):
+    """Feature rows as the dense update leaves them: N(0,1) fp32 (uniform(-1,1) -> bf16 for c5) in rows
+    allocated up to a multiple of 4 (8) elements.  Returns (view [n, feat], fp32 host copy, row stride)."""
+    import torch
+
+    from artifact_amd.graphgen import features
+
+    mult = 8 if bf16 else 4
+    ld = (feat + mult - 1) // mult * mult
+    x32 = features(n, feat, seed=2000 + (int(name[1]) if name[1].isdigit() else 6), kind="uniform" if bf16 else "normal")
+    xbuf = torch.zeros((n, ld), dtype=torch.bfloat16 if bf16 else torch.float32, device=dev)
+    xbuf[:, :feat] = torch.from_numpy(x32).to(dev)
+    x = xbuf[:, :feat]
+    if bf16:
+        x32 = x.to(torch.float32).cpu().numpy()
+    return x, x32, ld
+
+
+def traffic_child(args):
+    """Body of a counter run (this script under `rocprofv3 --pmc ...`): the default layout of the workload, one
+    calibration copy of COPY_BYTES and a few aggregations, nothing else on the GPU."""
+    import ctypes
+
+    import torch
+
+    from artifact_amd import _lib
+    from artifact_amd.layout import lanes_per_row
+
+    L = _lib.lib()
+    dev = torch.device("cuda:0")
+    name, ps = args.workload, args.part_size
+    feat = args.feat or FEAT[name]
+    bf16, normalized = name == "c5", name != "c3"
+    d, _, _ = load_or_build(name, ps, args.cache_dir)
+    n = len(d["indptr"]) - 1
+    reuse, _, _ = build_layouts(d, n, ps, lanes_per_row(feat, bf16), 2 if bf16 else 4, args, want_forced=False)
+    reuse.upload()
+    if normalized:
+        reuse.set_degrees(torch.from_numpy(np.diff(d["indptr"]).astype(np.float32)).to(dev))
+    x, _, ld = make_features(name, n, feat, bf16, dev)
+    pad = args.padded_output and ld != feat
+    out = torch.empty((n, ld if pad else feat), dtype=torch.float32, device=dev)[:, :feat]
+    a = torch.empty(COPY_BYTES // 4, dtype=torch.float32, device=dev).normal_()
+    b = torch.empty_like(a)
+    torch.cuda.synchronize()
+    _lib.check(L.rof_device_copy(ctypes.c_void_p(b.data_ptr()), ctypes.c_void_p(a.data_ptr()), COPY_BYTES,
+                                 ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    for _ in range(4):
+        reuse.aggregate(x, normalized, out=out, feat_dim=feat, pad_columns=pad)
+    torch.cuda.synchronize()
+
+
+def measure_traffic(args, passthrough):
+    """HBM-side bytes per launch from rocprofv3 counter runs of this script (one counter set per run, as the
+    hardware collects them), started as child processes *before* this process initialises the GPU.
+    Returns a dict, or {"error": ...} when the profiler is missing or a run fails."""
+    prof = shutil.which("rocprofv3") or "/opt/rocm/bin/rocprofv3"
+    if not os.path.exists(prof):
+        return {"error": "rocprofv3 not found"}
+    tmp = tempfile.mkdtemp(prefix="rof_pmc_", dir="/tmp")
+    env = dict(os.environ, TMPDIR="/tmp")
+    per = {}     # (counter, phase) -> mean value per dispatch; phase 0 = partial-sum launch, 1 = destination rows
+    copy = {}    # counter -> value of the calibration copy
+    try:
+        for tag, counters in (("fetch", ["FETCH_SIZE"]), ("write", ["WRITE_SIZE"]), ("tcc", ["TCC_HIT_sum", "TCC_MISS_sum"])):
+            out_dir = os.path.join(tmp, tag)
+            cmd = ["timeout", "-s", "KILL", "240", prof, "--pmc", *counters, "-d", out_dir, "-o", "rof", "-f", "csv",
+                   "--", sys.executable, os.path.abspath(__file__), "--traffic-child", *passthrough]
+            log(f"[bench] counter run: {' '.join(cmd[4:])}")
+            r = subprocess.run(cmd, cwd="/tmp", env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, timeout=300)
+            files = glob.glob(os.path.join(out_dir, "**", "*counter_collection.csv"), recursive=True)
+            if r.returncode != 0 or not files:
+                return {"error": f"rocprofv3 --pmc {' '.join(counters)} failed (rc {r.returncode}): "
+                                 + r.stdout.decode(errors="replace")[-300:]}
+            acc = collections.defaultdict(list)
+            with open(files[0]) as f:
+                for row in csv.DictReader(f):
+                    k = row["Kernel_Name"]
+                    if "rof_copy_kernel" in k:
+                        copy[row["Counter_Name"]] = float(row["Counter_Value"])
+                    elif "rof_rows_kernel" in k:
+                        # template arguments <XT, VEC, LPR, PHASE, OFF32>: PHASE 0 is the partial-sum launch
+                        phase = int(k.split("<")[1].split(">")[0].split(",")[3])
+                        acc[(row["Counter_Name"], min(phase, 1))].append(float(row["Counter_Value"]))
+            for k, v in acc.items():
+                per[k] = sum(v) / len(v)
+    except (OSError, subprocess.SubprocessError, ValueError, KeyError, IndexError) as ex:
+        return {"error": f"counter runs failed: {ex!r}"[:300]}
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
+    if "FETCH_SIZE" not in copy or "WRITE_SIZE" not in copy or ("FETCH_SIZE", 1) not in per:
+        return {"error": "counter output lacks the expected kernels"}
+    # the counters report KiB; what they read for a copy of known size gives the factor that turns them into bytes
+    f_scale = COPY_BYTES / (copy["FETCH_SIZE"] * 1024.0)
+    w_scale = COPY_BYTES / (copy["WRITE_SIZE"] * 1024.0)
+    res = {"source": "live: this script under rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE / TCC_HIT_sum TCC_MISS_sum, "
+                     "one counter set per child process, mean per dispatch over 4 aggregations",
+           "fetch_scale": f_scale, "write_scale": w_scale, "launch": {}}
+    for phase in (0, 1):
+        if ("FETCH_SIZE", phase) not in per:
+            continue
+        rd = per[("FETCH_SIZE", phase)] * 1024.0 * f_scale
+        wr = per.get(("WRITE_SIZE", phase), 0.0) * 1024.0 * w_scale
+        hit, miss = per.get(("TCC_HIT_sum", phase)), per.get(("TCC_MISS_sum", phase))
+        res["launch"][phase] = {"read_bytes": rd, "written_bytes": wr, "bytes": rd + wr,
+                                "tcc_hit_rate": hit / (hit + miss) if hit is not None and miss else None,
+                                "tcc_miss_x_128B": miss * 128.0 if miss is not None else None}
+    return res
+
+
+def restrided(t):
+    """Copy of `t` whose row stride is a multiple of four floats (the alternative to gathering packed rows in
+    place that the backward figures compare against)."""
+    f = t.shape[1]
+    pad = (-f) % 4
+    if pad == 0:
+        return t
+    buf = t.new_empty(t.shape[0], f + pad)
+    buf[:, :f].copy_(t)
+    buf[:, f:].zero_()
+    return buf
+
+
+def part_size_sweep(name, sizes, have, n, e, x, deg, normalized, feat, lpr, in_bytes, args, out):
+    """ms / GEdges/s per aggregation for each part size (upstream's drivers default to 3 and 5:
+    ROF_evaluation/ROF_main.py:73, cuda/middle-rof.py:20), with what the plan picked and what it saves."""
+    rows = []
+    for ps in sizes:
+        d = have.get(ps) or load_or_build(name, ps, args.cache_dir)[0]
+        reuse, plain, forced = build_layouts(d, n, ps, lpr, in_bytes, args)
+        row = {"part_size": ps, "picked_parts": int(len(d["index_picked"]))}
+        for tag, lay in (("reuse", reuse), ("reuse_disabled", plain), ("reuse_forced", forced)):
+            if lay is None:
+                continue
+            lay.upload()
+            if normalized:
+                lay.set_degrees(deg)
+            lay.aggregate(x, normalized, out=out, feat_dim=feat)
+            ms = float(np.median([lay.aggregate_timed(x, 10, normalized, out=out, feat_dim=feat)[0] for _ in range(3)]))
+            st = lay.stats()
+            row[tag + "_ms"] = ms
+            if tag == "reuse":
+                row.update(GEdges_per_s=e / (ms * 1e-3) / 1e9, materialised_groups=st["materialised_groups"],
+                           plan_saved_gathers_frac=1.0 - len(d["uniqpart_column_index"]) / max(1, e))
+            if tag == "reuse_forced":
+                row["forced_saved_gathers_frac"] = 1.0 - (st["gathered_rows"] + st["partial_reads"] - st["hub_segments"]) / max(1, e)
+            lay.close()
+        rows.append(row)
+    return rows
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -213,15 +391,18 @@ def main():
     ap.add_argument("--feat", type=int, default=0, help="override the aggregated width")
     ap.add_argument("--cache-dir", default="/tmp/rof_bench_cache")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-traffic", action="store_true", help="skip the rocprofv3 counter runs (HBM-side bytes)")
+    ap.add_argument("--no-sweep", action="store_true", help="skip the part-size sweep 2..5")
+    ap.add_argument("--quick", action="store_true", help="only the headline timing: no counters, sweep, model step or CPU leg")
+    ap.add_argument("--traffic-child", action="store_true", help=argparse.SUPPRESS)
     ap.add_argument("--xcd-run", type=int, default=0, help="launch tuning: workgroups per XCD run, destination rows")
     ap.add_argument("--xcd-run-partial", type=int, default=1, help="same for the partial-sum launches")
-    ap.add_argument("--packed-output", action="store_true",
-                    help="store the output as packed [N, feat] rows instead of rows of the input's stride")
+    ap.add_argument("--padded-output", action="store_true",
+                    help="store the output in rows of the input's stride (47 floats in rows of 48, rof_epilogue."
+                         "pad_columns) instead of the packed [N, feat] tensor the operator API returns")
     ap.add_argument("--hub-split", type=int, default=0, help="layout tuning: rows longer than this are segmented")
     ap.add_argument("--segment", type=int, default=0, help="layout tuning: entries per segment")
     ap.add_argument("--min-consumers", type=int, default=0, help="layout tuning: share groups with >= this many consumers")
-    ap.add_argument("--fold-sources", type=int, default=0,
-                    help="experiment: gather from source id %% K instead (all gathers hit cache); changes the result")
     ap.add_argument("--lds-pad", type=int, default=-1, help="launch tuning: unused LDS bytes per workgroup")
     ap.add_argument("--entry-order", default="descending", choices=["descending", "plan", "ascending"],
                     help="layout tuning: order of the gathered rows inside a task")
@@ -231,17 +412,41 @@ def main():
                          "greedy that upstream sketches")
     ap.add_argument("--hubs", type=int, default=16384, help="--search hub: number of hub sources")
     ap.add_argument("--block", type=int, default=8, help="--search hub: hubs per block (= part size of the plan)")
-    ap.add_argument("--calibrate-copy", action="store_true",
-                    help="also run one 1 GiB rof_copy_kernel launch (reference transfer for profiler byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: every machine of this build has a single MI355X and the aggregation "
                  "path has no multi-GPU part; run with --gpus 1")
+    if args.traffic_child:
+        return traffic_child(args)
+    if args.quick:
+        args.no_traffic = args.no_sweep = args.no_cpu_baseline = True
 
+    name, ps = args.workload, args.part_size
+    feat = args.feat or FEAT[name]
+    normalized = name != "c3"
+    bf16 = name == "c5"
+    default_opts = (not (args.hub_split or args.segment or args.min_consumers or args.tile_rows or args.xcd_run
+                         or args.xcd_run_partial != 1 or args.lds_pad >= 0)
+                    and args.search == "upstream" and args.entry_order == "descending")
+
+    # ---- host side first: graph and plan (cached on disk), then the counter runs in child processes; this
+    # process has not touched the GPU yet.  (PyTorch is imported before librof.so is loaded so that both use the
+    # HIP runtime PyTorch brings; importing it does not initialise the device.)
     import torch
 
+    d, t_gen, t_plan = load_or_build(name, ps, args.cache_dir)
+    traffic = {"error": "switched off (--no-traffic / --quick) or non-default options"}
+    if not args.no_traffic and default_opts:
+        passthrough = ["--workload", name, "--part-size", str(ps), "--cache-dir", args.cache_dir]
+        if args.feat:
+            passthrough += ["--feat", str(args.feat)]
+        if args.padded_output:
+            passthrough += ["--padded-output"]
+        traffic = measure_traffic(args, passthrough)
+        if "error" in traffic:
+            log(f"[bench] live counters unavailable: {traffic['error']}")
+
     from artifact_amd import _lib
-    from artifact_amd.graphgen import features
     from artifact_amd.layout import Layout, lanes_per_row
 
     L = _lib.lib()   # raises if the HIP library is missing
@@ -252,12 +457,7 @@ def main():
     if args.lds_pad >= 0:
         _lib.check(L.rof_set_lds_pad(args.lds_pad))
     dev = torch.device("cuda:0")
-    name, ps = args.workload, args.part_size
-    feat = args.feat or FEAT[name]
-    normalized = name != "c3"
-    bf16 = name == "c5"
 
-    d, t_gen, t_plan = load_or_build(name, ps, args.cache_dir)
     indptr, indices = d["indptr"], d["indices"]
     n, e = len(indptr) - 1, len(indices)
     if args.search == "hub":
@@ -283,42 +483,20 @@ def main():
             f"candidates")
     deg = torch.from_numpy(np.diff(indptr).astype(np.float32)).to(dev)
 
-    # features: N(0,1) fp32 (uniform(-1,1) -> bf16 for c5), rows padded to a multiple of 4 (8) elements
-    mult = 8 if bf16 else 4
-    ld = (feat + mult - 1) // mult * mult
-    x32 = features(n, feat, seed=2000 + (int(name[1]) if name[1].isdigit() else 6), kind="uniform" if bf16 else "normal")
-    xbuf = torch.zeros((n, ld), dtype=torch.bfloat16 if bf16 else torch.float32, device=dev)
-    xbuf[:, :feat] = torch.from_numpy(x32).to(dev)
-    x = xbuf[:, :feat]
-    if bf16:
-        x32 = x.to(torch.float32).cpu().numpy()
+    x, x32, ld = make_features(name, n, feat, bf16, dev)
     in_bytes = 2 if bf16 else 4
-
     lpr = lanes_per_row(feat, bf16)
-    if args.fold_sources:
-        d["uniqpart_column_index"] = (d["uniqpart_column_index"] % args.fold_sources).astype(np.uint32)
     t0 = time.time()
-    reuse = Layout.from_v2(d["uniqpart_column_index"], d["uniqpart_pointers"], d["part2Node_ptr"], d["part2Node_col"],
-                           n, ps, hub_split=args.hub_split, segment=args.segment, lanes_per_row=lpr,
-                           min_consumers=args.min_consumers, entry_order=args.entry_order, tile_rows=args.tile_rows, elem_bytes=in_bytes)
-    plain = Layout.from_v2(d["uniqpart_column_index"], d["uniqpart_pointers"], d["part2Node_ptr"], d["part2Node_col"],
-                           n, ps, disable_reuse=True, hub_split=args.hub_split, segment=args.segment, lanes_per_row=lpr,
-                           entry_order=args.entry_order, tile_rows=args.tile_rows, elem_bytes=in_bytes)
+    reuse, plain, forced = build_layouts(d, n, ps, lpr, in_bytes, args)
     t_layout = time.time() - t0
-    # when the cost model folds every group back (the plan saves too little), also time the plan with its
-    # profitable groups forced to be shared, so the cost of the reuse machinery stays visible
-    forced = None
-    if reuse.stats()["materialised_groups"] == 0 and len(d["index_picked"]) and not args.min_consumers:
-        forced = Layout.from_v2(d["uniqpart_column_index"], d["uniqpart_pointers"], d["part2Node_ptr"],
-                                d["part2Node_col"], n, ps, hub_split=args.hub_split, segment=args.segment,
-                                lanes_per_row=lpr, min_consumers=3, entry_order=args.entry_order, tile_rows=args.tile_rows, elem_bytes=in_bytes)
     for lay in (reuse, plain) + ((forced,) if forced else ()):
         lay.upload()
         if normalized:
             lay.set_degrees(deg)
-    # output rows as wide as the input rows (47 floats live in rows of 48) unless --packed-output: the kernel may
-    # then store whole 16-byte pieces (rof_epilogue.pad_columns); columns 0 .. feat-1 are the same either way
-    pad = (not args.packed_output) and ld != feat
+    # The output is the packed [N, feat] tensor the operator returns (reuse_conv_kernel.cu:303,1000).  With
+    # --padded-output it has rows as wide as the input rows (47 floats in rows of 48, rof_epilogue.pad_columns);
+    # columns 0 .. feat-1 are the same either way.
+    pad = args.padded_output and ld != feat
     ldo = ld if pad else feat
     out = torch.empty((n, ldo), dtype=torch.float32, device=dev)[:, :feat]
     out_plain = torch.empty((n, ldo), dtype=torch.float32, device=dev)[:, :feat]
@@ -366,7 +544,7 @@ def main():
         forced_info = {"min_consumers": 3, "event_ms": float(np.median(ev_f)),
                        "speedup_vs_reuse_disabled": float(np.median(ev_p2) / np.median(ev_f)),
                        "materialised_groups": fs["materialised_groups"],
-                       "saved_gathers_frac": 1.0 - fs["gathered_rows"] / max(1, e),
+                       "saved_gathers_frac": 1.0 - (fs["gathered_rows"] + fs["partial_reads"] - fs["hub_segments"]) / max(1, e),
                        "max_abs_diff_vs_reuse_disabled": float((out_f - out_plain).abs().max())}
         del out_f
     ms_a, ms_b = reuse.launch_times(x, max(5, args.steps // 2), normalized, out=out, feat_dim=feat, pad_columns=pad)
@@ -374,20 +552,23 @@ def main():
     torch.cuda.synchronize()
     max_diff = float((out - out_plain).abs().max())
 
-    # ---- the backward aggregation (same plan on the gradient, reuse_conv_kernel.cu:1021-1041): the gradient
-    # arrives packed [N, F]
     extra = {}
-    if not bf16:
-        from artifact_amd import ROF as rof_api
+    if not args.no_sweep and not args.feat and args.search == "upstream":
+        extra["part_size_sweep"] = part_size_sweep(name, (2, 3, 4, 5), {ps: d}, n, e, x, deg, normalized, feat, lpr,
+                                                   in_bytes, args, out_plain)
 
+    # ---- the backward aggregation (same plan on the gradient, reuse_conv_kernel.cu:1021-1041): the gradient
+    # arrives packed [N, F] and is gathered in place; the result is an intermediate and keeps padded rows
+    if not bf16 and not args.quick:
         grad = torch.randn((n, feat), device=dev)
+        gout = torch.empty((n, ld), dtype=torch.float32, device=dev)[:, :feat]
         ev0, ev1, ev2 = (torch.cuda.Event(enable_timing=True) for _ in range(3))
         t_pad, t_agg = [], []
         for _ in range(10):
             ev0.record()
-            gp = rof_api._restrided(grad)
+            gp = restrided(grad)
             ev1.record()
-            reuse.aggregate(gp, normalized, out=out_plain, feat_dim=feat)
+            reuse.aggregate(gp, normalized, out=gout, feat_dim=feat, pad_columns=True)
             ev2.record()
             torch.cuda.synchronize()
             t_pad.append(ev0.elapsed_time(ev1))
@@ -395,7 +576,7 @@ def main():
         t_packed = []
         for _ in range(10):
             ev0.record()
-            reuse.aggregate(grad, normalized, out=out_plain, feat_dim=feat)
+            reuse.aggregate(grad, normalized, out=gout, feat_dim=feat, pad_columns=True)
             ev1.record()
             torch.cuda.synchronize()
             t_packed.append(ev0.elapsed_time(ev1))
@@ -403,12 +584,12 @@ def main():
         # numbers are the alternative of re-striding the gradient to 16-byte rows first
         extra["backward_aggregation"] = {"packed_rows_ms": float(np.median(t_packed)),
                                          "restride_ms": float(np.median(t_pad)), "aggregate_ms": float(np.median(t_agg))}
-        del grad, gp
+        del grad, gp, gout
 
     # ---- continuity with the upstream micro-benchmark (ROF_evaluation/cuda/small-main.py:357-478): the whole
     # ROF.reuse_forward_v2 call, dense update included, 10 warm-ups + 100 runs, events on the current stream
     dims = {"c1": (32, 32), "c2": (128, 256), "c4": (100, 47)}.get(name)
-    if dims and not args.feat:
+    if dims and not args.feat and not args.quick:
         from artifact_amd import ROF as rof_api
         from artifact_amd.layout import LayoutFamily
 
@@ -420,7 +601,7 @@ def main():
                                                 layout=fam)[0]
         for _ in range(10):
             call()
-        ts = []
+        ts, tg = [], []
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         for _ in range(100):
             e0.record()
@@ -428,8 +609,16 @@ def main():
             e1.record()
             torch.cuda.synchronize()
             ts.append(e0.elapsed_time(e1))
+        for _ in range(20):
+            e0.record()
+            rof_api._update(xin, wgt)
+            e1.record()
+            torch.cuda.synchronize()
+            tg.append(e0.elapsed_time(e1))
         extra["whole_reuse_forward_v2"] = {"in_dim": dims[0], "out_dim": dims[1], "mean_ms": float(np.mean(ts)),
-                                           "std_ms": float(np.std(ts)), "median_ms": float(np.median(ts))}
+                                           "std_ms": float(np.std(ts)), "median_ms": float(np.median(ts)),
+                                           "dense_update_ms": float(np.median(tg)),
+                                           "minus_dense_update_ms": float(np.median(ts) - np.median(tg))}
         fam._by_lpr.clear()   # the layout is owned by this function, not by the family
         del xin, wgt
 
@@ -449,12 +638,14 @@ def main():
             ts.append(e0.elapsed_time(e1))
         return float(np.median(ts))
 
-    if normalized and not args.feat:
+    if normalized and not args.feat and not args.quick:
         bias_t = torch.randn(feat, device=dev)
         t_fused = timed(lambda: reuse.aggregate(x, True, out=out_plain, feat_dim=feat, bias=bias_t, relu=True))
         t_sep = timed(lambda: torch.relu_(reuse.aggregate(x, True, out=out_plain, feat_dim=feat).add_(bias_t)))
         extra["epilogue"] = {"fused_bias_relu_ms": t_fused, "separate_passes_ms": t_sep, "speedup": t_sep / t_fused}
-    if dims and not args.feat and not bf16:
+    if dims and not args.feat and not bf16 and not args.quick:
+        from artifact_amd import ROF as rof_api
+
         fin, fout = dims
         xin = torch.randn((n, fin), device=dev)
         wgt = torch.randn((fin, fout), device=dev)
@@ -488,31 +679,42 @@ def main():
 
     # ---- the workload's model step end to end (dense updates, bias, activation, backward where the workload has
     # one), upstream's sequence of separate passes against the fused layer; the aggregation layouts are shared
-    if not args.feat and name in MODEL_STEPS:
+    if not args.feat and name in MODEL_STEPS and not args.quick:
         extra["model_step"] = model_step(name, d, n, ps, deg, dev, timed)
-
-    if args.calibrate_copy:
-        import ctypes
-        a = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
-        b = torch.empty_like(a)
-        torch.cuda.synchronize()
-        _lib.check(L.rof_device_copy(ctypes.c_void_p(b.data_ptr()), ctypes.c_void_p(a.data_ptr()), a.numel() * 4,
-                                     ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
-        torch.cuda.synchronize()
-        del a, b
 
     st = reuse.stats()
     bytes_a, bytes_b = reuse.launch_bytes(feat, in_bytes)
     b_alg = reuse.algorithmic_bytes(feat, in_bytes)
     b_alg_plain = plain.algorithmic_bytes(feat, in_bytes)
     b_noreuse_model = e * (4 + feat * in_bytes) + n * (feat * 4 + 8)
-    achieved_b = bytes_b / (ms_b * 1e-3) / 1e9
-    default_opts = (not (args.hub_split or args.segment or args.min_consumers or args.fold_sources)
-                    and args.search == "upstream" and args.entry_order == "descending" and not args.tile_rows)
-    traffic = (PROFILED_TRAFFIC_BYTES.get((name, ps, feat), (None, None)) if default_opts and not args.packed_output
-               else (None, None))
-    achieved_a = bytes_a / (ms_a * 1e-3) / 1e9 if ms_a > 0 else 0.0
+    b_min = n * feat * in_bytes + 4 * e + n * feat * 4      # every feature row once, every column id, every output row
+    if "error" in traffic:
+        key = (name, ps, feat, not pad)
+        off = PROFILED_TRAFFIC.get(key) if default_opts else None
+        if off:
+            traffic = dict(off, source="offline profile (profiles/): the live counter runs were not available: "
+                                       + traffic["error"])
+    tl = traffic.get("launch", {})
 
+    def roof(phase, label, alg_bytes, ms):
+        t = tl.get(phase)
+        tb = t["bytes"] if t and ms > 0 else None
+        return {
+            "bound": "hbm", "kernel": label,
+            # achieved / frac: HBM-side bytes the launch really moved (profiler counters) over its duration
+            "achieved": tb / (ms * 1e-3) / 1e9 if tb else None, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": tb / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS if tb else None,
+            "traffic": tb, "traffic_read": t["read_bytes"] if t else None, "traffic_written": t["written_bytes"] if t else None,
+            "tcc_hit_rate": t.get("tcc_hit_rate") if t else None,
+            "tcc_miss_x_128B": t.get("tcc_miss_x_128B") if t else None,
+            "ms_per_launch": ms,
+            # the model figure: one gathered row per edge whether or not a cache served it; exceeds the HBM peak
+            # when rows gathered many times come from L2 / Infinity Cache
+            "algorithmic_bytes": alg_bytes, "algorithmic_GBs": alg_bytes / (ms * 1e-3) / 1e9 if ms > 0 else None,
+            "algorithmic_frac": alg_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS if ms > 0 else None,
+        }
+
+    layer_traffic = (tl[1]["bytes"] + (tl[0]["bytes"] if 0 in tl else 0.0)) if 1 in tl else None
     result = {
         "metric": "GEdges/s per aggregation layer (reuse plan), 1 MI355X",
         "value": e / (wall_ms * 1e-3) / 1e9,
@@ -527,28 +729,26 @@ def main():
         "dtype": "bf16->f32" if bf16 else "f32",
         "data": "synthetic",
         "config": {"workload": DESCR[name], "nodes": n, "edges": e, "feat": feat, "row_stride": ld, "out_row_stride": ldo,
+                   "output": "padded rows (pad_columns)" if pad else "packed [N, feat], as the operator API returns it",
                    "part_size": ps, "normalized": normalized, "search": args.search},
-        "roofline": {
-            "bound": "hbm", "kernel": "rof_rows_kernel (destination-row launch)",
-            "achieved": achieved_b, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved_b / HBM_PEAK_GBS,
-            "traffic": traffic[1], "bytes_per_launch": bytes_b, "ms_per_launch": ms_b,
-        },
+        "roofline": roof(1, "rof_rows_kernel (destination-row launch)", bytes_b, ms_b),
         # the launch before it (segments of long rows, swept in the order of their source ids): same kernel
         # template, second in duration
-        "roofline_partial_launch": {
-            "bound": "hbm", "kernel": "rof_rows_kernel (partial-sum launch)",
-            "achieved": achieved_a, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved_a / HBM_PEAK_GBS,
-            "traffic": traffic[0], "bytes_per_launch": bytes_a, "ms_per_launch": ms_a,
-        },
+        "roofline_partial_launch": roof(0, "rof_rows_kernel (partial-sum launch)", bytes_a, ms_a),
+        "traffic_source": traffic.get("source", traffic.get("error")),
+        "traffic_counter_scale": {"FETCH_SIZE": traffic.get("fetch_scale"), "WRITE_SIZE": traffic.get("write_scale")},
         "layer": {
             "event_ms": ev_ms, "event_ms_runs": ev_r, "per_call": spread, "launch1_ms": ms_a, "launch2_ms": ms_b,
-            "algorithmic_bytes": b_alg, "achieved_GBs": b_alg / (ev_ms * 1e-3) / 1e9,
-            "frac_of_hbm_peak": b_alg / (ev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "traffic": layer_traffic,
+            "frac_of_hbm_peak": layer_traffic / (ev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS if layer_traffic else None,
+            "b_min": b_min, "traffic_over_b_min": layer_traffic / b_min if layer_traffic else None,
+            "algorithmic_bytes": b_alg, "algorithmic_GBs": b_alg / (ev_ms * 1e-3) / 1e9,
+            "algorithmic_frac": b_alg / (ev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
             "no_reuse_model_bytes": b_noreuse_model,
         },
         "reuse_disabled": {
             "event_ms": plain_ms, "launch1_ms": pms_a, "launch2_ms": pms_b, "GEdges_per_s": e / (plain_ms * 1e-3) / 1e9,
-            "achieved_GBs": b_alg_plain / (plain_ms * 1e-3) / 1e9, "speedup_of_reuse": plain_ms / ev_ms,
+            "algorithmic_GBs": b_alg_plain / (plain_ms * 1e-3) / 1e9, "speedup_of_reuse": plain_ms / ev_ms,
             "max_abs_diff_vs_reuse": max_diff,
         },
         "reuse_forced": forced_info,
@@ -556,7 +756,7 @@ def main():
                  "folded_by_cost_model": bool(st["materialised_groups"] == 0 and st["groups"] > 0),
                  "gathered_rows": st["gathered_rows"], "partial_reads": st["partial_reads"],
                  "partial_rows": st["partial_rows"], "hub_segments": st["hub_segments"],
-                 "saved_gathers_frac": 1.0 - st["gathered_rows"] / max(1, e),
+                 "saved_gathers_frac": 1.0 - (st["gathered_rows"] + st["partial_reads"] - st["hub_segments"]) / max(1, e),
                  "cpu_graph_s": t_gen, "cpu_plan_s": t_plan, "cpu_layout_s": t_layout},
     }
 

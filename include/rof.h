@@ -1,9 +1,12 @@
 /* rof.h -- C ABI of the MI355X reuse-aware neighbour-aggregation library (librof.so).
  *
  * Every entry point is extern "C", takes plain pointers and sizes, returns 0 or a negative
- * rof_status, never throws, never exits the process and keeps no global state besides the
- * handles it returns.  Host-side functions are safe to call concurrently on different handles;
- * device-side functions enqueue on the hipStream_t they are given and do not synchronise.
+ * rof_status, never throws and never exits the process.  State lives in the handles it returns;
+ * the only process-wide state is the static device scratch of rof_aggregate_noalloc (one copy per
+ * GPU) and the launch-tuning settings of the benchmark interface in rof_bench.h, which are not meant
+ * to be changed while other threads launch.  Host-side functions are safe to call concurrently on
+ * different handles; device-side functions enqueue on the hipStream_t they are given and do not
+ * synchronise.
  *
  * Citations name the upstream interface each entry point replaces (paths relative to the
  * upstream tree).
@@ -213,9 +216,10 @@ int rof_aggregate(const rof_layout *layout, const void *x, int x_dtype, int64_t 
  *   next layer's GEMM or aggregation without a conversion pass.
  * pad_columns != 0: the caller allows the library to treat the rows as round_up(feat_dim, 4) (8 for bf16
  *   features) columns wide: ldx and ldo are at least that, the extra columns of x are readable, `bias` (if any) has
- *   that many elements, and the extra columns of `out` receive the aggregate of the extra columns of x.  Every
- *   lane then stores whole 16-byte pieces, and a large output qualifies for streaming stores (2.4 M x 47 floats
- *   in rows of 48: 1.24 ms against 1.32 ms).  Columns 0 .. feat_dim-1 are the same either way.
+ *   that many elements, and the extra columns of `out` receive the aggregate of the extra columns of x (whatever
+ *   they hold: uninitialised padding of x may put non-finite values into the padding of out, never into columns
+ *   0 .. feat_dim-1, which are the same either way).  Every piece a lane stores is then 16-byte aligned
+ *   (2.4 M x 47 floats: 1.23 ms in rows of 48 against 1.25 ms packed).
  * Rows of nodes without in-edges become act(self_weight * x[v] + bias).  ep == NULL is rof_aggregate. */
 typedef struct {
     const float *bias;
@@ -246,19 +250,6 @@ int rof_aggregate_epilogue(const rof_layout *layout, const void *x, int x_dtype,
 int rof_aggregate_noalloc(const rof_layout *layout, const void *x, int x_dtype, int64_t ldx, void *out, int64_t ldo,
                           int feat_dim, int normalized, const rof_epilogue *epilogue, void *stream);
 
-/* Timing helper for benchmarks: runs rof_aggregate_epilogue (rof_aggregate when epilogue == NULL) `iters` times on `stream` between two HIP
- * events recorded on that same stream and returns the mean milliseconds per call. */
-int rof_aggregate_timed(const rof_layout *layout, const void *x, int x_dtype, int64_t ldx, void *out, int64_t ldo,
-                        int feat_dim, int normalized, const rof_epilogue *epilogue, void *workspace,
-                        size_t workspace_bytes, void *stream, int iters, float *ms_per_call);
-
-/* Per-launch timing for the roofline report: ms_launch[1] = mean duration of the destination-row
- * launch alone (HIP events on `stream` around it), ms_launch[0] = mean duration of the whole call minus
- * that, i.e. the partial-sum launch.  No upstream counterpart. */
-int rof_aggregate_launch_times(const rof_layout *layout, const void *x, int x_dtype, int64_t ldx, void *out,
-                               int64_t ldo, int feat_dim, int normalized, const rof_epilogue *epilogue,
-                               void *workspace, size_t workspace_bytes, void *stream, int iters, float ms_launch[2]);
-
 /* Column sums of a row-major device matrix: out[c] = sum_r x[r, c], x float32 or bfloat16 [n, f] with row
  * stride ldx (elements), out float32[f].  This is the bias gradient of a layer (upstream leaves it to autograd's
  * reduction of `out + self.bias`, reuse_conv.py:147-150); summed in fp32 in a fixed order (bitwise repeatable).
@@ -266,22 +257,6 @@ int rof_aggregate_launch_times(const rof_layout *layout, const void *x, int x_dt
 size_t rof_column_sums_workspace_bytes(int64_t n, int f);
 int rof_column_sums(const void *x, int x_dtype, int64_t ldx, int64_t n, int f, float *out, void *workspace,
                     size_t workspace_bytes, void *stream);
-
-/* Plain device-to-device streaming copy (nbytes a multiple of 16, pointers 16-byte aligned).  Exists so
- * that a profiler's FETCH_SIZE / WRITE_SIZE counters can be calibrated against a transfer of known size.
- * No upstream counterpart. */
-int rof_device_copy(void *dst, const void *src, size_t nbytes, void *stream);
-
-/* Launch tuning: how many consecutive workgroups of the partial-sum launches / of the destination-row launch
- * stay on one XCD (each XCD has its own L2, so runs of neighbouring destination rows share gathered rows
- * there).  run_launch2 = 0 (the default) lets every layout use its own choice: one tile of destinations per
- * run when at least half of the neighbours lie within 8192 ids of their row (block-structured graphs), 16
- * workgroups otherwise.  Process-wide; no upstream counterpart. */
-int rof_set_xcd_run(int run_launch1, int run_launch2);
-
-/* Launch tuning: request `bytes` (0..65536) of unused LDS per workgroup, which caps how many workgroups
- * share a CU (160 KB LDS each) and with it the number of row gathers in flight.  Process-wide. */
-int rof_set_lds_pad(int bytes);
 
 #ifdef __cplusplus
 }

@@ -8,6 +8,29 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 
+def _memoise_workloads():
+    """Several tests build the same scaled-down workload graph; generate each once per session (the tests get
+    copies, so none can disturb another)."""
+    from artifact_amd import graphgen
+
+    raw, cache = graphgen.make_workload, {}
+
+    def make_workload(name, scale_down=0):
+        key = (name, scale_down)
+        if key not in cache:
+            ip, ix = raw(name, scale_down)
+            if len(ix) > 20_000_000:      # full-size graphs are built by one module each: not worth the memory
+                return ip, ix
+            cache[key] = (ip, ix)
+        ip, ix = cache[key]
+        return ip.copy(), ix.copy()
+
+    graphgen.make_workload = make_workload
+
+
+_memoise_workloads()
+
+
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 

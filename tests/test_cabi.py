@@ -11,10 +11,16 @@ from artifact_amd import _lib
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
+HEADERS = ("rof.h", "rof_bench.h")   # the library's interface and its benchmark / tuning interface
+
+
 def _declared():
-    text = open(os.path.join(ROOT, "include", "rof.h")).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(rof_[a-z0-9_]+)\s*\(", text)))
+    names = set()
+    for header in HEADERS:
+        text = open(os.path.join(ROOT, "include", header)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names |= set(re.findall(r"\b(rof_[a-z0-9_]+)\s*\(", text))
+    return sorted(names)
 
 
 def test_library_is_built_in_tree_and_loads():
@@ -27,13 +33,21 @@ def test_every_declared_symbol_is_exported():
     names = _declared()
     assert len(names) >= 25
     for name in names:
-        assert hasattr(L, name), f"{name} is declared in include/rof.h but not exported"
+        assert hasattr(L, name), f"{name} is declared in include/ but not exported"
     assert set(_lib.SYMBOLS) == set(names)
 
 
 def test_no_torch_types_in_signatures():
+    for header in HEADERS:
+        text = open(os.path.join(ROOT, "include", header)).read()
+        assert "torch" not in text.lower() and "at::" not in text and "#include <hip" not in text
+
+
+def test_benchmark_entry_points_are_not_in_the_product_header():
     text = open(os.path.join(ROOT, "include", "rof.h")).read()
-    assert "torch" not in text.lower() and "at::" not in text and "#include <hip" not in text
+    for name in ("rof_aggregate_timed", "rof_aggregate_launch_times", "rof_device_copy", "rof_set_xcd_run",
+                 "rof_set_lds_pad"):
+        assert name not in text
 
 
 def test_error_codes_and_messages():
@@ -47,6 +61,7 @@ def test_error_codes_and_messages():
     assert L.rof_plan_build(None, None, None, None, 0, 0, 3, 1, C.byref(h)) == -1
     assert L.rof_layout_from_v2(None, None, None, None, 0, 0, 3, None, C.byref(h)) == -1
     assert L.rof_aggregate(None, None, 0, 0, None, 0, 1, 1, None, 0, None) == -1
+    assert L.rof_aggregate_noalloc(None, None, 0, 0, None, 0, 1, 1, None, None) == -1
     assert L.rof_layout_workspace_bytes(None, 4) == 0
     assert L.rof_set_xcd_run(0, 1) == -1
     assert L.rof_set_xcd_run(1, 0) == 0                      # 0 for the destination-row launch: per-layout choice
