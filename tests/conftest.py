@@ -55,3 +55,17 @@ def oracle():
     from oracle import oracle as O
     O.lib()
     return O
+
+
+def pytest_terminal_summary(terminalreporter):
+    """How often the fp32 parity checks needed the summation term of their tolerance (helpers.close_fp32)."""
+    try:
+        from helpers import FP32_BAR_STATS as st
+    except ImportError:
+        return
+    if st["compared"]:
+        terminalreporter.write_line(
+            f"fp32 parity: {st['compared']} elements compared against float64 / the fp32 restatement; "
+            f"{st['beyond_strict']} ({100.0 * st['beyond_strict'] / st['compared']:.5f} %) beyond the strict bar "
+            f"1e-6 + 1e-5*|want| and inside the summation bound; largest error there {st['max_excess_ratio']:.2f}x the "
+            f"strict bar ({st['max_excess_abs']:.2e} above it)")

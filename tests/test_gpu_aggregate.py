@@ -15,6 +15,7 @@ from artifact_amd import reuse_search_ext as R            # noqa: E402
 from artifact_amd.graphgen import features, make_workload  # noqa: E402
 from artifact_amd.layout import Layout                     # noqa: E402
 from artifact_amd._lib import RofError                     # noqa: E402
+from helpers import close_fp32                             # noqa: E402
 
 
 def _case(name, scale_down, ps):
@@ -30,12 +31,8 @@ def _layout(plan, n, ps, **opts):
 
 def _close(got, want64, x_abs_rowsum=None, rtol=1e-5, atol=1e-6):
     """|got - want| <= atol + rtol*|want| + rtol*(sum of |terms|): the last term is the standard fp32
-    summation bound and matters only where cancellation makes |want| tiny."""
-    tol = atol + rtol * np.abs(want64)
-    if x_abs_rowsum is not None:
-        tol = tol + rtol * x_abs_rowsum
-    bad = np.abs(got - want64) > tol
-    assert not bad.any(), f"{bad.sum()} elements off, max err {np.abs(got - want64).max():.3e}"
+    summation bound and matters only where cancellation makes |want| tiny (helpers.close_fp32 counts how often)."""
+    close_fp32(got, want64, x_abs_rowsum, rtol, atol)
 
 
 @pytest.mark.parametrize("feat", [1, 3, 4, 32, 40, 47, 64, 100, 256, 300])

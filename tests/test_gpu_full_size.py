@@ -12,6 +12,7 @@ torch = pytest.importorskip("torch")
 from artifact_amd import reuse_search_ext as R            # noqa: E402
 from artifact_amd.graphgen import make_workload            # noqa: E402
 from artifact_amd.layout import Layout                     # noqa: E402
+from helpers import close_fp32                             # noqa: E402
 
 
 @pytest.fixture(scope="module")
@@ -64,7 +65,7 @@ def test_full_size_properties(big):
         nb = ix[ip[v]:ip[v + 1]]
         want = r[v] * (xh[nb] * r[nb, None]).sum(0) if len(nb) else np.zeros(47)
         mag = r[v] * (np.abs(xh[nb]) * r[nb, None]).sum(0) if len(nb) else np.zeros(47)
-        assert (np.abs(ah[v] - want) <= 1e-6 + 1e-5 * np.abs(want) + 1e-5 * mag).all(), v
+        close_fp32(ah[v], want, mag, what=f"row {v}")
 
 
 def test_full_size_epilogue_and_bias_gradient(big):

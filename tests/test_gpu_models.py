@@ -163,6 +163,43 @@ def test_training_learns_and_gin_runs():
     assert out.shape == (n, 4) and all(p.grad is not None for p in gin.parameters())
 
 
+def test_three_layer_gin_matches_a_dense_float64_model():
+    """The block-structured workload's model (3 x GIN 64 -> 64, sum aggregation, eps = 0, ReLU between) on a
+    scaled-down graph of the same generator: forward, input gradient and every parameter gradient against the
+    same model written with a dense float64 adjacency."""
+    ip, ix = make_workload("c3", 6)                                      # SBM, 4 blocks of 4096 nodes
+    n = len(ip) - 1
+    info = build_input_info(ip, ix, 3, device=DEV, min_consumers=2)
+    torch.manual_seed(5)
+    gin = ROF_GIN(64, 64, 64, 3, activation=torch.relu, eps=0.0).to(DEV)
+    x = torch.from_numpy(features(n, 64, seed=71)).to(DEV).requires_grad_(True)
+    coef = torch.from_numpy(features(n, 64, seed=72)).to(DEV)
+    out = gin(x, info)
+    (out * coef).sum().backward()
+    # dense float64 model: h <- W_l ((1 + eps) h + A h) + b_l
+    rows = np.repeat(np.arange(n), np.diff(ip))
+    a = torch.sparse_coo_tensor(np.stack([rows, ix.astype(np.int64)]), np.ones(len(ix)), (n, n)).coalesce()
+    ws = [(l.mlp.weight.detach().cpu().double().requires_grad_(True), l.mlp.bias.detach().cpu().double().requires_grad_(True))
+          for l in gin.layers]
+    xd = x.detach().cpu().double().requires_grad_(True)
+    h = xd
+    for i, (w, b) in enumerate(ws):
+        h = (h + torch.sparse.mm(a, h)) @ w.t() + b
+        if i != 2:
+            h = torch.relu(h)
+    (h * coef.cpu().double()).sum().backward()
+    # three sums over ~27 neighbours each compound the fp32 round-off: relative to the size of the whole result
+    def rel(got, want):
+        return ((got.detach().cpu().double() - want.detach()).norm() / want.detach().norm()).item()
+    assert rel(out, h) < 2e-6
+    assert rel(x.grad, xd.grad) < 5e-6
+    for layer, (w, b) in zip(gin.layers, ws):
+        assert rel(layer.mlp.weight.grad, w.grad) < 5e-6 and rel(layer.mlp.bias.grad, b.grad) < 5e-6
+    # element-wise at the stated bar, widened by the magnitude of the result (sums of sums: no per-term bound here)
+    scale = h.detach().abs().max().item()
+    assert (out.detach().cpu().double() - h.detach()).abs().max().item() <= 1e-5 * scale
+
+
 @pytest.mark.parametrize("fused", [False, True])
 def test_loss_curve_follows_a_dense_float64_model(fused):
     """Forty Adam steps of the two-layer GCN (no dropout) against the same model written with a dense float64

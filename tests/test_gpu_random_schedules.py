@@ -16,6 +16,7 @@ torch = pytest.importorskip("torch")
 
 from artifact_amd import reuse_search_ext as R            # noqa: E402
 from artifact_amd.layout import Layout                     # noqa: E402
+from helpers import close_fp32                             # noqa: E402
 
 LANES = [0, 4, 8, 10, 12, 16, 20, 32, 64]
 
@@ -107,8 +108,4 @@ def test_random_schedules_match_the_closed_form(oracle, block):
             want, mag = want + bias, mag + np.abs(bias)
         if relu:
             want = np.maximum(want, 0.0)
-        tol = 1e-6 + 1e-5 * np.abs(want) + 1e-5 * mag
-        if bf16_out:
-            tol = tol + 2.0 ** -8 * np.abs(want)
-        bad = np.abs(got - want) > tol
-        assert not bad.any(), f"{what}: {bad.sum()} off, max err {np.abs(got - want).max():.3e}"
+        close_fp32(got, want, mag, extra=2.0 ** -8 * np.abs(want) if bf16_out else None, what=what)

@@ -12,6 +12,7 @@ from artifact_amd import ROF                                              # noqa
 from artifact_amd import reuse_search_ext as R                            # noqa: E402
 from artifact_amd.graphgen import features, glorot, make_workload          # noqa: E402
 from artifact_amd.reuse_conv import ROF_GCNConv, ROF_GINConv, build_input_info  # noqa: E402
+from helpers import close_fp32                             # noqa: E402
 
 DEV = "cuda"
 
@@ -26,8 +27,7 @@ def _setup(wl="c1", sd=2, ps=3, fin=20, fout=47):
 
 
 def _close(got, want, mag, rtol=1e-5, atol=1e-6):
-    tol = atol + rtol * np.abs(want) + rtol * mag
-    assert (np.abs(got - want) <= tol).all(), f"max err {np.abs(got - want).max():.3e}"
+    close_fp32(got, want, mag, rtol, atol)
 
 
 def _call(kind, info, *lead):
