@@ -30,7 +30,8 @@ class RofError(RuntimeError):
 class LayoutOpts(C.Structure):
     _fields_ = [("min_consumers", C.c_int32), ("disable_reuse", C.c_int32), ("hub_split", C.c_int32),
                 ("segment", C.c_int32), ("lanes_per_row", C.c_int32), ("entry_order", C.c_int32),
-                ("tile_rows", C.c_int32), ("elem_bytes", C.c_int32)]
+                ("tile_rows", C.c_int32), ("elem_bytes", C.c_int32), ("local_groups", C.c_int32),
+                ("reserved", C.c_int32 * 3)]
 
 
 class Epilogue(C.Structure):

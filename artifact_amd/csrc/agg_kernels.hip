@@ -37,6 +37,7 @@
 #include <atomic>
 #include <mutex>
 #include <new>
+#include <vector>
 
 #include "agg_rows.h"
 #include "rof.h"
@@ -169,7 +170,18 @@ int upload_phase(const rof_phase_host &h, rof_phase_dev &d, bool with_scale, hip
     };
     int rc;
     if ((rc = put(&d.task_ptr, h.task_ptr))) return rc;
-    if ((rc = put(&d.task_nref, h.task_nref))) return rc;
+    if (h.task_nlds.empty()) {
+        if ((rc = put(&d.task_nref, h.task_nref))) return rc;
+    } else {
+        // the kernel reads one word per task: references in the low 24 bits, LDS rows above
+        std::vector<int32_t> packed(h.task_nref.size());
+        for (size_t i = 0; i < packed.size(); ++i) {
+            if (h.task_nref[i] >= (1 << 24) || h.task_nlds[i] >= 128) return ROF_ERR_UNSUPPORTED;
+            packed[i] = (int32_t)((uint32_t)h.task_nref[i] | ((uint32_t)h.task_nlds[i] << 24));
+        }
+        if ((rc = put(&d.task_nref, packed))) return rc;
+        HIP_TRY(hipStreamSynchronize(st));   // `packed` goes out of scope
+    }
     if ((rc = put(&d.task_out, h.task_out))) return rc;
     if ((rc = put(&d.col, h.col))) return rc;
     size_t wb = (h.col.size() ? h.col.size() : 1) * sizeof(float);
@@ -179,6 +191,19 @@ int upload_phase(const rof_phase_host &h, rof_phase_dev &d, bool with_scale, hip
         size_t sb = (size_t)(h.n_tasks ? h.n_tasks : 1) * sizeof(float);
         HIP_TRY(hipMalloc((void **)&d.scale, sb));
         *bytes += (int64_t)sb;
+    }
+    d.n_regular = h.lg_blocks > 0 ? h.n_regular : h.n_tasks;
+    d.lg_blocks = h.lg_blocks;
+    d.lg_max_rows = h.lg_max_rows;
+    d.lg_entries = (int64_t)h.lg_col.size();
+    if (h.lg_blocks > 0) {
+        if ((rc = put(&d.lg_task_first, h.lg_task_first))) return rc;
+        if ((rc = put(&d.lg_ptr, h.lg_ptr))) return rc;
+        if ((rc = put(&d.lg_task_ptr, h.lg_task_ptr))) return rc;
+        if ((rc = put(&d.lg_col, h.lg_col))) return rc;
+        size_t lb = (h.lg_col.size() ? h.lg_col.size() : 1) * sizeof(float);
+        HIP_TRY(hipMalloc((void **)&d.lg_w, lb));
+        *bytes += (int64_t)lb;
     }
     return ROF_OK;
 }
@@ -190,6 +215,11 @@ void free_phase(rof_phase_dev &d) {
     if (d.col) (void)hipFree(d.col);
     if (d.w) (void)hipFree(d.w);
     if (d.scale) (void)hipFree(d.scale);
+    if (d.lg_ptr) (void)hipFree(d.lg_ptr);
+    if (d.lg_task_first) (void)hipFree(d.lg_task_first);
+    if (d.lg_task_ptr) (void)hipFree(d.lg_task_ptr);
+    if (d.lg_col) (void)hipFree(d.lg_col);
+    if (d.lg_w) (void)hipFree(d.lg_w);
     d = rof_phase_dev();
 }
 
@@ -250,7 +280,7 @@ const char *rof_strerror(int status) {
     }
 }
 
-int rof_version(void) { return 1; }
+int rof_version(void) { return 2; }
 
 // Tuning knobs used by the benchmark sweeps.
 int rof_set_lds_pad(int bytes) {
@@ -335,6 +365,9 @@ int rof_layout_set_degrees(rof_layout *L, const float *deg, void *stream) {
     if (L->db.n_entries)
         hipLaunchKernelGGL(rof_entry_weights_kernel, dim3((unsigned)((L->db.n_entries + tb - 1) / tb)), dim3(tb), 0, st,
                            L->db.col, L->db.n_entries, deg, L->n, L->db.w);
+    if (L->db.lg_entries)
+        hipLaunchKernelGGL(rof_entry_weights_kernel, dim3((unsigned)((L->db.lg_entries + tb - 1) / tb)), dim3(tb), 0, st,
+                           L->db.lg_col, L->db.lg_entries, deg, L->n, L->db.lg_w);
     if (L->db.n_tasks)
         hipLaunchKernelGGL(rof_task_scale_kernel, dim3((unsigned)((L->db.n_tasks + tb - 1) / tb)), dim3(tb), 0, st,
                            L->db.task_out, L->db.n_tasks, deg, L->db.scale);
@@ -418,7 +451,7 @@ static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64
         a.n_tasks = d.n_tasks;
         a.xcd_run = g_xcd_run_a;
         a.vec_store = 1;
-        if ((rc = (x_dtype == ROF_F32 ? rofk::launch_rows_f32(a, 0, vec, off32, st) : rofk::launch_rows_bf16(a, 0, vec, off32, st)))) return rc;
+        if ((rc = (x_dtype == ROF_F32 ? rofk::launch_rows_f32(a, 0, vec, off32, 0, st) : rofk::launch_rows_bf16(a, 0, vec, off32, 0, st)))) return rc;
     }
     if (L->db.n_tasks && (launches & 2)) {   // last launch: destination rows
         a.task_ptr = L->db.task_ptr;
@@ -437,9 +470,22 @@ static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64
         a.bias = bias;
         a.relu = relu ? 1 : 0;
         a.self_weight = self_weight;
+        a.lg_task_first = L->db.lg_task_first;
+        a.lg_ptr = L->db.lg_ptr;
+        a.lg_task_ptr = L->db.lg_task_ptr;
+        a.lg_col = L->db.lg_col;
+        a.lg_w = normalized ? L->db.lg_w : nullptr;
         const int phase = ((int64_t)L->n * feat * (a.out_bf16 ? 2 : 4) >= kStreamOutBytes && a.vec_store && vec > 1 &&
                            (!a.out_bf16 || ldo % 2 == 0)) ? 2 : 1;
-        if ((rc = (x_dtype == ROF_F32 ? rofk::launch_rows_f32(a, phase, vec, off32, st) : rofk::launch_rows_bf16(a, phase, vec, off32, st)))) return rc;
+        a.n_tasks = L->db.n_regular;   // the clustered destinations at the end of the list have a launch of their own
+        if ((rc = (x_dtype == ROF_F32 ? rofk::launch_rows_f32(a, phase, vec, off32, 0, st) : rofk::launch_rows_bf16(a, phase, vec, off32, 0, st)))) return rc;
+        if (L->db.lg_blocks > 0) {
+            a.n_tasks = L->db.n_tasks;
+            a.n_blocks = L->db.lg_blocks;
+            a.xcd_run = 1;
+            if ((rc = (x_dtype == ROF_F32 ? rofk::launch_rows_f32(a, phase, vec, off32, L->db.lg_max_rows, st)
+                                          : rofk::launch_rows_bf16(a, phase, vec, off32, L->db.lg_max_rows, st)))) return rc;
+        }
     }
     return ROF_OK;
 }

@@ -48,6 +48,11 @@ struct AggArgs {
     int32_t relu;              // destination-row launch only: clamp the output at zero
     int32_t out_bf16;          // destination-row launch only: store bf16 (round to nearest even)
     float self_weight;         // destination-row launch only: + self_weight * x[out row] (0: none)
+    // cluster launch only (CLUSTER instantiations): workgroup i has its own list of short tasks lg_task_first[i] ..
+    // lg_task_first[i+1] and its local groups lg_ptr[i] .. lg_ptr[i+1] (local group j gathers
+    // lg_col[lg_task_ptr[j] .. lg_task_ptr[j+1])), which it sums into LDS before its tasks run
+    const int32_t *lg_ptr, *lg_task_ptr, *lg_col, *lg_task_first;
+    const float *lg_w;         // null: unweighted
 };
 
 // fp32 -> bf16, round to nearest even, NaN -> quiet NaN (the conversion PyTorch's .to(bfloat16) performs)
@@ -215,6 +220,75 @@ __device__ __forceinline__ void gather_sum(const char *xb, uint32_t xld, const c
     }
 }
 
+// Scale the finished sum of task t, apply the layer's epilogue (PHASE >= 1) and store this lane's piece of the
+// output row.  `acc` holds the columns cstart .. cstart + VEC - 1; `skip` of them repeat the neighbouring lane's.
+template <typename XT, int VEC, int PHASE>
+__device__ __forceinline__ void finish_row(const AggArgs &a, int32_t t, bool nonempty, const float (&acc)[VEC], const char *xb,
+                                           uint32_t xld, int cstart, int skip) {
+    // an empty task writes zeros whatever its scale is (a node without in-edges keeps the
+    // zero-initialised output upstream: reuse_conv_kernel.cu:303)
+    float s = 1.0f;
+    if (a.task_scale && nonempty) s = a.task_scale[t];
+    const int64_t at = (int64_t)a.task_out[t] * a.ldo + cstart;
+    float r[VEC];
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) r[k] = acc[k] * s;
+    if (PHASE >= 1) {   // epilogue of the layer: + own row, + bias, then ReLU (columns cstart .. cstart+VEC-1 exist)
+        if (a.self_weight != 0.0f) {
+            float own[VEC];
+            RowLoad<XT, VEC>::load(reinterpret_cast<const XT *>(xb + (int64_t)a.task_out[t] * xld), own);
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) r[k] = fmaf(a.self_weight, own[k], r[k]);
+        }
+        if (a.bias) {
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) r[k] = __fadd_rn(r[k], a.bias[cstart + k]);   // never fused into the scaling: same bits as a separate pass
+        }
+        if (a.relu) {
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) r[k] = fmaxf(r[k], 0.0f);
+        }
+    }
+    // A large output is not read again before the caches have turned over, so its rows are written as
+    // streaming stores (`nt`): they then do not push feature rows out of L2 and the Infinity Cache.
+    // Every lane stores whole 16-byte pieces (8-byte for bf16 output) wherever the piece starts on a 4-byte
+    // boundary -- gfx950 executes global_store_dwordx4 at any dword address, like the loads -- so packed rows
+    // (47 floats = 188 bytes) are written as one contiguous burst per row.  The lane that was shifted back
+    // to stay inside the row rewrites `skip` elements of its neighbour's piece with the same bits (both
+    // lanes sum the same entries in the same order).
+    constexpr bool stream = PHASE == 2;
+    if (PHASE >= 1 && a.out_bf16) {
+        uint16_t *o = reinterpret_cast<uint16_t *>(a.out) + at;
+        if (VEC >= 4 && a.vec_store && (at & 1) == 0) {
+#pragma unroll
+            for (int k = 0; k < VEC; k += 4) {
+                const rof_u2s t = {rof_bf16_bits(r[k]) | (rof_bf16_bits(r[k + 1]) << 16),
+                                   rof_bf16_bits(r[k + 2]) | (rof_bf16_bits(r[k + 3]) << 16)};
+                if (stream) __builtin_nontemporal_store(t, reinterpret_cast<rof_u2s *>(o + k));
+                else *reinterpret_cast<rof_u2s *>(o + k) = t;
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < VEC; ++k)
+                if (k >= skip && cstart + k < a.feat) o[k] = (uint16_t)rof_bf16_bits(r[k]);
+        }
+    } else {
+        float *o = reinterpret_cast<float *>(a.out) + at;
+        if (VEC >= 4 && a.vec_store) {
+#pragma unroll
+            for (int k = 0; k < VEC; k += 4) {
+                const rof_f4 t = {r[k], r[k + 1], r[k + 2], r[k + 3]};
+                if (stream) __builtin_nontemporal_store(t, reinterpret_cast<rof_f4 *>(o + k));
+                else *reinterpret_cast<rof_f4 *>(o + k) = t;
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < VEC; ++k)
+                if (k >= skip && cstart + k < a.feat) o[k] = r[k];
+        }
+    }
+}
+
 // PHASE 0: the partial-sum launches (no scaling, no epilogue); PHASE 1: the destination-row launch; PHASE 2: the
 // same with the output rows written as streaming stores and the index arrays read as streaming loads (large outputs,
 // hence large graphs).  (A run-time switch between the two kinds of store does
@@ -315,70 +389,103 @@ __global__ __launch_bounds__(256) void rof_rows_kernel(AggArgs a) {
             }
         }
 
-        const bool writer = valid && act && (!wave_mode || sub == 0);
-        if (writer) {
-            // an empty task writes zeros whatever its scale is (a node without in-edges keeps the
-            // zero-initialised output upstream: reuse_conv_kernel.cu:303)
-            float s = 1.0f;
-            if (a.task_scale && end > beg) s = a.task_scale[t];
-            const int64_t at = (int64_t)a.task_out[t] * a.ldo + cstart;
-            float r[VEC];
-#pragma unroll
-            for (int k = 0; k < VEC; ++k) r[k] = acc[k] * s;
-            if (PHASE >= 1) {   // epilogue of the layer: + own row, + bias, then ReLU (columns cstart .. cstart+VEC-1 exist)
-                if (a.self_weight != 0.0f) {
-                    float own[VEC];
-                    RowLoad<XT, VEC>::load(reinterpret_cast<const XT *>(xb + (int64_t)a.task_out[t] * xld), own);
-#pragma unroll
-                    for (int k = 0; k < VEC; ++k) r[k] = fmaf(a.self_weight, own[k], r[k]);
-                }
-                if (a.bias) {
-#pragma unroll
-                    for (int k = 0; k < VEC; ++k) r[k] = __fadd_rn(r[k], a.bias[cstart + k]);   // never fused into the scaling: same bits as a separate pass
-                }
-                if (a.relu) {
-#pragma unroll
-                    for (int k = 0; k < VEC; ++k) r[k] = fmaxf(r[k], 0.0f);
-                }
+        if (valid && act && (!wave_mode || sub == 0))
+            finish_row<XT, VEC, PHASE>(a, t, end > beg, acc, xb, xld, cstart, skip);
+    }
+}
+
+// The launch of the clustered destinations (PHASE >= 1 only).  Workgroup i holds cluster i: destinations that share
+// reuse groups.  It first sums its local groups lg_ptr[i] .. lg_ptr[i+1] into LDS rows, one lane group per group,
+// then works through its own list of short tasks (lg_task_first[i] .. lg_task_first[i+1], in rounds of 4 * G), and
+// those tasks add LDS rows instead of gathering the groups' sources.  An LDS row holds the LPR * VEC columns of the
+// current feature chunk, laid out by lane, so a lane reads back exactly the columns it accumulates.  (A kernel of
+// its own rather than a branch of rof_rows_kernel: there the extra live values cost an occupancy step, 6-8 % of
+// the launch.)
+template <typename XT, int VEC, int LPR, int PHASE, bool OFF32>
+__global__ __launch_bounds__(256) void rof_cluster_kernel(AggArgs a) {
+    static_assert(PHASE >= 1, "clusters belong to the destination-row launch");
+    constexpr int G = 64 / LPR;
+    constexpr int kLdsRow = LPR * VEC + 4;
+    HIP_DYNAMIC_SHARED(float, lds_rows)
+    const int hw = blockIdx.x;
+    const int xcd = hw % kXcds, nth = hw / kXcds;
+    const int run = a.xcd_run;
+    const int cb = ((nth / run) * kXcds + xcd) * run + (nth % run);
+    if (cb >= a.n_blocks) return;
+
+    const int lane = threadIdx.x & 63;
+    const int sub = lane / LPR, li = lane % LPR;
+    const int wid = threadIdx.x >> 6;
+    const bool idle = (G * LPR < 64) && lane >= G * LPR;   // lanes left over when LPR does not divide 64
+    const int32_t ct0 = a.lg_task_first[cb], ct1 = a.lg_task_first[cb + 1];
+    const int32_t lg0 = a.lg_ptr[cb], lg1 = a.lg_ptr[cb + 1];
+    const uint32_t xld = (uint32_t)(a.ldx * (int64_t)sizeof(XT)), pld = (uint32_t)(a.ldp * 4);
+    constexpr bool kF32 = sizeof(XT) == 4;
+
+    for (int c0 = 0; c0 < a.feat; c0 += LPR * VEC) {
+        const int cbase = c0 + li * VEC;
+        const bool act = !idle && cbase < a.feat;
+        const int cstart = (VEC > 1 && cbase + VEC > a.feat) ? a.feat - VEC : cbase;   // see rof_rows_kernel
+        const int skip = cbase - cstart;
+        const char *xb = reinterpret_cast<const char *>(a.x) + (size_t)cstart * sizeof(XT);
+        const char *pb = reinterpret_cast<const char *>(a.part) + (size_t)cstart * 4;
+
+        if (c0 > 0) __syncthreads();   // the previous chunk's rows have been read by every task
+        for (int g0 = lg0 + wid * G; g0 < lg1; g0 += kWavesPerBlock * G) {
+            const int g = g0 + sub;
+            int32_t gb = 0, ge = 0;
+            if (!idle && g < lg1) {
+                gb = a.lg_task_ptr[g];
+                ge = a.lg_task_ptr[g + 1];
             }
-            // A large output is not read again before the caches have turned over, so its rows are written as
-            // streaming stores (`nt`): they then do not push feature rows out of L2 and the Infinity Cache.
-            // Every lane stores whole 16-byte pieces (8-byte for bf16 output) wherever the piece starts on a 4-byte
-            // boundary -- gfx950 executes global_store_dwordx4 at any dword address, like the loads -- so packed rows
-            // (47 floats = 188 bytes) are written as one contiguous burst per row.  The lane that was shifted back
-            // to stay inside the row rewrites `skip` elements of its neighbour's piece with the same bits (both
-            // lanes sum the same entries in the same order).
-            constexpr bool stream = PHASE == 2;
-            if (PHASE >= 1 && a.out_bf16) {
-                uint16_t *o = reinterpret_cast<uint16_t *>(a.out) + at;
-                if (VEC >= 4 && a.vec_store && (at & 1) == 0) {
+            float part[VEC];
 #pragma unroll
-                    for (int k = 0; k < VEC; k += 4) {
-                        const rof_u2s t = {rof_bf16_bits(r[k]) | (rof_bf16_bits(r[k + 1]) << 16),
-                                           rof_bf16_bits(r[k + 2]) | (rof_bf16_bits(r[k + 3]) << 16)};
-                        if (stream) __builtin_nontemporal_store(t, reinterpret_cast<rof_u2s *>(o + k));
-                        else *reinterpret_cast<rof_u2s *>(o + k) = t;
-                    }
-                } else {
+            for (int k = 0; k < VEC; ++k) part[k] = 0.0f;
+            gather_sum<XT, VEC, LPR, false, false, OFF32, false>(xb, xld, nullptr, 0, 0, 0, a.lg_col, a.lg_w, gb, ge, lane,
+                                                                 sub, li, act, part);
+            if (!idle && g < lg1) {
+                float *row = lds_rows + (g - lg0) * kLdsRow + li * VEC;
 #pragma unroll
-                    for (int k = 0; k < VEC; ++k)
-                        if (k >= skip && cstart + k < a.feat) o[k] = (uint16_t)rof_bf16_bits(r[k]);
-                }
+                for (int k = 0; k < VEC; ++k) row[k] = part[k];
+            }
+        }
+        __syncthreads();
+
+        for (int32_t t0 = ct0 + wid * G; t0 < ct1; t0 += kWavesPerBlock * G) {   // one lane group per task
+            const int32_t t = t0 + sub;
+            const bool valid = !idle && t < ct1;
+            int32_t first = 0, beg = 0, mid = 0, end = 0, nlds = 0;
+            if (valid) {
+                first = a.task_ptr[t];
+                end = a.task_ptr[t + 1];
+                const uint32_t packed = (uint32_t)a.task_nref[t];   // references in the low 24 bits, LDS rows above
+                nlds = (int32_t)(packed >> 24);
+                beg = first + nlds;
+                mid = beg + (int32_t)(packed & 0xffffffu);
+            }
+            float acc[VEC];
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) acc[k] = 0.0f;
+            for (int j = 0; j < nlds; ++j) {
+                const float *row = lds_rows + a.col[first + j] * kLdsRow + li * VEC;
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) acc[k] += row[k];
+            }
+            if (kF32) {
+                if (__any(mid > beg))
+                    gather_sum<XT, VEC, LPR, false, true, OFF32, PHASE == 2>(xb, xld, pb, pld, a.nsplit, 0, a.col, a.w, beg, end,
+                                                                            lane, sub, li, act, acc);
+                else
+                    gather_sum<XT, VEC, LPR, false, false, OFF32, PHASE == 2>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, beg, end,
+                                                                             lane, sub, li, act, acc);
             } else {
-                float *o = reinterpret_cast<float *>(a.out) + at;
-                if (VEC >= 4 && a.vec_store) {
-#pragma unroll
-                    for (int k = 0; k < VEC; k += 4) {
-                        const rof_f4 t = {r[k], r[k + 1], r[k + 2], r[k + 3]};
-                        if (stream) __builtin_nontemporal_store(t, reinterpret_cast<rof_f4 *>(o + k));
-                        else *reinterpret_cast<rof_f4 *>(o + k) = t;
-                    }
-                } else {
-#pragma unroll
-                    for (int k = 0; k < VEC; ++k)
-                        if (k >= skip && cstart + k < a.feat) o[k] = r[k];
-                }
+                if (__any(mid > beg))
+                    gather_sum<float, VEC, LPR, false, false, OFF32, PHASE == 2>(pb, pld, nullptr, 0, 0, a.nsplit, a.col, a.w,
+                                                                                beg, mid, lane, sub, li, act, acc);
+                gather_sum<XT, VEC, LPR, false, false, OFF32, PHASE == 2>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, mid, end, lane,
+                                                                         sub, li, act, acc);
             }
+            if (valid && act) finish_row<XT, VEC, PHASE>(a, t, end > first, acc, xb, xld, cstart, skip);
         }
     }
 }
@@ -394,33 +501,48 @@ inline int rof_lanes_per_row(int feat, int vec) {
     return 64;
 }
 
-template <typename XT, int VEC, int PHASE, bool OFF32>
-int launch_lpr(const AggArgs &a0, int lpr, hipStream_t st) {
+// CLUSTER: a.n_blocks clusters (one workgroup each) that need `lds_rows` LDS rows; otherwise the tasks [0, n_tasks)
+// of `a`, the first n_wave of them long.
+template <typename XT, int VEC, int PHASE, bool OFF32, bool CLUSTER>
+int launch_lpr(const AggArgs &a0, int lpr, int lds_rows, hipStream_t st) {
     AggArgs a = a0;
     const int g = 64 / lpr;
-    const int64_t shorts = (int64_t)a.n_tasks - a.n_wave;
-    const int64_t waves = a.n_wave + (shorts + g - 1) / g;
-    if (waves == 0) return ROF_OK;
-    a.n_blocks = (int32_t)((waves + kWavesPerBlock - 1) / kWavesPerBlock);
+    if (!CLUSTER) {
+        const int64_t shorts = (int64_t)a.n_tasks - a.n_wave;
+        const int64_t waves = a.n_wave + (shorts + g - 1) / g;
+        a.n_blocks = (int32_t)((waves + kWavesPerBlock - 1) / kWavesPerBlock);
+    }
+    if (a.n_blocks == 0) return ROF_OK;
+    // LDS rows of the workgroup-local groups (none: 0 bytes) on top of the benchmark interface's padding
+    const int64_t lds = (int64_t)g_lds_pad + (CLUSTER ? (int64_t)lds_rows * (lpr * VEC + 4) * 4 : 0);
+    if (lds > 64 * 1024) return ROF_ERR_UNSUPPORTED;
     const int64_t span = (int64_t)kXcds * a.xcd_run;
     const int64_t grid = (a.n_blocks + span - 1) / span * span;
     dim3 gr((unsigned)grid), bl(64 * kWavesPerBlock);
+#define ROF_LAUNCH(LPR)                                                                                              \
+    do {                                                                                                             \
+        if constexpr (CLUSTER)                                                                                       \
+            hipLaunchKernelGGL((rof_cluster_kernel<XT, VEC, LPR, PHASE < 1 ? 1 : PHASE, OFF32>), gr, bl, (unsigned)lds, st, a); \
+        else                                                                                                         \
+            hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, LPR, PHASE, OFF32>), gr, bl, (unsigned)lds, st, a);         \
+    } while (0)
     switch (lpr) {
-        case 4: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 4, PHASE, OFF32>), gr, bl, g_lds_pad, st, a); break;
-        case 8: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 8, PHASE, OFF32>), gr, bl, g_lds_pad, st, a); break;
+        case 4: ROF_LAUNCH(4); break;
+        case 8: ROF_LAUNCH(8); break;
         case 10:
-            if constexpr (VEC > 1) hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 10, PHASE, OFF32>), gr, bl, g_lds_pad, st, a);
+            if constexpr (VEC > 1) ROF_LAUNCH(10);
             break;
         case 12:
-            if constexpr (VEC > 1) hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 12, PHASE, OFF32>), gr, bl, g_lds_pad, st, a);
+            if constexpr (VEC > 1) ROF_LAUNCH(12);
             break;
         case 20:
-            if constexpr (VEC > 1) hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 20, PHASE, OFF32>), gr, bl, g_lds_pad, st, a);
+            if constexpr (VEC > 1) ROF_LAUNCH(20);
             break;
-        case 16: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 16, PHASE, OFF32>), gr, bl, g_lds_pad, st, a); break;
-        case 32: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 32, PHASE, OFF32>), gr, bl, g_lds_pad, st, a); break;
-        default: hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, 64, PHASE, OFF32>), gr, bl, g_lds_pad, st, a); break;
+        case 16: ROF_LAUNCH(16); break;
+        case 32: ROF_LAUNCH(32); break;
+        default: ROF_LAUNCH(64); break;
     }
+#undef ROF_LAUNCH
     HIP_TRY(hipGetLastError());
     return ROF_OK;
 }
@@ -429,8 +551,9 @@ int launch_lpr(const AggArgs &a0, int lpr, hipStream_t st) {
 // 2: destination rows with streaming stores.
 // off32: every byte offset into the feature matrix and into the partial-sum workspace fits 32 bits and
 // every row id fits 24 bits, so the kernels may use the short address arithmetic.
-int launch_rows_f32(const AggArgs &a, int phase, int vec, bool off32, hipStream_t st);
-int launch_rows_bf16(const AggArgs &a, int phase, int vec, bool off32, hipStream_t st);
+// lds_rows > 0: the cluster launch (a.n_blocks workgroups, phase >= 1) whose workgroups need that many LDS rows.
+int launch_rows_f32(const AggArgs &a, int phase, int vec, bool off32, int lds_rows, hipStream_t st);
+int launch_rows_bf16(const AggArgs &a, int phase, int vec, bool off32, int lds_rows, hipStream_t st);
 
 }  // namespace rofk
 

@@ -61,6 +61,9 @@ int32_t default_cut(int32_t groups, int32_t elem_bytes) {
 const int64_t kMinSavedBytes = 256000000;
 const int64_t kMinSavedShare = 10;   // net saving >= 1/10 of all gathers
 const int32_t kTileRows = 4096;      // short tasks are length-sorted inside tiles of this many rows
+// A workgroup of clustered destinations is kept when its local groups save at least this many row gathers: below
+// that the two barriers and the serial start of the workgroup cost more than the gathers it avoids.
+const int64_t kMinClusterSaving = 8;
 
 bool ptr_ok(const int32_t *p, int64_t n, int64_t *total) {
     if (!p || p[0] != 0) return false;
@@ -97,24 +100,46 @@ bool v2_is_canonical(const int32_t *uptr, const int32_t *dptr, const int32_t *dc
 }
 
 struct TaskList {   // tasks in natural order, before sorting
-    ivec ptr{0}, nref, out, col;
+    ivec ptr{0}, nref, out, col, nlds;
     void begin_task(int32_t out_row) { out.push_back(out_row); }
-    void end_task(int32_t refs) {
+    void end_task(int32_t refs, int32_t lds_rows = 0) {
         nref.push_back(refs);
+        nlds.push_back(lds_rows);
         ptr.push_back((int32_t)col.size());
     }
 };
 
-// Long tasks first (descending), then short tasks tile by tile, each tile descending.  `groups`: short tasks
-// that share a wavefront.  With `band` (one key per task: the highest source id it gathers) both kinds are
-// ordered by descending key instead.
-void order_tasks(const ivec &ptr, int64_t tile_rows, int32_t groups, const ivec *band, ivec &order, int32_t &n_wave) {
+// Short tasks placed by the schedule builder rather than by the tile order: whole workgroups of destinations that
+// share reuse groups (see build_clusters), with the groups each workgroup sums into LDS.
+struct Clusters {
+    ivec tasks;                       // destination tasks of the cluster section, cluster by cluster
+    ivec task_first{0};               // per cluster: its range in `tasks`
+    int32_t cut = 0;                  // rows up to this many entries counted as short when the clusters were formed
+    ivec lg_ptr{0}, lg_task_ptr{0}, lg_col;   // per workgroup: its local groups; per local group: its sources
+    int32_t max_rows = 0;
+    // destination -> (group, LDS row) pairs served from LDS
+    ivec of_node;                     // index into ptr, or -1
+    ivec ptr{0}, group, row;
+};
+
+// Cut between long tasks (a wavefront each) and short ones (a lane group each) for a launch of these task lengths.
+int32_t short_cut(const int64_t T, const int64_t over, int32_t groups) {
+    return over + (T - over + groups - 1) / groups >= kWavesToFill ? kShortRow : kShortRowSmall;
+}
+
+// Long tasks first (descending), then the short tasks tile by tile, each tile descending, and last the tasks of
+// `placed` in their given order (the clustered short tasks, may be null).  `groups`: short tasks that share a
+// wavefront.  With `band` (one key per task: the highest source id it gathers) both kinds are ordered by descending
+// key instead.
+void order_tasks(const ivec &ptr, int64_t tile_rows, int32_t groups, const ivec *band, const ivec *placed, int32_t fixed_cut,
+                 ivec &order, int32_t &n_wave) {
     int64_t T = (int64_t)ptr.size() - 1;
     order.clear();
     order.reserve(T);
     int64_t over = 0;
     for (int64_t t = 0; t < T; ++t) over += ptr[t + 1] - ptr[t] > kShortRow;
-    const int32_t cut = over + (T - over + groups - 1) / groups >= kWavesToFill ? kShortRow : kShortRowSmall;
+    // (`placed` tasks were chosen as short ones against `fixed_cut`, which then has to be the cut used here)
+    const int32_t cut = fixed_cut > 0 ? fixed_cut : short_cut(T, over, groups);
     ivec longs;
     for (int64_t t = 0; t < T; ++t)
         if (ptr[t + 1] - ptr[t] > cut) longs.push_back((int32_t)t);
@@ -134,19 +159,26 @@ void order_tasks(const ivec &ptr, int64_t tile_rows, int32_t groups, const ivec 
                      [&ptr](int32_t x, int32_t y) { return ptr[x + 1] - ptr[x] > ptr[y + 1] - ptr[y]; });
     n_wave = (int32_t)longs.size();
     order = longs;
+    std::vector<char> taken;
+    if (placed && !placed->empty()) {
+        taken.assign(T, 0);
+        for (int32_t t : *placed) taken[t] = 1;
+    }
     std::vector<ivec> bucket(cut + 1);
     for (int64_t t0 = 0; t0 < T; t0 += tile_rows) {
         int64_t t1 = std::min(T, t0 + tile_rows);
         for (auto &b : bucket) b.clear();
         for (int64_t t = t0; t < t1; ++t) {
             int32_t len = ptr[t + 1] - ptr[t];
-            if (len <= cut) bucket[len].push_back((int32_t)t);
+            if (len <= cut && (taken.empty() || !taken[t])) bucket[len].push_back((int32_t)t);
         }
         for (int32_t len = cut; len >= 0; --len) order.insert(order.end(), bucket[len].begin(), bucket[len].end());
     }
+    if (placed) order.insert(order.end(), placed->begin(), placed->end());
 }
 
-void finalize_phase(const TaskList &tl, int64_t tile_rows, int32_t groups, bool by_band, rof_phase_host &ph) {
+void finalize_phase(const TaskList &tl, int64_t tile_rows, int32_t groups, bool by_band, rof_phase_host &ph,
+                    const Clusters *cl = nullptr) {
     int64_t T = (int64_t)tl.out.size();
     ivec order, band;
     if (by_band) {
@@ -156,8 +188,21 @@ void finalize_phase(const TaskList &tl, int64_t tile_rows, int32_t groups, bool 
             band[t] = first < tl.ptr[t + 1] ? tl.col[first] : -1;
         }
     }
-    order_tasks(tl.ptr, tile_rows, groups, by_band ? &band : nullptr, order, ph.n_wave);
+    order_tasks(tl.ptr, tile_rows, groups, by_band ? &band : nullptr, cl ? &cl->tasks : nullptr,
+                (cl && !cl->tasks.empty()) ? cl->cut : 0, order, ph.n_wave);
     ph.n_tasks = (int32_t)T;
+    ph.n_regular = ph.n_tasks;
+    if (cl && !cl->tasks.empty()) {
+        ph.n_regular = ph.n_tasks - (int32_t)cl->tasks.size();
+        ph.lg_blocks = (int32_t)cl->lg_ptr.size() - 1;
+        ph.lg_task_first = cl->task_first;
+        for (int32_t &f : ph.lg_task_first) f += ph.n_regular;   // positions in the ordered task list
+        ph.lg_ptr = cl->lg_ptr;
+        ph.lg_task_ptr = cl->lg_task_ptr;
+        ph.lg_col = cl->lg_col;
+        ph.lg_max_rows = cl->max_rows;
+        ph.task_nlds.resize(T);
+    }
     ph.task_ptr.assign(T + 1, 0);
     ph.task_nref.resize(T);
     ph.task_out.resize(T);
@@ -166,6 +211,7 @@ void finalize_phase(const TaskList &tl, int64_t tile_rows, int32_t groups, bool 
         ph.task_ptr[i + 1] = ph.task_ptr[i] + (tl.ptr[t + 1] - tl.ptr[t]);
         ph.task_nref[i] = tl.nref[t];
         ph.task_out[i] = tl.out[t];
+        if (!ph.task_nlds.empty()) ph.task_nlds[i] = tl.nlds[t];
     }
     ph.col.resize(tl.col.size());
 #pragma omp parallel for schedule(dynamic, 4096)
@@ -173,6 +219,149 @@ void finalize_phase(const TaskList &tl, int64_t tile_rows, int32_t groups, bool 
         int32_t t = order[i];
         int32_t len = tl.ptr[t + 1] - tl.ptr[t];
         if (len) memcpy(ph.col.data() + ph.task_ptr[i], tl.col.data() + tl.ptr[t], (size_t)len * sizeof(int32_t));
+    }
+}
+
+// Workgroup-local reuse.  A reuse group whose consumers sit in one workgroup is summed once by that workgroup into
+// LDS and read from there by each consumer: no partial row travels through memory and no launch is added (upstream
+// keeps the partial sum of a part in shared memory too and fans it out with atomics, reuse_conv_kernel.cu:876-952;
+// here the consumers come to the partial sum instead).  The schedule builder is free to order destination tasks, so
+// it brings consumers together: the short destinations (one lane group each) that consume a group with at least two
+// such consumers are sorted by the first such group they consume and cut into clusters of up to kClusterTasks
+// (preferably where the group changes); one workgroup works through a cluster's tasks in rounds.  In every cluster
+// the groups that at least two of its destinations consume become local groups, most saving first, as far as the
+// LDS rows go.  Clusters that save fewer than `min_saving` row gathers are dissolved (their destinations return to
+// the tile order).  full_len[v]: entries of destination v with every group expanded.
+const int32_t kClusterTasks = 64;
+// One workgroup works through a cluster alone, 4 * `groups` tasks at a time, so a cluster is also limited by its
+// work: at most this many entries per lane group.  (Clusters of 64 rows of up to 64 entries each at one row per
+// wavefront took longer than the whole launch of all other rows.)
+const int32_t kClusterDepth = 96;
+// The clusters run as a launch of their own (~8 us with its tail on MI355X): they are kept only if together they
+// save at least this many bytes of row gathers.
+const int64_t kMinLocalSavedBytes = 64000000;
+
+void build_clusters(const rof_layout *L, const ivec &ng_ptr, const ivec &ng, const ivec &full_len, int32_t cut,
+                    int32_t groups, int32_t max_rows, int64_t min_saving, Clusters &cl) {
+    const int32_t n = L->n;
+    const int64_t G = (int64_t)L->group_ptr.size() - 1;
+    cl.of_node.assign(n, -1);
+    if (G == 0) return;
+    auto glen = [&](int32_t g) { return L->group_ptr[g + 1] - L->group_ptr[g]; };
+    // groups with at least two short consumers
+    ivec short_consumers(G, 0);
+    for (int32_t v = 0; v < n; ++v)
+        if (full_len[v] <= cut)
+            for (int32_t j = ng_ptr[v]; j < ng_ptr[v + 1]; ++j) short_consumers[ng[j]]++;
+    struct Cand { int32_t key, len, v; };
+    std::vector<Cand> cand;
+    for (int32_t v = 0; v < n; ++v) {
+        if (full_len[v] > cut) continue;
+        for (int32_t j = ng_ptr[v]; j < ng_ptr[v + 1]; ++j)
+            if (short_consumers[ng[j]] >= 2 && glen(ng[j]) >= 2) {
+                cand.push_back({ng[j], full_len[v], v});   // ng lists a node's groups in ascending order
+                break;
+            }
+    }
+    if ((int64_t)cand.size() < 2) return;
+    std::sort(cand.begin(), cand.end(), [](const Cand &a, const Cand &b) {
+        return a.key != b.key ? a.key < b.key : a.len != b.len ? a.len > b.len : a.v < b.v;
+    });
+    ivec count(G, 0), touched, pick;
+    ivec row_of(G, -1);
+    size_t b0 = 0;
+    while (b0 < cand.size()) {
+        // whole runs of destinations with the same first group while they fit -- by tasks, and by the LDS rows
+        // their shared groups need; a run that does not fit is split only if the cluster would otherwise stay
+        // less than half full
+        size_t b1 = b0;
+        int32_t shared = 0;   // groups that at least two destinations of the cluster consume
+        int64_t work = 0;     // entries of the cluster's rows
+        const int64_t max_work = (int64_t)4 * groups * kClusterDepth;
+        touched.clear();
+        auto add = [&](size_t i0, size_t i1) {
+            for (size_t i = i0; i < i1; ++i)
+                for (int32_t j = ng_ptr[cand[i].v]; j < ng_ptr[cand[i].v + 1]; ++j) {
+                    const int32_t c = count[ng[j]]++;
+                    if (c == 0) touched.push_back(ng[j]);
+                    shared += c == 1 && glen(ng[j]) >= 2;
+                }
+        };
+        auto remove = [&](size_t i0, size_t i1) {
+            for (size_t i = i0; i < i1; ++i)
+                for (int32_t j = ng_ptr[cand[i].v]; j < ng_ptr[cand[i].v + 1]; ++j)
+                    shared -= --count[ng[j]] == 1 && glen(ng[j]) >= 2;
+        };
+        while (b1 < cand.size() && b1 - b0 < (size_t)kClusterTasks) {
+            size_t run = b1;
+            while (run < cand.size() && cand[run].key == cand[b1].key) ++run;
+            if (run - b0 > (size_t)kClusterTasks) {
+                if (b1 - b0 >= (size_t)kClusterTasks / 2) break;
+                run = b0 + kClusterTasks;
+            }
+            int64_t run_work = 0;
+            for (size_t i = b1; i < run; ++i) {
+                run_work += cand[i].len;
+                if (work + run_work > max_work && i > b0 + 1) {   // the part of the run that still fits (two rows at least)
+                    run_work -= cand[i].len;
+                    run = i;
+                    break;
+                }
+            }
+            if (run == b1) break;
+            work += run_work;
+            add(b1, run);
+            if (shared > max_rows && b1 > b0) {   // this run's groups no longer fit into the LDS rows
+                remove(b1, run);
+                break;
+            }
+            b1 = run;
+            if (work >= max_work) break;
+        }
+        pick.clear();
+        for (int32_t g : touched)
+            if (count[g] >= 2 && glen(g) >= 2) pick.push_back(g);
+        std::sort(pick.begin(), pick.end(), [&](int32_t a, int32_t b) {
+            const int64_t sa = (int64_t)(count[a] - 1) * glen(a), sb = (int64_t)(count[b] - 1) * glen(b);
+            return sa != sb ? sa > sb : a < b;
+        });
+        if ((int32_t)pick.size() > max_rows) pick.resize(max_rows);
+        int64_t saving = 0;
+        for (int32_t g : pick) saving += (int64_t)(count[g] - 1) * glen(g) - count[g] / 4;   // four LDS reads ~ one gather
+        if (!pick.empty() && saving >= min_saving) {
+            for (size_t r = 0; r < pick.size(); ++r) {
+                row_of[pick[r]] = (int32_t)r;
+                cl.lg_col.insert(cl.lg_col.end(), L->group_col.begin() + L->group_ptr[pick[r]],
+                                 L->group_col.begin() + L->group_ptr[pick[r] + 1]);
+                cl.lg_task_ptr.push_back((int32_t)cl.lg_col.size());
+            }
+            cl.lg_ptr.push_back((int32_t)cl.lg_task_ptr.size() - 1);
+            cl.max_rows = std::max(cl.max_rows, (int32_t)pick.size());
+            // inside the cluster: by what is left of each row, longest first, so that the lane groups that share
+            // a wavefront finish together
+            std::vector<std::pair<int32_t, int32_t>> rest;   // (remaining entries, destination)
+            for (size_t i = b0; i < b1; ++i) {
+                const int32_t v = cand[i].v;
+                int32_t len = full_len[v];
+                cl.of_node[v] = (int32_t)cl.ptr.size() - 1;
+                for (int32_t j = ng_ptr[v]; j < ng_ptr[v + 1]; ++j)
+                    if (row_of[ng[j]] >= 0) {
+                        cl.group.push_back(ng[j]);
+                        cl.row.push_back(row_of[ng[j]]);
+                        len -= glen(ng[j]) - 1;
+                    }
+                cl.ptr.push_back((int32_t)cl.group.size());
+                rest.push_back({len, v});
+            }
+            std::sort(rest.begin(), rest.end(), [](const std::pair<int32_t, int32_t> &a, const std::pair<int32_t, int32_t> &b) {
+                return a.first != b.first ? a.first > b.first : a.second < b.second;
+            });
+            for (auto &p : rest) cl.tasks.push_back(p.second);
+            cl.task_first.push_back((int32_t)cl.tasks.size());
+            for (int32_t g : pick) row_of[g] = -1;
+        }
+        for (int32_t g : touched) count[g] = 0;
+        b0 = b1;
     }
 }
 
@@ -203,8 +392,47 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
             for (int32_t j = L->group_dst_ptr[g]; j < L->group_dst_ptr[g + 1]; ++j) ng[at[L->group_dst[j]]++] = (int32_t)g;
     }
 
-    // Which groups are computed once and shared.  A group is worth a partial-sum row when the row
-    // gathers it saves exceed the partial-row reads plus the one write it adds.
+    // Workgroup-local sharing first (cost-model mode only): consumers that the schedule can bring together in one
+    // workgroup take the group's sum from LDS; what is decided below for the partial-sum workspace then concerns
+    // the remaining consumers only.
+    Clusters cl;
+    cl.of_node.assign(n, -1);
+    const int32_t local_groups = o ? o->local_groups : 0;
+    ivec served(G, 0);   // consumers of each group that read it from LDS
+    if (!disable && min_consumers == 0 && local_groups >= 0 && G > 0) {
+        ivec full_len(n);
+        int64_t over = 0;
+        for (int32_t v = 0; v < n; ++v) {
+            int64_t len = L->res_ptr[v + 1] - L->res_ptr[v];
+            for (int32_t j = ng_ptr[v]; j < ng_ptr[v + 1]; ++j) len += L->group_ptr[ng[j] + 1] - L->group_ptr[ng[j]];
+            full_len[v] = (int32_t)std::min<int64_t>(len, INT32_MAX);
+            const int64_t task_len = len > hub_split ? (len + segment - 1) / segment : len;
+            over += task_len > kShortRow;
+        }
+        // sharing only shortens rows, so a row that is short now stays short, and rows above the segment cut are
+        // no candidates
+        const int32_t cut = short_cut(n, over, groups);
+        cl.cut = cut;
+        // LDS rows per workgroup: 16 KB at the width this layout is built for, at most 32 rows (a kernel that is
+        // launched at a greater width than that still stays within the 64 KB a workgroup may ask for)
+        const int32_t row_bytes = lpr * 16 * ((o && o->elem_bytes == 2) ? 2 : 1);
+        const int32_t max_rows = std::max(4, std::min(32, (16 << 10) / row_bytes));
+        build_clusters(L, ng_ptr, ng, full_len, std::min(cut, hub_split), groups, max_rows, local_groups > 0 ? local_groups : kMinClusterSaving, cl);
+        for (int32_t v = 0; v < n; ++v)
+            if (cl.of_node[v] >= 0)
+                for (int32_t j = cl.ptr[cl.of_node[v]]; j < cl.ptr[cl.of_node[v] + 1]; ++j) served[cl.group[j]]++;
+        // what the clusters save: every consumer's copy of a local group's sources but the one the cluster gathers
+        int64_t local_saved = -(int64_t)cl.lg_col.size();
+        for (int64_t g = 0; g < G; ++g) local_saved += (int64_t)served[g] * (L->group_ptr[g + 1] - L->group_ptr[g]);
+        if (local_groups == 0 && local_saved * lpr * 16 < kMinLocalSavedBytes) {   // not worth a launch of their own
+            cl = Clusters();
+            cl.of_node.assign(n, -1);
+            std::fill(served.begin(), served.end(), 0);
+        }
+    }
+
+    // Which groups are computed once and shared through the workspace.  A group is worth a partial-sum row when the
+    // row gathers it saves exceed the partial-row reads plus the one write it adds.
     auto worth = [&](int64_t cnt, int64_t len) {
         if (disable) return false;
         if (min_consumers < 0) return true;   // every group, even one nobody consumes (v1 cache rows)
@@ -215,7 +443,7 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     // a plan whose sharing would not repay its extra launch is executed with every group folded back
     int64_t saved = 0;
     for (int64_t g = 0; g < G; ++g) {
-        int64_t cnt = L->group_dst_ptr[g + 1] - L->group_dst_ptr[g], len = L->group_ptr[g + 1] - L->group_ptr[g];
+        int64_t cnt = L->group_dst_ptr[g + 1] - L->group_dst_ptr[g] - served[g], len = L->group_ptr[g + 1] - L->group_ptr[g];
         if (worth(cnt, len)) saved += (cnt - 1) * len - cnt;
     }
     const bool too_small = min_consumers == 0 && (saved * lpr * 16 < kMinSavedBytes ||   // a lane holds 16 bytes of a row
@@ -225,7 +453,7 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     TaskList tg, ts, tb;
     for (int64_t g = 0; g < G; ++g) {
         if (too_small) break;
-        if (!worth(L->group_dst_ptr[g + 1] - L->group_dst_ptr[g], L->group_ptr[g + 1] - L->group_ptr[g])) continue;
+        if (!worth(L->group_dst_ptr[g + 1] - L->group_dst_ptr[g] - served[g], L->group_ptr[g + 1] - L->group_ptr[g])) continue;
         slot_of[g] = (int32_t)slots++;
         tg.begin_task(slot_of[g]);
         tg.col.insert(tg.col.end(), L->group_col.begin() + L->group_ptr[g], L->group_col.begin() + L->group_ptr[g + 1]);
@@ -237,35 +465,46 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     tb.nref.reserve(n);
     tb.out.reserve(n);
     tb.col.reserve(L->res_col.size() + L->group_dst.size());
-    int64_t gathered = (int64_t)tg.col.size(), reads = 0, segments = 0, nearby = 0;
-    ivec row;   // one destination's entries: references first, then feature rows
+    int64_t gathered = (int64_t)tg.col.size() + (int64_t)cl.lg_col.size(), reads = 0, segments = 0, nearby = 0, lds_reads = 0;
+    ivec row;   // one destination's entries: LDS rows first, then references, then feature rows
+    ivec local_row(G, -1);
     for (int32_t v = 0; v < n; ++v) {
         row.clear();
-        int32_t refs = 0;
+        int32_t refs = 0, nlds = 0;
+        if (cl.of_node[v] >= 0)
+            for (int32_t j = cl.ptr[cl.of_node[v]]; j < cl.ptr[cl.of_node[v] + 1]; ++j) {
+                local_row[cl.group[j]] = cl.row[j];
+                row.push_back(cl.row[j]);
+                ++nlds;
+            }
         for (int32_t j = ng_ptr[v]; j < ng_ptr[v + 1]; ++j)
-            if (slot_of[ng[j]] >= 0) {
+            if (local_row[ng[j]] < 0 && slot_of[ng[j]] >= 0) {
                 row.push_back(n + slot_of[ng[j]]);
                 ++refs;
             }
         for (int32_t j = ng_ptr[v]; j < ng_ptr[v + 1]; ++j) {
             int32_t g = ng[j];
-            if (slot_of[g] < 0)
+            if (local_row[g] < 0 && slot_of[g] < 0)
                 row.insert(row.end(), L->group_col.begin() + L->group_ptr[g], L->group_col.begin() + L->group_ptr[g + 1]);
         }
+        if (nlds)
+            for (int32_t j = cl.ptr[cl.of_node[v]]; j < cl.ptr[cl.of_node[v] + 1]; ++j) local_row[cl.group[j]] = -1;
         row.insert(row.end(), L->res_col.begin() + L->res_ptr[v], L->res_col.begin() + L->res_ptr[v + 1]);
         // The order of the summands is free.  Walking the feature matrix monotonically keeps consecutive
         // gathers of a task close in memory (same pages, neighbouring lines); measured on MI355X against the
         // plan's own order: descending ids 2-3 % faster, ascending 1 % faster, a random order 20 % slower.
-        if (entry_order == 0) std::sort(row.begin() + refs, row.end(), std::greater<int32_t>());
-        else if (entry_order == 2) std::sort(row.begin() + refs, row.end());
+        if (entry_order == 0) std::sort(row.begin() + nlds + refs, row.end(), std::greater<int32_t>());
+        else if (entry_order == 2) std::sort(row.begin() + nlds + refs, row.end());
         const int64_t len = (int64_t)row.size();
-        for (int64_t j = refs; j < len; ++j) nearby += std::abs(row[j] - v) < 2 * kTileRows;
-        gathered += len - refs;
+        for (int64_t j = nlds + refs; j < len; ++j) nearby += std::abs(row[j] - v) < 2 * kTileRows;
+        gathered += len - refs - nlds;
         reads += refs;
+        lds_reads += nlds;
         tb.begin_task(v);
         if (len > hub_split) {
             // A long row is cut into segments; each becomes a partial-sum task of the middle launch
             // (after the groups it may reference, before the rows), and the row itself just adds them up.
+            // (Rows served from LDS are short: nlds is 0 here.)
             int32_t nseg = 0;
             for (int64_t s0 = 0; s0 < len; s0 += segment) {
                 int64_t s1 = std::min<int64_t>(len, s0 + segment);
@@ -281,7 +520,7 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
             tb.end_task(nseg);
         } else {
             tb.col.insert(tb.col.end(), row.begin(), row.end());
-            tb.end_task(refs);
+            tb.end_task(refs, nlds);
         }
     }
     if (slots + (int64_t)n >= INT32_MAX || tb.col.size() >= (size_t)INT32_MAX) return ROF_ERR_UNSUPPORTED;
@@ -299,7 +538,9 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     L->partial_reads = reads;
     finalize_phase(tg, 1 << 30, groups, false, L->g);
     finalize_phase(ts, 1 << 30, groups, entry_order == 0, L->s);   // the sweep needs the descending lists
-    finalize_phase(tb, tile_rows, groups, false, L->b);
+    finalize_phase(tb, tile_rows, groups, false, L->b, &cl);
+    L->n_local_groups = (int64_t)cl.lg_task_ptr.size() - 1;
+    L->lds_reads = lds_reads;
     L->gathered_before_rows = (int64_t)tg.col.size();
     for (size_t t = 0; t < ts.out.size(); ++t) L->gathered_before_rows += (ts.ptr[t + 1] - ts.ptr[t]) - ts.nref[t];
     return ROF_OK;
@@ -519,6 +760,13 @@ int rof_layout_export(const rof_layout *L, rof_bag **out) {
         put("b_task_nref", L->b.task_nref);
         put("b_task_out", L->b.task_out);
         put("b_col", L->b.col);
+        put("b_task_nlds", L->b.task_nlds);
+        put("b_lg_ptr", L->b.lg_ptr);
+        put("b_lg_task_ptr", L->b.lg_task_ptr);
+        put("b_lg_col", L->b.lg_col);
+        put("b_lg_task_first", L->b.lg_task_first);
+        bag->arr["b_shape"] = {(uint32_t)L->b.n_wave, (uint32_t)L->b.n_regular, (uint32_t)L->b.lg_blocks,
+                               (uint32_t)L->b.lg_max_rows};
     } catch (const std::bad_alloc &) {
         delete bag;
         return ROF_ERR_ALLOC;
@@ -527,9 +775,9 @@ int rof_layout_export(const rof_layout *L, rof_bag **out) {
     return ROF_OK;
 }
 
-int rof_layout_stats(const rof_layout *L, int64_t s[16]) {
+int rof_layout_stats(const rof_layout *L, int64_t s[20]) {
     if (!L || !s) return ROF_ERR_ARG;
-    memset(s, 0, 16 * sizeof(int64_t));
+    memset(s, 0, 20 * sizeof(int64_t));
     s[0] = L->n;
     s[1] = L->e_orig;
     s[2] = (int64_t)L->group_ptr.size() - 1;
@@ -546,6 +794,10 @@ int rof_layout_stats(const rof_layout *L, int64_t s[16]) {
     s[13] = L->b.n_wave;
     s[14] = L->canonical ? 1 : 0;
     s[15] = L->gathered_before_rows;
+    s[16] = L->n_local_groups;
+    s[17] = L->lds_reads;
+    s[18] = L->b.lg_blocks;
+    s[19] = L->b.lg_blocks > 0 ? L->b.lg_max_rows : 0;
     return ROF_OK;
 }
 

@@ -16,10 +16,23 @@ struct rof_bag {
 // (ids >= the node count, pointing into the workspace), the rest are feature rows -- and writes
 // their weighted sum to output row task_out[t].  Tasks [0, n_wave) are long and get a whole
 // wavefront each; the remaining ones are short and share a wavefront.
+//
+// Destination-row phase only: workgroup-local reuse groups.  The tasks [n_regular, n_tasks) at the end of the list
+// are *clustered*: destinations that share reuse groups, brought together by the schedule builder and run by a
+// launch of their own, one workgroup per cluster.  Cluster i has the tasks lg_task_first[i] .. lg_task_first[i+1]
+// (any number of short tasks, worked through in rounds).  Its workgroup first sums the cluster's local groups
+// lg_ptr[i] .. lg_ptr[i+1] into LDS rows 0, 1, ... (local group j gathers lg_col[lg_task_ptr[j] ..
+// lg_task_ptr[j+1])), and the tasks then take those partial sums from LDS: the first task_nlds[t] entries of such
+// a task are LDS row numbers (before the task_nref[t] partial-sum rows and the feature rows).
 struct rof_phase_host {
     std::vector<int32_t> task_ptr, task_nref, task_out, col;
     int32_t n_wave = 0;
     int32_t n_tasks = 0;
+    std::vector<int32_t> task_nlds;                  // empty: no task reads LDS rows
+    std::vector<int32_t> lg_ptr, lg_task_ptr, lg_col, lg_task_first;
+    int32_t n_regular = 0;                           // tasks of the ordinary launch (= n_tasks without clusters)
+    int32_t lg_blocks = 0;                           // clusters
+    int32_t lg_max_rows = 0;                         // most LDS rows any cluster needs
 };
 
 struct rof_phase_dev {
@@ -28,6 +41,11 @@ struct rof_phase_dev {
     float *scale = nullptr;   // per task: rsqrt(deg[task_out]) (destination rows only)
     int32_t n_wave = 0, n_tasks = 0;
     int64_t n_entries = 0;
+    // workgroup-local groups (destination rows only); task_nref then carries task_nlds in its top 8 bits
+    int32_t *lg_ptr = nullptr, *lg_task_ptr = nullptr, *lg_col = nullptr, *lg_task_first = nullptr;
+    float *lg_w = nullptr;
+    int64_t lg_entries = 0;
+    int32_t n_regular = 0, lg_blocks = 0, lg_max_rows = 0;
 };
 
 struct rof_layout {
@@ -43,6 +61,7 @@ struct rof_layout {
     int32_t xcd_run = 16;     // consecutive workgroups of the destination-row launch kept on one XCD
     int64_t n_slots = 0;      // rows of the partial-sum workspace
     int64_t n_materialised = 0, n_segments = 0, gathered_rows = 0, partial_reads = 0, gathered_before_rows = 0;
+    int64_t n_local_groups = 0, lds_reads = 0;   // workgroup-local groups (summed into LDS) and the reads of them
     // device copies
     rof_phase_dev dg, ds, db;
     bool uploaded = false, weights_set = false;

@@ -18,12 +18,13 @@ NOALLOC_WORKSPACE_BYTES = 64 << 20   # ROF_NOALLOC_WORKSPACE_BYTES of include/ro
 
 STAT_NAMES = ("nodes", "edges", "groups", "materialised_groups", "gathered_rows", "partial_reads", "partial_rows",
               "hub_segments", "tasks_a", "tasks_b", "device_bytes", "part_size", "wave_tasks_a", "wave_tasks_b",
-              "canonical", "gathered_rows_a")
+              "canonical", "gathered_rows_a", "local_groups", "lds_reads", "cluster_workgroups", "lds_rows")
 
 EXPORT_NAMES = ("group_ptr", "group_col", "group_dst_ptr", "group_dst", "res_ptr", "res_col", "canonical", "xcd_run",
                 "uniqpart_column_index", "uniqpart_pointers", "part2Node_ptr", "part2Node_col",
                 "g_task_ptr", "g_task_nref", "g_task_out", "g_col", "s_task_ptr", "s_task_nref", "s_task_out", "s_col",
-                "b_task_ptr", "b_task_nref", "b_task_out", "b_col")
+                "b_task_ptr", "b_task_nref", "b_task_out", "b_col", "b_task_nlds", "b_lg_ptr", "b_lg_task_ptr", "b_lg_col", "b_lg_task_first",
+                "b_shape")
 
 
 def column_sums(t):
@@ -61,7 +62,7 @@ ENTRY_ORDERS = {"descending": 0, "plan": 1, "ascending": 2}
 
 
 def _opts(min_consumers=0, disable_reuse=False, hub_split=0, segment=0, lanes_per_row=0, entry_order="descending",
-          tile_rows=0, elem_bytes=0):
+          tile_rows=0, elem_bytes=0, local_groups=0):
     o = LayoutOpts()
     o.min_consumers = int(min_consumers)
     o.disable_reuse = int(bool(disable_reuse))
@@ -71,6 +72,7 @@ def _opts(min_consumers=0, disable_reuse=False, hub_split=0, segment=0, lanes_pe
     o.entry_order = ENTRY_ORDERS[entry_order]
     o.tile_rows = int(tile_rows)
     o.elem_bytes = int(elem_bytes)
+    o.local_groups = int(local_groups)
     return o
 
 
@@ -163,10 +165,12 @@ class Layout:
         r = bag_take(h, EXPORT_NAMES, dtype=np.int32)
         r["canonical"] = bool(r["canonical"][0])
         r["xcd_run"] = int(r["xcd_run"][0])
+        r["b_shape"] = dict(zip(("n_wave", "n_regular", "lg_blocks", "lg_max_rows"),
+                                (int(v) for v in r["b_shape"])))
         return r
 
     def stats(self):
-        s = (C.c_int64 * 16)()
+        s = (C.c_int64 * 20)()
         check(_lib.lib().rof_layout_stats(self._h, s))
         return {k: int(s[i]) for i, k in enumerate(STAT_NAMES)}
 

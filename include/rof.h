@@ -34,7 +34,7 @@ typedef enum {
 
 const char *rof_strerror(int status);
 const char *rof_last_device_error(void); /* thread-local text of the last HIP failure */
-int rof_version(void);
+int rof_version(void);   /* 2: rof_layout_opts has local_groups, rof_layout_stats fills 20 counters */
 
 /* ------------------------------------------------------------------------------------------
  * Host side 1: the reuse-plan builder.  Stays on the CPU (OpenMP); every array is bit-exact
@@ -142,6 +142,10 @@ typedef struct {
     int32_t elem_bytes;      /* bytes per element of the rows that will be gathered: 4 (float32, also 0) or 2        */
                              /* (bfloat16, whose partial-sum rows are twice as wide as its gathered rows).  Steers   */
                              /* the default hub_split.                                                              */
+    int32_t local_groups;    /* workgroup-local sharing (min_consumers = 0 only): short destinations that consume the */
+                             /* same groups are placed in one workgroup, which sums those groups once into LDS;      */
+                             /* 0 = on, a workgroup must save at least 8 row gathers; k > 0 = at least k; -1 = off    */
+    int32_t reserved[3];
 } rof_layout_opts;
 
 /* v2 tensors: replaces the plan arguments of reuse_forward_v2 / reuse_backward_v2
@@ -165,16 +169,21 @@ int rof_layout_from_parts(const int32_t *column_index, const int32_t *part_point
 
 /* Canonical arrays of the layout (host copies, int32 viewed as uint32):
  *   "group_ptr"[G+1] "group_col"  "group_dst_ptr"[G+1] "group_dst"  "res_ptr"[N+1] "res_col"
+ * the schedule of the three launches ("g_*", "s_*", "b_*": task_ptr, task_nref, task_out, col; for the destination
+ * rows also "b_task_nlds", "b_lg_ptr", "b_lg_task_ptr", "b_lg_col", "b_lg_task_first" and "b_shape" = long tasks, tasks of
+ * the ordinary launch, clusters, LDS rows per cluster)
  * and the v2 tensors reconstructed from them ("uniqpart_column_index", "uniqpart_pointers",
  * "part2Node_ptr", "part2Node_col"), which equal the input of rof_layout_from_v2 bit for bit
  * whenever that input has the upstream builder's canonical shape. */
 int rof_layout_export(const rof_layout *layout, rof_bag **out);
 
-/* Counters: [0] nodes [1] original edges [2] groups [3] materialised groups [4] gathered rows per
+/* Counters: [0] nodes [1] original edges [2] groups [3] groups materialised in the workspace [4] gathered rows per
  * pass (E_u) [5] partial-row reads (R) [6] partial rows written (incl. hub segments) [7] hub segments
  * [8] phase-A tasks [9] phase-B tasks [10] device bytes held [11] part_size [12] long tasks of launch 1 [13] of launch 2
- * [14] canonical flag [15] rows gathered by launch 1. */
-int rof_layout_stats(const rof_layout *layout, int64_t stats[16]);
+ * [14] canonical flag [15] rows gathered by launch 1 [16] workgroup-local groups (summed into LDS; a group counts once
+ * per workgroup that sums it) [17] reads of them [18] workgroups that hold clustered destinations [19] LDS rows the
+ * destination-row launch asks for per workgroup. */
+int rof_layout_stats(const rof_layout *layout, int64_t stats[20]);
 
 /* Copy the schedule to the current HIP device (idempotent). */
 int rof_layout_upload(rof_layout *layout, void *stream);

@@ -81,19 +81,50 @@ def case_inputs(c):
 
 
 def emulate_schedule(ex, n, x, w_of, s_of, n_slots):
-    """Run the exported schedule (groups, segments, rows) in float64 numpy, checking its structure."""
+    """Run the exported schedule (groups, segments, rows) in float64 numpy, checking its structure: references only
+    to partial rows that an earlier launch wrote, one writer per output row, LDS rows only inside the cluster
+    (workgroup) that sums them."""
     feat = x.shape[1]
     part = np.zeros((n_slots, feat))
     written = np.zeros(n_slots, dtype=bool)
     out = np.zeros((n, feat))
     for ph in ("g", "s", "b"):
         tp, nr, to, col = ex[ph + "_task_ptr"], ex[ph + "_task_nref"], ex[ph + "_task_out"], ex[ph + "_col"]
+        nlds = ex.get("b_task_nlds") if ph == "b" else None
+        if nlds is None or len(nlds) == 0:
+            nlds = np.zeros(len(to), dtype=np.int64)
+        block_of, lds = None, {}
+        if ph == "b" and ex.get("b_shape", {}).get("lg_blocks", 0) > 0:
+            sh = ex["b_shape"]
+            tf = ex["b_lg_task_first"]
+            assert len(tf) == sh["lg_blocks"] + 1 and tf[0] == sh["n_regular"] >= sh["n_wave"] and (np.diff(tf) >= 2).all()
+            assert tf[-1] == len(to)
+
+            def block_of(t):   # cluster that owns task t, or None
+                b = int(np.searchsorted(tf, t, side="right")) - 1
+                return b if 0 <= b < sh["lg_blocks"] else None
+            lp, ltp, lcol = ex["b_lg_ptr"], ex["b_lg_task_ptr"], ex["b_lg_col"]
+            assert len(lp) == sh["lg_blocks"] + 1 and lp[0] == 0 and lp[-1] == len(ltp) - 1
+            for b in range(sh["lg_blocks"]):
+                rows = []
+                assert 0 < lp[b + 1] - lp[b] <= sh["lg_max_rows"]
+                for j in range(lp[b], lp[b + 1]):
+                    acc = np.zeros(feat)
+                    for i in range(ltp[j], ltp[j + 1]):
+                        assert 0 <= lcol[i] < n
+                        acc += w_of(lcol[i]) * x[lcol[i]]
+                    rows.append(acc)
+                lds[b] = rows
         seen = set()
         for t in range(len(to)):
             acc = np.zeros(feat)
             for i in range(tp[t], tp[t + 1]):
                 c = col[i]
-                if i < tp[t] + nr[t]:
+                if i < tp[t] + nlds[t]:
+                    rows = lds.get(block_of(t))
+                    assert rows is not None and 0 <= c < len(rows), "LDS row outside the workgroup that sums it"
+                    acc += rows[c]
+                elif i < tp[t] + nlds[t] + nr[t]:
                     assert c >= n and written[c - n], "reference to a partial row that is not ready"
                     acc += part[c - n]
                 else:

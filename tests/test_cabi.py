@@ -75,7 +75,7 @@ def test_error_codes_and_messages():
     assert L.rof_column_sums_workspace_bytes(1000, 47) == 2048 * 47 * 4 and L.rof_column_sums_workspace_bytes(0, 47) == 0
     assert L.rof_plan_hub_patterns(None, None, 0, 0, 16, 8, C.byref(h)) == -1
     assert L.rof_plan_dynamic_greedy(None, None, None, None, 0, 0, 3, C.byref(h)) == -1
-    assert C.sizeof(_lib.Epilogue) == 32 and C.sizeof(_lib.LayoutOpts) == 32         # the structs of include/rof.h
+    assert C.sizeof(_lib.Epilogue) == 32 and C.sizeof(_lib.LayoutOpts) == 48         # the structs of include/rof.h
     with pytest.raises(_lib.RofError, match="invalid argument"):
         _lib.check(-1)
 

@@ -411,3 +411,45 @@ def test_rows_taken_as_whole_vectors_give_the_same_columns(oracle, feat, bf16_in
         assert got.stride(0) == ld                                 # rows of the padded width, returned as a view
         with pytest.raises(RofError):
             lay.aggregate(x, pad_columns=True, out=torch.empty((n, feat), device="cuda", dtype=want.dtype), **kw)
+
+
+@pytest.mark.parametrize("feat,bf16,build_lanes", [(64, False, 16), (47, False, 12), (3, False, 4), (300, False, 64),
+                                                   (256, True, 32), (100, True, 16), (64, False, 64), (520, False, 4)])
+def test_groups_summed_in_lds_by_the_workgroup_of_their_consumers(oracle, feat, bf16, build_lanes):
+    """Planted reuse: destinations that share groups sit in one workgroup, which sums the groups once into LDS
+    (local_groups=8: kept whatever the plan saves in total; the default needs 64 MB of saved gathers).  Widths cover one and several feature chunks per row (the LDS rows are rewritten per
+    chunk), the scalar instantiation, bf16 rows, and layouts built for another width than they are run at."""
+    indptr, indices, plan = _case("hr", 6, 3)
+    n = len(indptr) - 1
+    x = features(n, feat, seed=31)
+    deg = np.diff(indptr).astype(np.float32)
+    lay = _layout(plan, n, 3, lanes_per_row=build_lanes, elem_bytes=2 if bf16 else 4, local_groups=8)
+    st = lay.stats()
+    assert st["cluster_workgroups"] > 0 and st["lds_reads"] > 0 and st["materialised_groups"] == 0
+    plain = _layout(plan, n, 3, disable_reuse=True, lanes_per_row=build_lanes)
+    xt = torch.from_numpy(x).cuda()
+    if bf16:
+        xt = xt.to(torch.bfloat16)
+        x = xt.float().cpu().numpy()
+    degt = torch.from_numpy(deg).cuda()
+    for normalized in (True, False):
+        if normalized:
+            lay.set_degrees(degt)
+            plain.set_degrees(degt)
+        out = torch.full((n, feat), float("nan"), device="cuda")
+        lay.aggregate(xt, normalized=normalized, out=out)
+        got = out.cpu().numpy()
+        want = oracle.closed_form(indptr, indices, x, deg, normalized=normalized)
+        mag = oracle.closed_form(indptr, indices, np.abs(x), deg, normalized=normalized)
+        _close(got, want, mag)
+        ref = plain.aggregate(xt, normalized=normalized)
+        _close(got, ref.cpu().numpy().astype(np.float64), mag)                 # same sum, another bracketing
+        assert torch.equal(out, lay.aggregate(xt, normalized=normalized))      # repeatable bit for bit
+    # the fused store and the entry point without allocations take the same path
+    bias = torch.randn(feat, device="cuda")
+    fused = lay.aggregate(xt, normalized=True, bias=bias, relu=True, self_weight=0.5)
+    sep = torch.relu(lay.aggregate(xt, normalized=True, self_weight=0.5) + bias)
+    assert torch.equal(fused, sep)
+    again = torch.empty_like(fused)
+    lay.aggregate_noalloc(xt, again, normalized=True, bias=bias, relu=True, self_weight=0.5)
+    assert torch.equal(again, fused)

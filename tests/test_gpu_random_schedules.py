@@ -59,7 +59,8 @@ def test_random_schedules_match_the_closed_form(oracle, block):
         ip, ix = random_csr(rng, n, ps)
         opts = dict(hub_split=int(rng.choice([0, 8, 33, 100])), segment=int(rng.choice([0, 1, 5, 16])),
                     lanes_per_row=int(rng.choice(LANES)), entry_order=str(rng.choice(["descending", "plan", "ascending"])),
-                    tile_rows=int(rng.choice([0, 64])), elem_bytes=int(rng.choice([0, 2, 4])))
+                    tile_rows=int(rng.choice([0, 64])), elem_bytes=int(rng.choice([0, 2, 4])),
+                    local_groups=int(rng.choice([0, 0, 1, 30, -1])))
         use_plan = rng.random() < 0.6
         if use_plan:
             t = sp.csr_matrix((np.ones(len(ix), np.int8), ix, ip), shape=(n, n)).tocsc()   # the graphs are directed

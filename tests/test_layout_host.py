@@ -84,8 +84,9 @@ def test_schedule_computes_the_closed_form(oracle, opts):
         assert np.allclose(got, oracle.closed_form(ip, ix, x), rtol=1e-12, atol=1e-12)
         # bookkeeping used by the roofline report
         nref = int(ex["g_task_nref"].sum() + ex["s_task_nref"].sum() + ex["b_task_nref"].sum())
-        total = len(ex["g_col"]) + len(ex["s_col"]) + len(ex["b_col"])
-        assert st["partial_reads"] == nref and st["gathered_rows"] == total - nref
+        nlds = int(ex["b_task_nlds"].sum())
+        total = len(ex["g_col"]) + len(ex["s_col"]) + len(ex["b_col"]) + len(ex["b_lg_col"])
+        assert st["partial_reads"] == nref and st["gathered_rows"] == total - nref - nlds and st["lds_reads"] == nlds
         assert st["edges"] == len(ix) and st["tasks_b"] == n
         assert st["partial_rows"] == st["materialised_groups"] + st["hub_segments"]
         if opts.get("disable_reuse"):
@@ -96,8 +97,9 @@ def test_schedule_computes_the_closed_form(oracle, opts):
 
 
 def test_sharing_is_gated_by_the_bytes_it_saves():
-    """The same plan is executed with its groups shared when rows are wide and folded back when they are
-    narrow: what one more launch has to repay is bytes (net saved gathers x row bytes, 16 per lane)."""
+    """Sharing through the workspace (workgroup-local sharing switched off): the same plan is executed with its
+    groups shared when rows are wide and folded back when they are narrow: what one more launch has to repay is
+    bytes (net saved gathers x row bytes, 16 per lane)."""
     ip, ix = make_workload("hr", 5)                          # 32 768 nodes, most neighbours in shared anchor sets
     n = len(ip) - 1
     plan = R.build_plan(ip, ix, 3)
@@ -105,13 +107,55 @@ def test_sharing_is_gated_by_the_bytes_it_saves():
     cnt = cnt[cnt >= 3]                                      # groups the per-group rule shares at ps = 3
     net = int(((cnt - 1) * 3 - cnt).sum())
     assert net * 32 * 16 < 256_000_000 <= net * 64 * 16      # 512-byte rows: below the gate; 1024-byte rows: above
-    narrow = _v2(plan, n, 3, lanes_per_row=32).stats()
-    wide = _v2(plan, n, 3, lanes_per_row=64).stats()
+    narrow = _v2(plan, n, 3, lanes_per_row=32, local_groups=-1).stats()
+    wide = _v2(plan, n, 3, lanes_per_row=64, local_groups=-1).stats()
     assert narrow["materialised_groups"] == 0 and narrow["gathered_rows"] == len(ix)
     assert wide["materialised_groups"] == len(cnt)
     assert len(ix) - wide["gathered_rows"] - wide["partial_reads"] == net
     forced = _v2(plan, n, 3, lanes_per_row=32, min_consumers=3).stats()   # an explicit threshold bypasses the gate
     assert forced["materialised_groups"] == len(cnt)
+
+
+@pytest.mark.parametrize("lanes,wl,sd,ps", [(16, "hr", 5, 3), (16, "hr", 6, 2), (64, "hr", 6, 4), (12, "hr", 5, 3),
+                                            (32, "c1", 2, 2), (8, "c2", 5, 3)])
+def test_consumers_of_a_group_are_clustered_into_workgroups_that_sum_it_in_lds(oracle, lanes, wl, sd, ps):
+    """Short destinations that share groups are placed in one cluster (workgroup) whose local groups are summed once
+    into LDS rows.  The exported schedule is executed in float64 (which also checks that LDS rows are read only
+    inside the cluster that sums them) and the bookkeeping is checked.  local_groups=8: clusters that save 8 gathers
+    are kept whatever they save in total (by default a plan's clusters must repay their launch: 64 MB of gathers,
+    which these small graphs do not hold)."""
+    ip, ix = make_workload(wl, sd)
+    n = len(ip) - 1
+    plan = R.build_plan(ip, ix, ps)
+    lay = _v2(plan, n, ps, lanes_per_row=lanes, local_groups=8)
+    if wl != "hr":
+        assert _v2(plan, n, ps, lanes_per_row=lanes).stats()["cluster_workgroups"] == 0  # too little to repay a launch
+    ex, st = lay.export(), lay.stats()
+    sh = ex["b_shape"]
+    x = np.random.default_rng(1).standard_normal((n, 2))
+    r = 1.0 / np.sqrt(np.maximum(np.diff(ip), 1).astype(np.float64))
+    got = emulate_schedule(ex, n, x, lambda c: r[c], lambda v: r[v], st["partial_rows"])
+    assert np.allclose(got, oracle.closed_form(ip, ix, x), rtol=1e-12, atol=1e-12)
+    assert st["cluster_workgroups"] == sh["lg_blocks"] and st["local_groups"] == len(ex["b_lg_task_ptr"]) - 1
+    assert st["lds_reads"] == int(ex["b_task_nlds"].sum()) and st["lds_rows"] == (sh["lg_max_rows"] if sh["lg_blocks"] else 0)
+    if wl == "hr":
+        # planted reuse: almost every destination is served from LDS and most gathers disappear without any
+        # partial row going through the workspace
+        assert st["cluster_workgroups"] > 0 and st["materialised_groups"] == 0
+        assert st["gathered_rows"] < 0.65 * len(ix)
+        lens = np.diff(ex["b_lg_ptr"])
+        assert lens.min() >= 1 and lens.max() <= st["lds_rows"] <= 32
+        tf = ex["b_lg_task_first"]
+        assert np.diff(tf).max() <= 64
+        # every local group is read by at least two tasks of its cluster
+        for b in range(min(sh["lg_blocks"], 50)):
+            rows = []
+            for t in range(tf[b], tf[b + 1]):
+                rows += ex["b_col"][ex["b_task_ptr"][t]:ex["b_task_ptr"][t] + ex["b_task_nlds"][t]].tolist()
+            cnt = np.bincount(rows, minlength=lens[b])
+            assert (cnt >= 2).all()
+    off = _v2(plan, n, ps, lanes_per_row=lanes, local_groups=-1).stats()
+    assert off["cluster_workgroups"] == 0 and off["lds_reads"] == 0
 
 
 @pytest.mark.parametrize("lanes,elem,cut,seg", [(64, 4, 128, 32), (32, 4, 128, 32), (32, 2, 256, 64), (16, 4, 384, 96),
