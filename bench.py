@@ -42,6 +42,7 @@ HBM_PEAK_GBS = 8000.0
 # (workload, part size, width, packed output) with default layout options; the JSON then says "offline profile".
 PROFILED_TRAFFIC = {}
 COPY_BYTES = 1 << 30   # size of the calibration copy the counter runs include
+CHILD_AGGREGATIONS = 4  # aggregations a counter run executes
 
 DESCR = {
     "c1": "c1: R-MAT 2^14 nodes, avg deg 16, self loops, GCN sym-norm, F=32, fp32",
@@ -277,7 +278,7 @@ def traffic_child(args):
     torch.cuda.synchronize()
     _lib.check(L.rof_device_copy(ctypes.c_void_p(b.data_ptr()), ctypes.c_void_p(a.data_ptr()), COPY_BYTES,
                                  ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
-    for _ in range(4):
+    for _ in range(CHILD_AGGREGATIONS):
         reuse.aggregate(x, normalized, out=out, feat_dim=feat, pad_columns=pad)
     torch.cuda.synchronize()
 
@@ -310,12 +311,13 @@ def measure_traffic(args, passthrough):
                     k = row["Kernel_Name"]
                     if "rof_copy_kernel" in k:
                         copy[row["Counter_Name"]] = float(row["Counter_Value"])
-                    elif "rof_rows_kernel" in k:
-                        # template arguments <XT, VEC, LPR, PHASE, OFF32>: PHASE 0 is the partial-sum launch
+                    elif "rof_rows_kernel" in k or "rof_cluster_kernel" in k:
+                        # template arguments <XT, VEC, LPR, PHASE, OFF32>: PHASE 0 are the partial-sum launches (shared
+                        # groups, segments of long rows), the others the destination rows (and their clusters)
                         phase = int(k.split("<")[1].split(">")[0].split(",")[3])
                         acc[(row["Counter_Name"], min(phase, 1))].append(float(row["Counter_Value"]))
             for k, v in acc.items():
-                per[k] = sum(v) / len(v)
+                per[k] = sum(v) / CHILD_AGGREGATIONS   # per aggregation: a phase may consist of two launches
     except (OSError, subprocess.SubprocessError, ValueError, KeyError, IndexError) as ex:
         return {"error": f"counter runs failed: {ex!r}"[:300]}
     finally:
@@ -326,7 +328,7 @@ def measure_traffic(args, passthrough):
     f_scale = COPY_BYTES / (copy["FETCH_SIZE"] * 1024.0)
     w_scale = COPY_BYTES / (copy["WRITE_SIZE"] * 1024.0)
     res = {"source": "live: this script under rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE / TCC_HIT_sum TCC_MISS_sum, "
-                     "one counter set per child process, mean per dispatch over 4 aggregations",
+                     f"one counter set per child process, mean over {CHILD_AGGREGATIONS} aggregations",
            "fetch_scale": f_scale, "write_scale": w_scale, "launch": {}}
     for phase in (0, 1):
         if ("FETCH_SIZE", phase) not in per:
@@ -373,6 +375,7 @@ def part_size_sweep(name, sizes, have, n, e, x, deg, normalized, feat, lpr, in_b
             row[tag + "_ms"] = ms
             if tag == "reuse":
                 row.update(GEdges_per_s=e / (ms * 1e-3) / 1e9, materialised_groups=st["materialised_groups"],
+                           clusters=st["cluster_workgroups"], local_groups=st["local_groups"],
                            plan_saved_gathers_frac=1.0 - len(d["uniqpart_column_index"]) / max(1, e))
             if tag == "reuse_forced":
                 row["forced_saved_gathers_frac"] = 1.0 - (st["gathered_rows"] + st["partial_reads"] - st["hub_segments"]) / max(1, e)
@@ -425,7 +428,7 @@ def main():
     feat = args.feat or FEAT[name]
     normalized = name != "c3"
     bf16 = name == "c5"
-    default_opts = (not (args.hub_split or args.segment or args.min_consumers or args.tile_rows or args.xcd_run
+    default_opts = (not (args.hub_split or args.segment or args.tile_rows or args.xcd_run
                          or args.xcd_run_partial != 1 or args.lds_pad >= 0)
                     and args.search == "upstream" and args.entry_order == "descending")
 
@@ -442,6 +445,8 @@ def main():
             passthrough += ["--feat", str(args.feat)]
         if args.padded_output:
             passthrough += ["--padded-output"]
+        if args.min_consumers:
+            passthrough += ["--min-consumers", str(args.min_consumers)]
         traffic = measure_traffic(args, passthrough)
         if "error" in traffic:
             log(f"[bench] live counters unavailable: {traffic['error']}")
@@ -690,7 +695,7 @@ def main():
     b_min = n * feat * in_bytes + 4 * e + n * feat * 4      # every feature row once, every column id, every output row
     if "error" in traffic:
         key = (name, ps, feat, not pad)
-        off = PROFILED_TRAFFIC.get(key) if default_opts else None
+        off = PROFILED_TRAFFIC.get(key) if default_opts and not args.min_consumers else None
         if off:
             traffic = dict(off, source="offline profile (profiles/): the live counter runs were not available: "
                                        + traffic["error"])
@@ -753,10 +758,16 @@ def main():
         },
         "reuse_forced": forced_info,
         "plan": {"groups": st["groups"], "materialised_groups": st["materialised_groups"],
-                 "folded_by_cost_model": bool(st["materialised_groups"] == 0 and st["groups"] > 0),
+                 "folded_by_cost_model": bool(st["materialised_groups"] == 0 and st["local_groups"] == 0 and st["groups"] > 0),
                  "gathered_rows": st["gathered_rows"], "partial_reads": st["partial_reads"],
                  "partial_rows": st["partial_rows"], "hub_segments": st["hub_segments"],
+                 "local_groups": st["local_groups"], "lds_reads": st["lds_reads"], "clusters": st["cluster_workgroups"],
                  "saved_gathers_frac": 1.0 - (st["gathered_rows"] + st["partial_reads"] - st["hub_segments"]) / max(1, e),
+                 "executed_as": ("reuse-disabled schedule (the cost model folded every group)"
+                                 if st["materialised_groups"] == 0 and st["local_groups"] == 0 else
+                                 "groups shared" + (" in LDS by clustered workgroups" if st["local_groups"] else "")
+                                 + (" and" if st["local_groups"] and st["materialised_groups"] else "")
+                                 + (" through workspace rows" if st["materialised_groups"] else "")),
                  "cpu_graph_s": t_gen, "cpu_plan_s": t_plan, "cpu_layout_s": t_layout},
     }
 

@@ -144,7 +144,8 @@ typedef struct {
                              /* the default hub_split.                                                              */
     int32_t local_groups;    /* workgroup-local sharing (min_consumers = 0 only): short destinations that consume the */
                              /* same groups are placed in one workgroup, which sums those groups once into LDS;      */
-                             /* 0 = on, a workgroup must save at least 8 row gathers; k > 0 = at least k; -1 = off    */
+                             /* 0 = on: a cluster must save 8 row gathers and an eighth of its rows' gathers, and all  */
+                             /* clusters together 64 MB of gathers; k > 0 = every cluster that saves k; -1 = off      */
     int32_t reserved[3];
 } rof_layout_opts;
 
