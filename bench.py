@@ -40,7 +40,21 @@ HBM_PEAK_GBS = 8000.0
 # rocprofv3 summaries under profiles/ (FETCH_SIZE x its copy-calibrated factor + WRITE_SIZE).  Used only when the
 # live counter runs are switched off or fail, and only for the configurations they were measured on:
 # (workload, part size, width, packed output) with default layout options; the JSON then says "offline profile".
-PROFILED_TRAFFIC = {}
+def _offline(read0, written0, hit0, read1, written1, hit1):
+    launch = {1: {"read_bytes": read1, "written_bytes": written1, "bytes": read1 + written1, "tcc_hit_rate": hit1,
+                  "tcc_miss_x_128B": None}}
+    if read0 is not None:
+        launch[0] = {"read_bytes": read0, "written_bytes": written0, "bytes": read0 + written0, "tcc_hit_rate": hit0,
+                     "tcc_miss_x_128B": None}
+    return {"fetch_scale": 2.0, "write_scale": 1.0, "launch": launch}
+
+
+PROFILED_TRAFFIC = {
+    ("c4", 3, 47, True): _offline(1.75e9, 0.029e9, 0.69, 5.87e9, 0.50e9, 0.44),     # profiles/rof_rows_kernel_c4_f47.md
+    ("c5", 3, 256, True): _offline(23.38e9, 1.55e9, 0.53, 19.32e9, 4.71e9, 0.41),   # profiles/rof_rows_kernel_c5_bf16.md
+    ("c3", 3, 64, True): _offline(None, None, None, 1.04e9, 0.27e9, 0.82),          # profiles/rof_rows_kernel_c3_f64.md
+    ("hr", 3, 64, True): _offline(None, None, None, 1.36e9, 0.27e9, 0.20),          # profiles/rof_cluster_kernel_hr_f64.md
+}
 COPY_BYTES = 1 << 30   # size of the calibration copy the counter runs include
 CHILD_AGGREGATIONS = 4  # aggregations a counter run executes
 
@@ -290,6 +304,8 @@ def measure_traffic(args, passthrough):
     prof = shutil.which("rocprofv3") or "/opt/rocm/bin/rocprofv3"
     if not os.path.exists(prof):
         return {"error": "rocprofv3 not found"}
+    if "rocprof" in os.environ.get("LD_PRELOAD", "") or os.environ.get("ROCPROFILER_REGISTER_FORCE_LOAD"):
+        return {"error": "this process already runs under a profiler"}
     tmp = tempfile.mkdtemp(prefix="rof_pmc_", dir="/tmp")
     env = dict(os.environ, TMPDIR="/tmp")
     per = {}     # (counter, phase) -> mean value per dispatch; phase 0 = partial-sum launch, 1 = destination rows
