@@ -1,15 +1,16 @@
 // gfx950 (CDNA4, wave64) kernels of the reuse-aware neighbour aggregation: C ABI, launch logic and the
-// small helper kernels.  The row-gather kernel itself is in agg_rows.h (instantiated in
-// agg_rows_f32.hip / agg_rows_bf16.hip).
+// small helper kernels.  The row-gather kernels themselves are in agg_rows.h (instantiated in
+// agg_rows_*_partial.hip, agg_rows_*_dst.hip and agg_cluster_*.hip).
 //
 // One kernel template does all the summing.  A *task* gathers a list of rows and writes their
 // weighted sum to one output row:
 //     out[task_out[t], :] = scale[t] * sum_i w[i] * row(col[i])        i in task_ptr[t] .. task_ptr[t+1]
 // where row(c) is x[c, :] for c < nsplit and the partial-sum row part[c - nsplit, :] otherwise
-// (the first task_nref[t] entries of a task are of the second kind).  Up to three launches in stream
+// (the first task_nref[t] entries of a task are of the second kind).  Up to four launches in stream
 // order: reuse groups that several destinations share -> partial-sum rows; segments of very long rows
-// (which may read group rows) -> partial-sum rows; every destination row -> out.  There are no
-// atomics: each output row has one writer.
+// (which may read group rows) -> partial-sum rows; every destination row -> out; and, for destinations that the
+// schedule has clustered around groups they share, one workgroup per cluster that sums those groups once into LDS
+// before it gathers the cluster's rows (rof_cluster_kernel).  There are no atomics: each output row has one writer.
 //
 // Mapping to the machine:
 //   * the feature dimension runs across lanes, VEC consecutive elements per lane (one 16-byte
@@ -451,7 +452,7 @@ static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64
         a.n_tasks = d.n_tasks;
         a.xcd_run = g_xcd_run_a;
         a.vec_store = 1;
-        if ((rc = (x_dtype == ROF_F32 ? rofk::launch_rows_f32(a, 0, vec, off32, 0, st) : rofk::launch_rows_bf16(a, 0, vec, off32, 0, st)))) return rc;
+        if ((rc = rofk::launch_rows(x_dtype != ROF_F32, a, 0, vec, off32, 0, st))) return rc;
     }
     if (L->db.n_tasks && (launches & 2)) {   // last launch: destination rows
         a.task_ptr = L->db.task_ptr;
@@ -478,13 +479,12 @@ static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64
         const int phase = ((int64_t)L->n * feat * (a.out_bf16 ? 2 : 4) >= kStreamOutBytes && a.vec_store && vec > 1 &&
                            (!a.out_bf16 || ldo % 2 == 0)) ? 2 : 1;
         a.n_tasks = L->db.n_regular;   // the clustered destinations at the end of the list have a launch of their own
-        if ((rc = (x_dtype == ROF_F32 ? rofk::launch_rows_f32(a, phase, vec, off32, 0, st) : rofk::launch_rows_bf16(a, phase, vec, off32, 0, st)))) return rc;
+        if ((rc = rofk::launch_rows(x_dtype != ROF_F32, a, phase, vec, off32, 0, st))) return rc;
         if (L->db.lg_blocks > 0) {
             a.n_tasks = L->db.n_tasks;
             a.n_blocks = L->db.lg_blocks;
             a.xcd_run = 1;
-            if ((rc = (x_dtype == ROF_F32 ? rofk::launch_rows_f32(a, phase, vec, off32, L->db.lg_max_rows, st)
-                                          : rofk::launch_rows_bf16(a, phase, vec, off32, L->db.lg_max_rows, st)))) return rc;
+            if ((rc = rofk::launch_rows(x_dtype != ROF_F32, a, phase, vec, off32, L->db.lg_max_rows, st))) return rc;
         }
     }
     return ROF_OK;

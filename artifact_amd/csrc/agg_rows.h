@@ -1,5 +1,5 @@
-// Row-gather kernel of the reuse-aware aggregation and its launcher template, shared by the two
-// translation units that instantiate it (fp32 and bf16 features are compiled separately so that the
+// Row-gather kernels of the reuse-aware aggregation and their launcher template, shared by the
+// translation units that instantiate them (by feature type and by launch, compiled separately so that the
 // build can run them in parallel).  See agg_kernels.hip for the description of the scheme.
 #ifndef ROF_AGG_ROWS_H_
 #define ROF_AGG_ROWS_H_
@@ -547,13 +547,27 @@ int launch_lpr(const AggArgs &a0, int lpr, int lds_rows, hipStream_t st) {
     return ROF_OK;
 }
 
-// Instantiated in agg_rows_f32.hip / agg_rows_bf16.hip.  phase 0: partial-sum launches, 1: destination rows,
-// 2: destination rows with streaming stores.
+// Instantiated in agg_rows_{f32,bf16}_partial.hip (partial-sum launches), agg_rows_{f32,bf16}_dst.hip (destination
+// rows; phase 1, or 2 = streaming stores) and agg_cluster_{f32,bf16}.hip (the clustered destination rows: a.n_blocks
+// clusters whose workgroups need lds_rows LDS rows), one translation unit each so that the build runs them side by side.
 // off32: every byte offset into the feature matrix and into the partial-sum workspace fits 32 bits and
 // every row id fits 24 bits, so the kernels may use the short address arithmetic.
-// lds_rows > 0: the cluster launch (a.n_blocks workgroups, phase >= 1) whose workgroups need that many LDS rows.
-int launch_rows_f32(const AggArgs &a, int phase, int vec, bool off32, int lds_rows, hipStream_t st);
-int launch_rows_bf16(const AggArgs &a, int phase, int vec, bool off32, int lds_rows, hipStream_t st);
+int launch_rows_f32_partial(const AggArgs &a, int vec, bool off32, hipStream_t st);
+int launch_rows_f32_dst(const AggArgs &a, int phase, int vec, bool off32, hipStream_t st);
+int launch_rows_f32_cluster(const AggArgs &a, int phase, int vec, bool off32, int lds_rows, hipStream_t st);
+int launch_rows_bf16_partial(const AggArgs &a, int vec, bool off32, hipStream_t st);
+int launch_rows_bf16_dst(const AggArgs &a, int phase, int vec, bool off32, hipStream_t st);
+int launch_rows_bf16_cluster(const AggArgs &a, int phase, int vec, bool off32, int lds_rows, hipStream_t st);
+
+// phase 0: partial-sum launches, 1: destination rows, 2: destination rows with streaming stores; lds_rows > 0: the
+// cluster launch of the destination rows
+inline int launch_rows(bool bf16, const AggArgs &a, int phase, int vec, bool off32, int lds_rows, hipStream_t st) {
+    if (phase == 0) return bf16 ? launch_rows_bf16_partial(a, vec, off32, st) : launch_rows_f32_partial(a, vec, off32, st);
+    if (lds_rows > 0)
+        return bf16 ? launch_rows_bf16_cluster(a, phase, vec, off32, lds_rows, st)
+                    : launch_rows_f32_cluster(a, phase, vec, off32, lds_rows, st);
+    return bf16 ? launch_rows_bf16_dst(a, phase, vec, off32, st) : launch_rows_f32_dst(a, phase, vec, off32, st);
+}
 
 }  // namespace rofk
 

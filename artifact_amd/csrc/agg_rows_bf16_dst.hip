@@ -1,0 +1,19 @@
+// bf16-feature instantiations of the row-gather kernel: the destination-row launch (PHASE 1 and 2).
+#include "agg_rows.h"
+
+namespace rofk {
+
+template <int PHASE>
+static int launch(const AggArgs &a, int vec, bool off32, hipStream_t st) {
+    const int lpr = rof_lanes_per_row(a.feat, vec);
+    if (vec == 8)
+        return off32 ? launch_lpr<uint16_t, 8, PHASE, true, false>(a, lpr, 0, st)
+                     : launch_lpr<uint16_t, 8, PHASE, false, false>(a, lpr, 0, st);
+    return launch_lpr<uint16_t, 1, PHASE, false, false>(a, lpr, 0, st);
+}
+
+int launch_rows_bf16_dst(const AggArgs &a, int phase, int vec, bool off32, hipStream_t st) {
+    return phase == 1 ? launch<1>(a, vec, off32, st) : launch<2>(a, vec, off32, st);
+}
+
+}  // namespace rofk

@@ -286,14 +286,17 @@ def test_own_row_term_of_the_epilogue(oracle, feat, bf16):
     _close(got.cpu().numpy(), np.maximum(ref, 0), mag)
 
 
-def test_aggregation_is_capturable_in_a_hip_graph(oracle):
+@pytest.mark.parametrize("wl,sd,opts", [("c1", 1, dict(min_consumers=2)),        # three launches: groups, segments, rows
+                                        ("hr", 6, dict(local_groups=8))])        # rows, then the clusters' launch
+def test_aggregation_is_capturable_in_a_hip_graph(oracle, wl, sd, opts):
     """rof_aggregate_epilogue only enqueues kernels (no allocation, no synchronisation, no memset), so a layer's
     aggregation can be captured once and replayed: three replays on fresh inputs, with eager work between them,
     each equal to the eager result bit for bit."""
-    indptr, indices, plan = _case("c1", 1, 3)
+    indptr, indices, plan = _case(wl, sd, 3)
     n = len(indptr) - 1
     feat = 32
-    lay = _layout(plan, n, 3, min_consumers=2)               # three launches: groups, segments, rows
+    lay = _layout(plan, n, 3, **opts)
+    assert lay.stats()["cluster_workgroups" if "local_groups" in opts else "materialised_groups"] > 0
     lay.set_degrees(torch.from_numpy(np.diff(indptr).astype(np.float32)).cuda())
     bias = torch.from_numpy(features(1, feat, seed=30)[0]).cuda()
     x = torch.zeros((n, feat), device="cuda")
