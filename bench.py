@@ -297,6 +297,24 @@ def traffic_child(args):
     torch.cuda.synchronize()
 
 
+def read_counter_csv(path):
+    """One rocprofv3 counter_collection.csv of a counter run -> ({(counter, phase): value per aggregation},
+    {counter: value of the calibration copy}).  Phase 0 = the partial-sum launches (shared groups, segments of long
+    rows; template argument PHASE of the kernel name <XT, VEC, LPR, PHASE, OFF32>), phase 1 = the destination rows
+    and their clusters.  A phase may consist of two launches, so the dispatches of one phase are summed and divided
+    by the number of aggregations the run executes."""
+    acc, copy = collections.defaultdict(float), {}
+    with open(path) as f:
+        for row in csv.DictReader(f):
+            k = row["Kernel_Name"]
+            if "rof_copy_kernel" in k:
+                copy[row["Counter_Name"]] = float(row["Counter_Value"])
+            elif "rof_rows_kernel" in k or "rof_cluster_kernel" in k:
+                phase = int(k.split("<")[1].split(">")[0].split(",")[3])
+                acc[(row["Counter_Name"], min(phase, 1))] += float(row["Counter_Value"])
+    return {k: v / CHILD_AGGREGATIONS for k, v in acc.items()}, copy
+
+
 def measure_traffic(args, passthrough):
     """HBM-side bytes per launch from rocprofv3 counter runs of this script (one counter set per run, as the
     hardware collects them), started as child processes *before* this process initialises the GPU.
@@ -321,19 +339,9 @@ def measure_traffic(args, passthrough):
             if r.returncode != 0 or not files:
                 return {"error": f"rocprofv3 --pmc {' '.join(counters)} failed (rc {r.returncode}): "
                                  + r.stdout.decode(errors="replace")[-300:]}
-            acc = collections.defaultdict(list)
-            with open(files[0]) as f:
-                for row in csv.DictReader(f):
-                    k = row["Kernel_Name"]
-                    if "rof_copy_kernel" in k:
-                        copy[row["Counter_Name"]] = float(row["Counter_Value"])
-                    elif "rof_rows_kernel" in k or "rof_cluster_kernel" in k:
-                        # template arguments <XT, VEC, LPR, PHASE, OFF32>: PHASE 0 are the partial-sum launches (shared
-                        # groups, segments of long rows), the others the destination rows (and their clusters)
-                        phase = int(k.split("<")[1].split(">")[0].split(",")[3])
-                        acc[(row["Counter_Name"], min(phase, 1))].append(float(row["Counter_Value"]))
-            for k, v in acc.items():
-                per[k] = sum(v) / CHILD_AGGREGATIONS   # per aggregation: a phase may consist of two launches
+            rows_per_phase, copy_values = read_counter_csv(files[0])
+            copy.update(copy_values)
+            per.update(rows_per_phase)
     except (OSError, subprocess.SubprocessError, ValueError, KeyError, IndexError) as ex:
         return {"error": f"counter runs failed: {ex!r}"[:300]}
     finally:

@@ -158,6 +158,49 @@ def test_consumers_of_a_group_are_clustered_into_workgroups_that_sum_it_in_lds(o
     assert off["cluster_workgroups"] == 0 and off["lds_reads"] == 0
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_random_graphs_with_shared_neighbour_sets_through_clusters(oracle, seed):
+    """Random directed graphs whose rows are built from a pool of shared neighbour sets (so that many short rows
+    consume the same groups), random lane counts, cuts and cluster thresholds: the exported schedule, run in float64,
+    gives the closed form, and every structural rule of the clusters holds (helpers.emulate_schedule)."""
+    import scipy.sparse as sp
+
+    rng = np.random.default_rng(100 + seed)
+    n = int(rng.integers(200, 1500))
+    ps = int(rng.integers(2, 5))
+    sets = [np.sort(rng.choice(n, ps * int(rng.integers(1, 4)), replace=False)) for _ in range(int(rng.integers(3, 40)))]
+    rows = []
+    for v in range(n):
+        kind = rng.random()
+        if kind < 0.1:
+            rows.append(np.zeros(0, dtype=np.int64))
+        elif kind < 0.75:
+            pick = rng.choice(len(sets), int(rng.integers(1, 4)), replace=False)
+            extra = rng.choice(n, int(rng.integers(0, 6)), replace=False)
+            rows.append(np.unique(np.concatenate([sets[j] for j in pick] + [extra])))
+        else:
+            rows.append(np.unique(rng.choice(n, int(rng.integers(1, min(n, 200))), replace=False)))
+    ip = np.r_[0, np.cumsum([len(r) for r in rows])].astype(np.int32)
+    ix = np.concatenate(rows).astype(np.int32)
+    t = sp.csr_matrix((np.ones(len(ix), np.int8), ix, ip), shape=(n, n)).tocsc()
+    plan = R.build_plan(ip, ix, ps, t.indptr, t.indices)
+    opts = dict(lanes_per_row=int(rng.choice([4, 8, 12, 16, 32, 64])), local_groups=int(rng.choice([1, 4, 8, 30])),
+                hub_split=int(rng.choice([0, 24, 100])), segment=int(rng.choice([0, 8])),
+                elem_bytes=int(rng.choice([2, 4])), entry_order=str(rng.choice(["descending", "plan", "ascending"])))
+    lay = _v2(plan, n, ps, **opts)
+    ex, st = lay.export(), lay.stats()
+    x = rng.standard_normal((n, 2))
+    w = rng.uniform(0.5, 2.0, n)
+    got = emulate_schedule(ex, n, x, lambda c: w[c], lambda v: w[v], st["partial_rows"])
+    a = sp.csr_matrix((np.ones(len(ix)), ix, ip), shape=(n, n))
+    want = w[:, None] * (a @ (w[:, None] * x))
+    assert np.allclose(got, want, rtol=1e-11, atol=1e-11), opts
+    assert st["lds_reads"] == int(ex["b_task_nlds"].sum()) and st["cluster_workgroups"] == ex["b_shape"]["lg_blocks"]
+    total = len(ex["g_col"]) + len(ex["s_col"]) + len(ex["b_col"]) + len(ex["b_lg_col"])
+    nref = int(ex["g_task_nref"].sum() + ex["s_task_nref"].sum() + ex["b_task_nref"].sum())
+    assert st["gathered_rows"] == total - nref - st["lds_reads"] <= len(ix)
+
+
 @pytest.mark.parametrize("lanes,elem,cut,seg", [(64, 4, 128, 32), (32, 4, 128, 32), (32, 2, 256, 64), (16, 4, 384, 96),
                                                 (12, 4, 640, 160), (8, 0, 640, 160)])
 def test_long_rows_are_cut_by_width_and_their_segments_swept_by_source_id(lanes, elem, cut, seg):
