@@ -66,6 +66,11 @@ thread_local char g_dev_err[256] = "";
 // stored whole (scalar instantiation, bf16 rows of odd stride) keep ordinary stores: streamed element by element
 // they were 17 % slower.
 constexpr int64_t kStreamOutBytes = 128 << 20;
+// Partial rows of one launch beyond this many bytes are written as streaming stores: the destination rows read them
+// only after the launch has ended, by which time rows of a workspace this large have left the caches anyway, and
+// until then they would take the place of feature rows there.  (Below it the partial rows are still in L2 when
+// they are read: streaming them costs time.)
+constexpr int64_t kStreamPartialBytes = 64 << 20;
 
 // rsqrt of the in-degree, correctly rounded like __frsqrt_rn (reuse_conv_kernel.cu:254,276)
 __device__ __forceinline__ float rsqrt_rn(float d) { return (float)(1.0 / sqrt((double)d)); }
@@ -452,7 +457,8 @@ static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64
         a.n_tasks = d.n_tasks;
         a.xcd_run = g_xcd_run_a;
         a.vec_store = 1;
-        if ((rc = rofk::launch_rows(x_dtype != ROF_F32, a, 0, vec, off32, 0, st))) return rc;
+        const int phase = (int64_t)d.n_tasks * feat * 4 >= kStreamPartialBytes && vec > 1 ? 3 : 0;
+        if ((rc = rofk::launch_rows(x_dtype != ROF_F32, a, phase, vec, off32, 0, st))) return rc;
     }
     if (L->db.n_tasks && (launches & 2)) {   // last launch: destination rows
         a.task_ptr = L->db.task_ptr;

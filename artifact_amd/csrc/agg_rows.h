@@ -220,7 +220,7 @@ __device__ __forceinline__ void gather_sum(const char *xb, uint32_t xld, const c
     }
 }
 
-// Scale the finished sum of task t, apply the layer's epilogue (PHASE >= 1) and store this lane's piece of the
+// Scale the finished sum of task t, apply the layer's epilogue (PHASE 1 and 2) and store this lane's piece of the
 // output row.  `acc` holds the columns cstart .. cstart + VEC - 1; `skip` of them repeat the neighbouring lane's.
 template <typename XT, int VEC, int PHASE>
 __device__ __forceinline__ void finish_row(const AggArgs &a, int32_t t, bool nonempty, const float (&acc)[VEC], const char *xb,
@@ -233,7 +233,8 @@ __device__ __forceinline__ void finish_row(const AggArgs &a, int32_t t, bool non
     float r[VEC];
 #pragma unroll
     for (int k = 0; k < VEC; ++k) r[k] = acc[k] * s;
-    if (PHASE >= 1) {   // epilogue of the layer: + own row, + bias, then ReLU (columns cstart .. cstart+VEC-1 exist)
+    constexpr bool kDst = PHASE == 1 || PHASE == 2;   // a destination-row launch
+    if (kDst) {   // epilogue of the layer: + own row, + bias, then ReLU (columns cstart .. cstart+VEC-1 exist)
         if (a.self_weight != 0.0f) {
             float own[VEC];
             RowLoad<XT, VEC>::load(reinterpret_cast<const XT *>(xb + (int64_t)a.task_out[t] * xld), own);
@@ -256,8 +257,8 @@ __device__ __forceinline__ void finish_row(const AggArgs &a, int32_t t, bool non
     // (47 floats = 188 bytes) are written as one contiguous burst per row.  The lane that was shifted back
     // to stay inside the row rewrites `skip` elements of its neighbour's piece with the same bits (both
     // lanes sum the same entries in the same order).
-    constexpr bool stream = PHASE == 2;
-    if (PHASE >= 1 && a.out_bf16) {
+    constexpr bool stream = PHASE == 2 || PHASE == 3;
+    if (kDst && a.out_bf16) {
         uint16_t *o = reinterpret_cast<uint16_t *>(a.out) + at;
         if (VEC >= 4 && a.vec_store && (at & 1) == 0) {
 #pragma unroll
@@ -289,9 +290,10 @@ __device__ __forceinline__ void finish_row(const AggArgs &a, int32_t t, bool non
     }
 }
 
-// PHASE 0: the partial-sum launches (no scaling, no epilogue); PHASE 1: the destination-row launch; PHASE 2: the
-// same with the output rows written as streaming stores and the index arrays read as streaming loads (large outputs,
-// hence large graphs).  (A run-time switch between the two kinds of store does
+// PHASE 0: the partial-sum launches (no scaling, no epilogue); PHASE 3: the same with the partial rows written as
+// streaming stores (a workspace too large to stay in the caches until the destination rows read it); PHASE 1: the
+// destination-row launch; PHASE 2: the same with the output rows written as streaming stores and the index arrays
+// read as streaming loads (large outputs, hence large graphs).  (A run-time switch between the two kinds of store does
 // not survive the optimiser, which merges the two stores into an ordinary one.)
 template <typename XT, int VEC, int LPR, int PHASE, bool OFF32>
 __global__ __launch_bounds__(256) void rof_rows_kernel(AggArgs a) {
@@ -403,7 +405,7 @@ __global__ __launch_bounds__(256) void rof_rows_kernel(AggArgs a) {
 // the launch.)
 template <typename XT, int VEC, int LPR, int PHASE, bool OFF32>
 __global__ __launch_bounds__(256) void rof_cluster_kernel(AggArgs a) {
-    static_assert(PHASE >= 1, "clusters belong to the destination-row launch");
+    static_assert(PHASE == 1 || PHASE == 2, "clusters belong to the destination-row launch");
     constexpr int G = 64 / LPR;
     constexpr int kLdsRow = LPR * VEC + 4;
     HIP_DYNAMIC_SHARED(float, lds_rows)
@@ -522,7 +524,7 @@ int launch_lpr(const AggArgs &a0, int lpr, int lds_rows, hipStream_t st) {
 #define ROF_LAUNCH(LPR)                                                                                              \
     do {                                                                                                             \
         if constexpr (CLUSTER)                                                                                       \
-            hipLaunchKernelGGL((rof_cluster_kernel<XT, VEC, LPR, PHASE < 1 ? 1 : PHASE, OFF32>), gr, bl, (unsigned)lds, st, a); \
+            hipLaunchKernelGGL((rof_cluster_kernel<XT, VEC, LPR, (PHASE == 2 ? 2 : 1), OFF32>), gr, bl, (unsigned)lds, st, a); \
         else                                                                                                         \
             hipLaunchKernelGGL((rof_rows_kernel<XT, VEC, LPR, PHASE, OFF32>), gr, bl, (unsigned)lds, st, a);         \
     } while (0)
@@ -547,22 +549,23 @@ int launch_lpr(const AggArgs &a0, int lpr, int lds_rows, hipStream_t st) {
     return ROF_OK;
 }
 
-// Instantiated in agg_rows_{f32,bf16}_partial.hip (partial-sum launches), agg_rows_{f32,bf16}_dst.hip (destination
+// Instantiated in agg_rows_{f32,bf16}_partial.hip (partial-sum launches; stream: phase 3), agg_rows_{f32,bf16}_dst.hip (destination
 // rows; phase 1, or 2 = streaming stores) and agg_cluster_{f32,bf16}.hip (the clustered destination rows: a.n_blocks
 // clusters whose workgroups need lds_rows LDS rows), one translation unit each so that the build runs them side by side.
 // off32: every byte offset into the feature matrix and into the partial-sum workspace fits 32 bits and
 // every row id fits 24 bits, so the kernels may use the short address arithmetic.
-int launch_rows_f32_partial(const AggArgs &a, int vec, bool off32, hipStream_t st);
+int launch_rows_f32_partial(const AggArgs &a, bool stream, int vec, bool off32, hipStream_t st);
 int launch_rows_f32_dst(const AggArgs &a, int phase, int vec, bool off32, hipStream_t st);
 int launch_rows_f32_cluster(const AggArgs &a, int phase, int vec, bool off32, int lds_rows, hipStream_t st);
-int launch_rows_bf16_partial(const AggArgs &a, int vec, bool off32, hipStream_t st);
+int launch_rows_bf16_partial(const AggArgs &a, bool stream, int vec, bool off32, hipStream_t st);
 int launch_rows_bf16_dst(const AggArgs &a, int phase, int vec, bool off32, hipStream_t st);
 int launch_rows_bf16_cluster(const AggArgs &a, int phase, int vec, bool off32, int lds_rows, hipStream_t st);
 
-// phase 0: partial-sum launches, 1: destination rows, 2: destination rows with streaming stores; lds_rows > 0: the
-// cluster launch of the destination rows
+// phase 0: partial-sum launches, 3: the same with streaming stores; 1: destination rows, 2: destination rows with
+// streaming stores; lds_rows > 0: the cluster launch of the destination rows
 inline int launch_rows(bool bf16, const AggArgs &a, int phase, int vec, bool off32, int lds_rows, hipStream_t st) {
-    if (phase == 0) return bf16 ? launch_rows_bf16_partial(a, vec, off32, st) : launch_rows_f32_partial(a, vec, off32, st);
+    if (phase == 0 || phase == 3)
+        return bf16 ? launch_rows_bf16_partial(a, phase == 3, vec, off32, st) : launch_rows_f32_partial(a, phase == 3, vec, off32, st);
     if (lds_rows > 0)
         return bf16 ? launch_rows_bf16_cluster(a, phase, vec, off32, lds_rows, st)
                     : launch_rows_f32_cluster(a, phase, vec, off32, lds_rows, st);
