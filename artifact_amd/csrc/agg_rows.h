@@ -260,7 +260,14 @@ __device__ __forceinline__ void finish_row(const AggArgs &a, int32_t t, bool non
     constexpr bool stream = PHASE == 2 || PHASE == 3;
     if (kDst && a.out_bf16) {
         uint16_t *o = reinterpret_cast<uint16_t *>(a.out) + at;
-        if (VEC >= 4 && a.vec_store && (at & 1) == 0) {
+        if (VEC == 8 && a.vec_store && (at & 1) == 0) {   // the lane's 8 columns are one 16-byte piece
+            const rof_u4 t = {rof_bf16_bits(r[0]) | (rof_bf16_bits(r[1 % VEC]) << 16),   // (% VEC: well-formed in the
+                              rof_bf16_bits(r[2 % VEC]) | (rof_bf16_bits(r[3 % VEC]) << 16),   //  narrower instantiations)
+                              rof_bf16_bits(r[4 % VEC]) | (rof_bf16_bits(r[5 % VEC]) << 16),
+                              rof_bf16_bits(r[6 % VEC]) | (rof_bf16_bits(r[7 % VEC]) << 16)};
+            if (stream) __builtin_nontemporal_store(t, reinterpret_cast<rof_u4 *>(o));
+            else *reinterpret_cast<rof_u4 *>(o) = t;
+        } else if (VEC >= 4 && a.vec_store && (at & 1) == 0) {
 #pragma unroll
             for (int k = 0; k < VEC; k += 4) {
                 const rof_u2s t = {rof_bf16_bits(r[k]) | (rof_bf16_bits(r[k + 1]) << 16),
@@ -275,7 +282,25 @@ __device__ __forceinline__ void finish_row(const AggArgs &a, int32_t t, bool non
         }
     } else {
         float *o = reinterpret_cast<float *>(a.out) + at;
-        if (VEC >= 4 && a.vec_store) {
+        if (VEC == 8 && stream && a.vec_store && (a.feat & 15) == 0) {
+            // A lane holds 8 columns = 32 bytes, so each of its two 16-byte stores would leave a 16-byte hole
+            // between lanes, and streaming stores are not merged in L2: such rows reached memory as partial
+            // lines (WRITE_SIZE 9-13 % above the bytes stored).  Neighbouring lanes swap halves instead -- the even
+            // lane of a pair hands over its upper four columns for the odd lane's lower four -- and both store
+            // instructions then write one gap-free run of 16 bytes per lane.  (feat % 16 == 0: every lane has its
+            // partner, in the same row, and no lane is shifted.)
+            const bool odd = (cstart >> 3) & 1;
+            float got[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) got[k] = __shfl_xor(odd ? r[k % VEC] : r[(4 + k) % VEC], 1);
+            const rof_f4 lo = {odd ? got[0] : r[0], odd ? got[1] : r[1 % VEC], odd ? got[2] : r[2 % VEC],
+                               odd ? got[3] : r[3 % VEC]};
+            const rof_f4 hi = {odd ? r[4 % VEC] : got[0], odd ? r[5 % VEC] : got[1], odd ? r[6 % VEC] : got[2],
+                               odd ? r[7 % VEC] : got[3]};
+            float *p = o - (odd ? 4 : 0);   // even: columns B .. B+3 and B+8 .. B+11; odd: B+4 .. B+7 and B+12 .. B+15
+            __builtin_nontemporal_store(lo, reinterpret_cast<rof_f4 *>(p));
+            __builtin_nontemporal_store(hi, reinterpret_cast<rof_f4 *>(p + 8));
+        } else if (VEC >= 4 && a.vec_store) {
 #pragma unroll
             for (int k = 0; k < VEC; k += 4) {
                 const rof_f4 t = {r[k], r[k + 1], r[k + 2], r[k + 3]};

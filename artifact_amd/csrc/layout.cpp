@@ -313,6 +313,7 @@ void build_clusters(const rof_layout *L, const ivec &ng_ptr, const ivec &ng, con
             add(b1, run);
             if (shared > max_rows && b1 > b0) {   // this run's groups no longer fit into the LDS rows
                 remove(b1, run);
+                work -= run_work;
                 break;
             }
             b1 = run;

@@ -357,6 +357,37 @@ def test_byte_offsets_between_2_and_4_gib():
     assert torch.allclose(got[:rows].double(), want, rtol=1e-5, atol=1e-5)
 
 
+@pytest.mark.parametrize("feat", [16, 48, 24])
+def test_streamed_rows_of_bf16_features_are_exact_on_integers(feat):
+    """bf16 rows put 8 columns on a lane.  Partial rows of a launch that writes 64 MB or more and output rows of
+    128 MB or more are written with streaming stores, for which neighbouring lanes swap halves when the width is a
+    multiple of 16 (16: two active lanes per row; 48: six) and which fall back to the lane's own two pieces
+    otherwise (24).  Small integers in bf16, unnormalised: every sum is exact."""
+    from artifact_amd.layout import lanes_per_row
+    dev = "cuda"
+    rng = np.random.default_rng(16 + feat)
+    n, long_rows, per, short_rows = 2_200_000, 40_000, 64, 300_000
+    nbr_long = np.sort(rng.integers(0, n, (long_rows, per)), axis=1)
+    nbr_short = np.sort(rng.integers(0, n, (short_rows, 8)), axis=1)
+    deg = np.zeros(n, np.int64)
+    deg[:long_rows] = per
+    deg[long_rows:long_rows + short_rows] = 8
+    ip = np.r_[0, np.cumsum(deg)].astype(np.int32)
+    ix = np.r_[nbr_long.ravel(), nbr_short.ravel()].astype(np.int32)
+    lay = Layout.from_csr(ip, ix, hub_split=32, segment=1, lanes_per_row=lanes_per_row(feat, True), elem_bytes=2)
+    assert lay.stats()["hub_segments"] == long_rows * per           # 2.56 M partial rows: >= 64 MB at 16 columns
+    assert lay.workspace_bytes(feat) >= 64 << 20 and n * feat * 4 >= 128 << 20
+    xi = rng.integers(-8, 9, (n, feat)).astype(np.float32)
+    x = torch.from_numpy(xi).to(dev).to(torch.bfloat16)
+    got = torch.full((n, feat), float("nan"), device=dev)
+    lay.aggregate(x, normalized=False, out=got)
+    got = got.cpu().numpy()
+    assert np.array_equal(got[:long_rows], xi[nbr_long].sum(1))
+    assert np.array_equal(got[long_rows:long_rows + short_rows], xi[nbr_short].sum(1))
+    assert not got[long_rows + short_rows:].any()
+    lay.close()
+
+
 def test_byte_offsets_above_4_gib_and_row_ids_above_2_pow_24():
     """The long address arithmetic (64-bit multiply per row): (1) a feature matrix of 4.6 GB gathered from its
     top, bottom and middle; (2) 17 M nodes, so that row ids need more than 24 bits, with bf16 rows."""
