@@ -72,6 +72,24 @@ constexpr int64_t kStreamOutBytes = 128 << 20;
 // they are read: streaming them costs time.)
 constexpr int64_t kStreamPartialBytes = 64 << 20;
 
+// Wavefronts per SIMD of the destination-row launch.  On a heavy-tailed graph whose feature matrix is far larger
+// than the L2s, the launch mixes gathers of hub rows, which hit, with gathers that miss, and the miss path of a CU
+// slows down when too many lines are asked for at once: with two row gathers in flight per lane group, rows of up
+// to 64 bytes (16 rows per wavefront) run best at 6 wavefronts per SIMD, rows of two 128-byte lines (129-256 bytes)
+// at 7, all others with every slot taken.  Measured on the 2.4 M-node R-MAT graph (destination-row launch at 8 / 7 /
+// 6 wavefronts): 16 floats 570 / 558 / 549 us, 32 floats 570 / 581 / 600, 47 floats 972 / 922 / 934, 64 floats
+// 982 / 931 / 938, 100 floats 1052 / 1086 / 1144.  Every other case loses 2-10 % per slot given up: matrices that
+// the caches serve (2^18 nodes x 40 floats; the block model, whose rows gather from their own neighbourhood), the
+// partial-sum launches, and graphs without hub rows (uniform degrees, 2^20 nodes x 64 floats: 689 / 700 us).  The
+// layout knows the latter by having no segmented rows.
+constexpr int64_t kColdMatrixBytes = 128 << 20;   // 4x the L2 of the eight XCDs; the 42 MB matrix above is served, the 154 MB one (16 floats) is not
+int dst_wave_cap(const rof_layout *L, int64_t matrix_bytes, int64_t row_bytes) {
+    if (L->local_sources || L->n_segments == 0 || matrix_bytes < kColdMatrixBytes) return 0;
+    if (row_bytes <= 64) return 6;
+    if (row_bytes > 128 && row_bytes <= 256) return 7;
+    return 0;
+}
+
 // rsqrt of the in-degree, correctly rounded like __frsqrt_rn (reuse_conv_kernel.cu:254,276)
 __device__ __forceinline__ float rsqrt_rn(float d) { return (float)(1.0 / sqrt((double)d)); }
 
@@ -485,7 +503,9 @@ static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64
         const int phase = ((int64_t)L->n * feat * (a.out_bf16 ? 2 : 4) >= kStreamOutBytes && a.vec_store && vec > 1 &&
                            (!a.out_bf16 || ldo % 2 == 0)) ? 2 : 1;
         a.n_tasks = L->db.n_regular;   // the clustered destinations at the end of the list have a launch of their own
+        a.wave_cap = dst_wave_cap(L, (int64_t)L->n * ldx * esz, (int64_t)feat * esz);
         if ((rc = rofk::launch_rows(x_dtype != ROF_F32, a, phase, vec, off32, 0, st))) return rc;
+        a.wave_cap = 0;
         if (L->db.lg_blocks > 0) {
             a.n_tasks = L->db.n_tasks;
             a.n_blocks = L->db.lg_blocks;

@@ -6,6 +6,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstdint>
 
 #include "rof.h"
@@ -43,6 +44,7 @@ struct AggArgs {
     int32_t n_wave, n_tasks;
     int32_t n_blocks;          // logical workgroups
     int32_t xcd_run;           // consecutive logical workgroups kept on one XCD
+    int32_t wave_cap;          // host side only: at most this many wavefronts per SIMD (0: as many as fit)
     int32_t vec_store;         // output rows start on 4-byte boundaries: whole-vector stores
     const float *bias;         // destination-row launch only: added to every output row (null: none)
     int32_t relu;              // destination-row launch only: clamp the output at zero
@@ -68,6 +70,7 @@ __device__ __forceinline__ uint32_t rof_bf16_bits(float f) {
 constexpr int kGathersInFlight = 2;
 constexpr int kWavesPerBlock = 4;
 constexpr int kXcds = 8;
+constexpr int64_t kLdsPerCu = 160 * 1024;
 
 template <typename XT, int VEC>
 struct RowLoad;
@@ -138,6 +141,16 @@ __device__ __forceinline__ const char *row_ptr(int32_t c, const char *xb, uint32
     return b + (uint64_t)r * l;
 }
 
+// Byte address of a lane for ds_bpermute: a per-lane base plus a compile-time constant, added where it is used.
+// Left to the compiler, the 2 * LPR lane numbers of the hand-offs below are loop invariants that it keeps in as
+// many registers (an occupancy step at 10, 12 and 20 lanes per row); the volatile statement pins the addition to
+// its place, one instruction and one short-lived register per hand-off.
+__device__ __forceinline__ int lane_addr(int base, int offset) {
+    int r;
+    asm volatile("v_add_u32 %0, %2, %1" : "=v"(r) : "v"(base), "i"(offset));
+    return r;
+}
+
 // Sum the entries [beg, end) of one task into acc.  WAVE: all lane groups of the wavefront share
 // the task (beg/end wave-uniform) and take every G-th entry; otherwise each lane group owns its
 // task.  ST is the element type of the source rows.  Blocks of U entries that are complete for every
@@ -176,10 +189,12 @@ __device__ __forceinline__ void gather_sum(const char *xb, uint32_t xld, const c
             float wt[U];
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                const int slot = WAVE ? (j0 + u) * G + sub : (j0 + u);          // entry of the chunk
-                const int from = WAVE ? slot : sub * LPR + slot;                // lane that fetched it
-                c[u] = __shfl(mycol, from);
-                wt[u] = __shfl(myw, from);
+                // entry (j0 + u) * G + sub of the wave's chunk (WAVE), entry j0 + u of the lane group's chunk
+                // otherwise: fetched by the lane of that number / by lane sub * LPR + j0 + u
+                constexpr int kStep = WAVE ? G * 4 : 4;
+                const int addr = lane_addr(WAVE ? sub * 4 : sub * LPR * 4, (j0 + u) * kStep);
+                c[u] = __builtin_amdgcn_ds_bpermute(addr, mycol);
+                wt[u] = __int_as_float(__builtin_amdgcn_ds_bpermute(addr, __float_as_int(myw)));
             }
             const int last = WAVE ? (j0 + U - 1) * G + sub : (j0 + U - 1);
             const bool full = __all(idle || base + last < end);
@@ -395,7 +410,8 @@ __global__ __launch_bounds__(256) void rof_rows_kernel(AggArgs a) {
                 for (int k = 0; k < VEC; ++k) {
                     float tot = acc[k];
 #pragma unroll
-                    for (int g = 1; g < G; ++g) tot += __shfl(acc[k], (li + g * LPR) & 63);
+                    for (int g = 1; g < G; ++g)   // from lane li + g * LPR (< 64)
+                        tot += __int_as_float(__builtin_amdgcn_ds_bpermute(lane_addr(li * 4, g * LPR * 4), __float_as_int(acc[k])));
                     acc[k] = tot;
                 }
             }
@@ -540,8 +556,12 @@ int launch_lpr(const AggArgs &a0, int lpr, int lds_rows, hipStream_t st) {
         a.n_blocks = (int32_t)((waves + kWavesPerBlock - 1) / kWavesPerBlock);
     }
     if (a.n_blocks == 0) return ROF_OK;
-    // LDS rows of the workgroup-local groups (none: 0 bytes) on top of the benchmark interface's padding
-    const int64_t lds = (int64_t)g_lds_pad + (CLUSTER ? (int64_t)lds_rows * (lpr * VEC + 4) * 4 : 0);
+    // LDS rows of the workgroup-local groups (none: 0 bytes) on top of the benchmark interface's padding.  A cap
+    // on the wavefronts per SIMD (= workgroups of 4 wavefronts per CU) is put into effect by asking for so much
+    // unused LDS that no more workgroups fit into the CU's 160 KB.
+    int64_t lds = (int64_t)g_lds_pad + (CLUSTER ? (int64_t)lds_rows * (lpr * VEC + 4) * 4 : 0);
+    if (!CLUSTER && a.wave_cap >= 2 && a.wave_cap < 8)
+        lds = std::max<int64_t>(lds, (kLdsPerCu / (a.wave_cap + 1) + 2048) / 2048 * 2048);
     if (lds > 64 * 1024) return ROF_ERR_UNSUPPORTED;
     const int64_t span = (int64_t)kXcds * a.xcd_run;
     const int64_t grid = (a.n_blocks + span - 1) / span * span;

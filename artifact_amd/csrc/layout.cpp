@@ -536,7 +536,8 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     // graphs without that locality short runs balance the XCDs better (R-MAT: 16 is 2-6 % faster than 64, and
     // 1..16 measure alike).
     const int64_t tile_run = std::max<int64_t>(16, std::min<int64_t>(1024, tile_rows / (4 * groups)));
-    L->xcd_run = (gathered > 0 && nearby * 2 >= gathered) ? (int32_t)tile_run : 16;
+    L->local_sources = gathered > 0 && nearby * 2 >= gathered;
+    L->xcd_run = L->local_sources ? (int32_t)tile_run : 16;
     L->n_slots = slots;
     L->n_segments = segments;
     L->gathered_rows = gathered;
