@@ -76,17 +76,19 @@ constexpr int64_t kStreamPartialBytes = 64 << 20;
 // than the L2s, the launch mixes gathers of hub rows, which hit, with gathers that miss, and the miss path of a CU
 // slows down when too many lines are asked for at once: with two row gathers in flight per lane group, rows of up
 // to 64 bytes (16 rows per wavefront) run best at 6 wavefronts per SIMD, rows of two 128-byte lines (129-256 bytes)
-// at 7, all others with every slot taken.  Measured on the 2.4 M-node R-MAT graph (destination-row launch at 8 / 7 /
+// at 7 (6 when their stride lets them straddle a third line), all others with every slot taken.  Measured on the 2.4 M-node R-MAT graph (destination-row launch at 8 / 7 /
 // 6 wavefronts): 16 floats 570 / 558 / 549 us, 32 floats 570 / 581 / 600, 47 floats 972 / 922 / 934, 64 floats
 // 982 / 931 / 938, 100 floats 1052 / 1086 / 1144.  Every other case loses 2-10 % per slot given up: matrices that
 // the caches serve (2^18 nodes x 40 floats; the block model, whose rows gather from their own neighbourhood), the
 // partial-sum launches, and graphs without hub rows (uniform degrees, 2^20 nodes x 64 floats: 689 / 700 us).  The
 // layout knows the latter by having no segmented rows.
 constexpr int64_t kColdMatrixBytes = 128 << 20;   // 4x the L2 of the eight XCDs; the 42 MB matrix above is served, the 154 MB one (16 floats) is not
-int dst_wave_cap(const rof_layout *L, int64_t matrix_bytes, int64_t row_bytes) {
+int dst_wave_cap(const rof_layout *L, int64_t matrix_bytes, int64_t row_bytes, int64_t stride_bytes) {
     if (L->local_sources || L->n_segments == 0 || matrix_bytes < kColdMatrixBytes) return 0;
     if (row_bytes <= 64) return 6;
-    if (row_bytes > 128 && row_bytes <= 256) return 7;
+    // packed rows (47 floats 188 bytes apart) straddle a third line in 44 % of the cases: 1488 / 1448 / 1494 us per
+    // layer at 7 / 6 / 5 wavefronts, against 1257 / 1288 / 1371 for the same rows 192 bytes apart
+    if (row_bytes > 128 && row_bytes <= 256) return stride_bytes % 64 == 0 ? 7 : 6;
     return 0;
 }
 
@@ -503,7 +505,7 @@ static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64
         const int phase = ((int64_t)L->n * feat * (a.out_bf16 ? 2 : 4) >= kStreamOutBytes && a.vec_store && vec > 1 &&
                            (!a.out_bf16 || ldo % 2 == 0)) ? 2 : 1;
         a.n_tasks = L->db.n_regular;   // the clustered destinations at the end of the list have a launch of their own
-        a.wave_cap = dst_wave_cap(L, (int64_t)L->n * ldx * esz, (int64_t)feat * esz);
+        a.wave_cap = dst_wave_cap(L, (int64_t)L->n * ldx * esz, (int64_t)feat * esz, ldx * esz);
         if ((rc = rofk::launch_rows(x_dtype != ROF_F32, a, phase, vec, off32, 0, st))) return rc;
         a.wave_cap = 0;
         if (L->db.lg_blocks > 0) {
