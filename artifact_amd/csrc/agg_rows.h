@@ -155,13 +155,13 @@ __device__ __forceinline__ int lane_addr(int base, int offset) {
 // the task (beg/end wave-uniform) and take every G-th entry; otherwise each lane group owns its
 // task.  ST is the element type of the source rows.  Blocks of U entries that are complete for every
 // lane group run without any per-entry predicate; ragged ends are predicated entry by entry.
-template <typename ST, int VEC, int LPR, bool WAVE, bool DUAL, bool OFF32, bool STREAM_IDS>
+template <typename ST, int VEC, int LPR, bool WAVE, bool DUAL, bool OFF32, bool STREAM_IDS, int INFLIGHT = kGathersInFlight>
 __device__ __forceinline__ void gather_sum(const char *xb, uint32_t xld, const char *pb, uint32_t pld, int32_t nsplit,
                                            int32_t bias, const int32_t *__restrict__ col,
                                            const float *__restrict__ w, int32_t beg, int32_t end, int lane, int sub,
                                            int li, bool act, float (&acc)[VEC]) {
     constexpr int G = 64 / LPR;             // lane groups per wavefront; lanes >= G*LPR stay idle
-    constexpr int U = LPR >= kGathersInFlight ? kGathersInFlight : LPR;   // row gathers in flight per lane group
+    constexpr int U = LPR >= INFLIGHT ? INFLIGHT : LPR;   // row gathers in flight per lane group
     constexpr int CH = WAVE ? G * LPR : LPR;   // entries fetched per step by the wave / by the lane group
     static_assert(LPR % U == 0, "the unroll factor must divide the lanes per row");
     const bool idle = (G * LPR < 64) && lane >= G * LPR;
@@ -338,6 +338,10 @@ __device__ __forceinline__ void finish_row(const AggArgs &a, int32_t t, bool non
 template <typename XT, int VEC, int LPR, int PHASE, bool OFF32>
 __global__ __launch_bounds__(256) void rof_rows_kernel(AggArgs a) {
     constexpr int G = 64 / LPR;
+    // Rows of more than 512 bytes take a whole wavefront each, i.e. two rows in flight per wavefront; the partial-sum
+    // launches, whose sweep mostly hits in L2, run 6-9 % faster with four (2^18 nodes x 256 floats: 133 -> 124 us,
+    // 2.4 M nodes x 160 floats: 2.27 -> 2.13 ms; x 256 floats +0.6 %), the destination rows do not (+8 %, -4 %, +2 %)
+    constexpr int kU = ((PHASE == 0 || PHASE == 3) && LPR == 64) ? 4 : kGathersInFlight;
     // XCD-aware renumbering: the hardware deals workgroup ids round-robin to the 8 XCDs; give each
     // XCD runs of `xcd_run` consecutive logical workgroups instead of every 8th one.
     const int hw = blockIdx.x;
@@ -387,16 +391,16 @@ __global__ __launch_bounds__(256) void rof_rows_kernel(AggArgs a) {
             if (kF32) {
                 // only tasks that reference partial rows pay for the select between the two matrices
                 if (mid > beg)
-                    gather_sum<XT, VEC, LPR, true, true, OFF32, PHASE == 2>(xb, xld, pb, pld, a.nsplit, 0, a.col, a.w, beg, end,
+                    gather_sum<XT, VEC, LPR, true, true, OFF32, PHASE == 2, kU>(xb, xld, pb, pld, a.nsplit, 0, a.col, a.w, beg, end,
                                                                 lane, sub, li, act, acc);
                 else
-                    gather_sum<XT, VEC, LPR, true, false, OFF32, PHASE == 2>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, beg, end, lane,
+                    gather_sum<XT, VEC, LPR, true, false, OFF32, PHASE == 2, kU>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, beg, end, lane,
                                                                  sub, li, act, acc);
             } else {
                 if (mid > beg)
-                    gather_sum<float, VEC, LPR, true, false, OFF32, PHASE == 2>(pb, pld, nullptr, 0, 0, a.nsplit, a.col, a.w, beg,
+                    gather_sum<float, VEC, LPR, true, false, OFF32, PHASE == 2, kU>(pb, pld, nullptr, 0, 0, a.nsplit, a.col, a.w, beg,
                                                                     mid, lane, sub, li, act, acc);
-                gather_sum<XT, VEC, LPR, true, false, OFF32, PHASE == 2>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, mid, end, lane, sub,
+                gather_sum<XT, VEC, LPR, true, false, OFF32, PHASE == 2, kU>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, mid, end, lane, sub,
                                                              li, act, acc);
             }
             if ((G & (G - 1)) == 0) {   // power-of-two group count: butterfly
@@ -418,16 +422,16 @@ __global__ __launch_bounds__(256) void rof_rows_kernel(AggArgs a) {
         } else {
             if (kF32) {
                 if (__any(mid > beg))
-                    gather_sum<XT, VEC, LPR, false, true, OFF32, PHASE == 2>(xb, xld, pb, pld, a.nsplit, 0, a.col, a.w, beg, end,
+                    gather_sum<XT, VEC, LPR, false, true, OFF32, PHASE == 2, kU>(xb, xld, pb, pld, a.nsplit, 0, a.col, a.w, beg, end,
                                                                  lane, sub, li, act, acc);
                 else
-                    gather_sum<XT, VEC, LPR, false, false, OFF32, PHASE == 2>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, beg, end, lane,
+                    gather_sum<XT, VEC, LPR, false, false, OFF32, PHASE == 2, kU>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, beg, end, lane,
                                                                   sub, li, act, acc);
             } else {
                 if (__any(mid > beg))
-                    gather_sum<float, VEC, LPR, false, false, OFF32, PHASE == 2>(pb, pld, nullptr, 0, 0, a.nsplit, a.col, a.w, beg,
+                    gather_sum<float, VEC, LPR, false, false, OFF32, PHASE == 2, kU>(pb, pld, nullptr, 0, 0, a.nsplit, a.col, a.w, beg,
                                                                      mid, lane, sub, li, act, acc);
-                gather_sum<XT, VEC, LPR, false, false, OFF32, PHASE == 2>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, mid, end, lane, sub,
+                gather_sum<XT, VEC, LPR, false, false, OFF32, PHASE == 2, kU>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, mid, end, lane, sub,
                                                               li, act, acc);
             }
         }
