@@ -338,10 +338,12 @@ __device__ __forceinline__ void finish_row(const AggArgs &a, int32_t t, bool non
 template <typename XT, int VEC, int LPR, int PHASE, bool OFF32>
 __global__ __launch_bounds__(256) void rof_rows_kernel(AggArgs a) {
     constexpr int G = 64 / LPR;
-    // Rows of more than 512 bytes take a whole wavefront each, i.e. two rows in flight per wavefront; the partial-sum
-    // launches, whose sweep mostly hits in L2, run 6-9 % faster with four (2^18 nodes x 256 floats: 133 -> 124 us,
-    // 2.4 M nodes x 160 floats: 2.27 -> 2.13 ms; x 256 floats +0.6 %), the destination rows do not (+8 %, -4 %, +2 %)
-    constexpr int kU = ((PHASE == 0 || PHASE == 3) && LPR == 64) ? 4 : kGathersInFlight;
+    // The partial-sum launches sweep the feature matrix and mostly hit in L2; with rows of 16 lanes or more (4 rows
+    // per wavefront or fewer) two gathers in flight leave them short of requests and four run faster wherever the
+    // caches serve the sweep (2^18 nodes x 256 floats: 133 -> 124 us, x 128 floats: 70 -> 59 us; 2.4 M nodes x 160
+    // floats: 2.27 -> 2.13 ms, x 64 / 100 / 128 / 256 floats unchanged).  bf16 rows (8 values to widen per piece)
+    // measured 2 % slower with four, and the destination rows of the same widths +8 %, -4 % and +2 %: both keep two.
+    constexpr int kU = ((PHASE == 0 || PHASE == 3) && LPR >= 16 && sizeof(XT) == 4) ? 4 : kGathersInFlight;
     // XCD-aware renumbering: the hardware deals workgroup ids round-robin to the 8 XCDs; give each
     // XCD runs of `xcd_run` consecutive logical workgroups instead of every 8th one.
     const int hw = blockIdx.x;
