@@ -460,6 +460,8 @@ static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64
     a.nsplit = L->n;
     a.feat = feat;
     int rc;
+    // a feature matrix that the caches serve: more row gathers in flight in every launch (fp32 rows)
+    const bool deep = x_dtype == ROF_F32 && (int64_t)L->n * ldx * esz < kColdMatrixBytes;
     // launches 1 and 2: partial-sum rows (shared groups, then segments of long rows)
     const rof_phase_dev *partial[2] = {&L->dg, &L->ds};
     for (int i = 0; i < 2 && (launches & 1); ++i) {
@@ -477,7 +479,7 @@ static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64
         a.n_tasks = d.n_tasks;
         a.xcd_run = g_xcd_run_a;
         a.vec_store = 1;
-        const int phase = (int64_t)d.n_tasks * feat * 4 >= kStreamPartialBytes && vec > 1 ? 3 : 0;
+        const int phase = (int64_t)d.n_tasks * feat * 4 >= kStreamPartialBytes && vec > 1 ? 3 : deep ? 5 : 0;
         if ((rc = rofk::launch_rows(x_dtype != ROF_F32, a, phase, vec, off32, 0, st))) return rc;
     }
     if (L->db.n_tasks && (launches & 2)) {   // last launch: destination rows
@@ -503,7 +505,7 @@ static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64
         a.lg_col = L->db.lg_col;
         a.lg_w = normalized ? L->db.lg_w : nullptr;
         const int phase = ((int64_t)L->n * feat * (a.out_bf16 ? 2 : 4) >= kStreamOutBytes && a.vec_store && vec > 1 &&
-                           (!a.out_bf16 || ldo % 2 == 0)) ? 2 : 1;
+                           (!a.out_bf16 || ldo % 2 == 0)) ? 2 : deep ? 4 : 1;
         a.n_tasks = L->db.n_regular;   // the clustered destinations at the end of the list have a launch of their own
         a.wave_cap = dst_wave_cap(L, (int64_t)L->n * ldx * esz, (int64_t)feat * esz, ldx * esz);
         if ((rc = rofk::launch_rows(x_dtype != ROF_F32, a, phase, vec, off32, 0, st))) return rc;

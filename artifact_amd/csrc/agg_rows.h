@@ -235,7 +235,7 @@ __device__ __forceinline__ void gather_sum(const char *xb, uint32_t xld, const c
     }
 }
 
-// Scale the finished sum of task t, apply the layer's epilogue (PHASE 1 and 2) and store this lane's piece of the
+// Scale the finished sum of task t, apply the layer's epilogue (PHASE 1, 2 and 4) and store this lane's piece of the
 // output row.  `acc` holds the columns cstart .. cstart + VEC - 1; `skip` of them repeat the neighbouring lane's.
 template <typename XT, int VEC, int PHASE>
 __device__ __forceinline__ void finish_row(const AggArgs &a, int32_t t, bool nonempty, const float (&acc)[VEC], const char *xb,
@@ -248,7 +248,7 @@ __device__ __forceinline__ void finish_row(const AggArgs &a, int32_t t, bool non
     float r[VEC];
 #pragma unroll
     for (int k = 0; k < VEC; ++k) r[k] = acc[k] * s;
-    constexpr bool kDst = PHASE == 1 || PHASE == 2;   // a destination-row launch
+    constexpr bool kDst = PHASE == 1 || PHASE == 2 || PHASE == 4;   // a destination-row launch
     if (kDst) {   // epilogue of the layer: + own row, + bias, then ReLU (columns cstart .. cstart+VEC-1 exist)
         if (a.self_weight != 0.0f) {
             float own[VEC];
@@ -334,7 +334,8 @@ __device__ __forceinline__ void finish_row(const AggArgs &a, int32_t t, bool non
 // streaming stores (a workspace too large to stay in the caches until the destination rows read it); PHASE 1: the
 // destination-row launch; PHASE 2: the same with the output rows written as streaming stores and the index arrays
 // read as streaming loads (large outputs, hence large graphs).  (A run-time switch between the two kinds of store does
-// not survive the optimiser, which merges the two stores into an ordinary one.)
+// not survive the optimiser, which merges the two stores into an ordinary one.)  PHASE 5 and 4: PHASE 0 and 1 with
+// more row gathers in flight, for feature matrices that the caches serve (fp32 rows only).
 template <typename XT, int VEC, int LPR, int PHASE, bool OFF32>
 __global__ __launch_bounds__(256) void rof_rows_kernel(AggArgs a) {
     constexpr int G = 64 / LPR;
@@ -343,7 +344,12 @@ __global__ __launch_bounds__(256) void rof_rows_kernel(AggArgs a) {
     // caches serve the sweep (2^18 nodes x 256 floats: 133 -> 124 us, x 128 floats: 70 -> 59 us; 2.4 M nodes x 160
     // floats: 2.27 -> 2.13 ms, x 64 / 100 / 128 / 256 floats unchanged).  bf16 rows (8 values to widen per piece)
     // measured 2 % slower with four, and the destination rows of the same widths +8 %, -4 % and +2 %: both keep two.
-    constexpr int kU = ((PHASE == 0 || PHASE == 3) && LPR >= 16 && sizeof(XT) == 4) ? 4 : kGathersInFlight;
+    // A matrix that the caches serve answers quickly, and two gathers per lane group leave every launch short of
+    // requests: four (five at 10 lanes per row) measured -18 % on the 2^14-node workload (32 floats), -8.5 % at
+    // 2^18 nodes x 32 floats, -15 % at 2^14 x 256; 0 on the block model and +2 ... +8 % on matrices of 0.27-2.5 GB.
+    constexpr bool kDeep = PHASE == 4 || PHASE == 5;
+    constexpr int kU = kDeep ? (LPR % 4 == 0 ? 4 : LPR % 5 == 0 ? 5 : kGathersInFlight)
+                             : ((PHASE == 0 || PHASE == 3) && LPR >= 16 && sizeof(XT) == 4) ? 4 : kGathersInFlight;
     // XCD-aware renumbering: the hardware deals workgroup ids round-robin to the 8 XCDs; give each
     // XCD runs of `xcd_run` consecutive logical workgroups instead of every 8th one.
     const int hw = blockIdx.x;
@@ -600,27 +606,28 @@ int launch_lpr(const AggArgs &a0, int lpr, int lds_rows, hipStream_t st) {
     return ROF_OK;
 }
 
-// Instantiated in agg_rows_{f32,bf16}_partial.hip (partial-sum launches; stream: phase 3), agg_rows_{f32,bf16}_dst.hip (destination
+// Instantiated in agg_rows_{f32,bf16}_partial.hip (partial-sum launches; phase 0, 3 or 5 / stream: phase 3), agg_rows_{f32,bf16}_dst.hip (destination
 // rows; phase 1, or 2 = streaming stores) and agg_cluster_{f32,bf16}.hip (the clustered destination rows: a.n_blocks
 // clusters whose workgroups need lds_rows LDS rows), one translation unit each so that the build runs them side by side.
 // off32: every byte offset into the feature matrix and into the partial-sum workspace fits 32 bits and
 // every row id fits 24 bits, so the kernels may use the short address arithmetic.
-int launch_rows_f32_partial(const AggArgs &a, bool stream, int vec, bool off32, hipStream_t st);
+int launch_rows_f32_partial(const AggArgs &a, int phase, int vec, bool off32, hipStream_t st);
 int launch_rows_f32_dst(const AggArgs &a, int phase, int vec, bool off32, hipStream_t st);
 int launch_rows_f32_cluster(const AggArgs &a, int phase, int vec, bool off32, int lds_rows, hipStream_t st);
 int launch_rows_bf16_partial(const AggArgs &a, bool stream, int vec, bool off32, hipStream_t st);
 int launch_rows_bf16_dst(const AggArgs &a, int phase, int vec, bool off32, hipStream_t st);
 int launch_rows_bf16_cluster(const AggArgs &a, int phase, int vec, bool off32, int lds_rows, hipStream_t st);
 
-// phase 0: partial-sum launches, 3: the same with streaming stores; 1: destination rows, 2: destination rows with
-// streaming stores; lds_rows > 0: the cluster launch of the destination rows
+// phase 0: partial-sum launches, 3: the same with streaming stores, 5: with more gathers in flight; 1: destination
+// rows, 2: with streaming stores, 4: with more gathers in flight (5 and 4 exist for fp32 vector rows with short
+// offsets and run as 0 and 1 otherwise); lds_rows > 0: the cluster launch of the destination rows
 inline int launch_rows(bool bf16, const AggArgs &a, int phase, int vec, bool off32, int lds_rows, hipStream_t st) {
-    if (phase == 0 || phase == 3)
-        return bf16 ? launch_rows_bf16_partial(a, phase == 3, vec, off32, st) : launch_rows_f32_partial(a, phase == 3, vec, off32, st);
+    if (phase == 0 || phase == 3 || phase == 5)
+        return bf16 ? launch_rows_bf16_partial(a, phase == 3, vec, off32, st) : launch_rows_f32_partial(a, phase, vec, off32, st);
     if (lds_rows > 0)
-        return bf16 ? launch_rows_bf16_cluster(a, phase, vec, off32, lds_rows, st)
-                    : launch_rows_f32_cluster(a, phase, vec, off32, lds_rows, st);
-    return bf16 ? launch_rows_bf16_dst(a, phase, vec, off32, st) : launch_rows_f32_dst(a, phase, vec, off32, st);
+        return bf16 ? launch_rows_bf16_cluster(a, phase == 2 ? 2 : 1, vec, off32, lds_rows, st)
+                    : launch_rows_f32_cluster(a, phase == 2 ? 2 : 1, vec, off32, lds_rows, st);
+    return bf16 ? launch_rows_bf16_dst(a, phase == 2 ? 2 : 1, vec, off32, st) : launch_rows_f32_dst(a, phase, vec, off32, st);
 }
 
 }  // namespace rofk

@@ -1,4 +1,5 @@
-// fp32-feature instantiations of the row-gather kernel: the destination-row launch (PHASE 1 and 2).
+// fp32-feature instantiations of the row-gather kernel: the destination-row launch (PHASE 1; PHASE 2 with streaming
+// stores; PHASE 4 with more gathers in flight).
 #include "agg_rows.h"
 
 namespace rofk {
@@ -13,7 +14,8 @@ static int launch(const AggArgs &a, int vec, bool off32, hipStream_t st) {
 }
 
 int launch_rows_f32_dst(const AggArgs &a, int phase, int vec, bool off32, hipStream_t st) {
-    return phase == 1 ? launch<1>(a, vec, off32, st) : launch<2>(a, vec, off32, st);
+    if (phase == 4 && vec == 4 && off32) return launch_lpr<float, 4, 4, true, false>(a, rof_lanes_per_row(a.feat, vec), 0, st);
+    return phase == 2 ? launch<2>(a, vec, off32, st) : launch<1>(a, vec, off32, st);
 }
 
 }  // namespace rofk
