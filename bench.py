@@ -300,8 +300,8 @@ def traffic_child(args):
 def read_counter_csv(path):
     """One rocprofv3 counter_collection.csv of a counter run -> ({(counter, phase): value per aggregation},
     {counter: value of the calibration copy}).  Phase 0 = the partial-sum launches (shared groups, segments of long
-    rows; template argument PHASE of the kernel name <XT, VEC, LPR, PHASE, OFF32> is 0, or 3 with streamed partial
-    rows), phase 1 = the destination rows and their clusters (PHASE 1 or 2).  A phase may consist of two launches, so the dispatches of one phase are summed and divided
+    rows; template argument PHASE of the kernel name <XT, VEC, LPR, PHASE, OFF32> is 0, 3 with streamed partial
+    rows or 5 with more gathers in flight), phase 1 = the destination rows and their clusters (PHASE 1, 2 or 4).  A phase may consist of two launches, so the dispatches of one phase are summed and divided
     by the number of aggregations the run executes."""
     acc, copy = collections.defaultdict(float), {}
     with open(path) as f:
@@ -311,9 +311,9 @@ def read_counter_csv(path):
                 copy[row["Counter_Name"]] = float(row["Counter_Value"])
             elif "rof_rows_kernel" in k or "rof_cluster_kernel" in k:
                 phase = int(k.split("<")[1].split(">")[0].split(",")[3])
-                if phase not in (0, 1, 2, 3):
+                if phase not in (0, 1, 2, 3, 4, 5):
                     raise ValueError(f"unknown launch kind in kernel name {k!r}")
-                acc[(row["Counter_Name"], 0 if phase in (0, 3) else 1)] += float(row["Counter_Value"])
+                acc[(row["Counter_Name"], 0 if phase in (0, 3, 5) else 1)] += float(row["Counter_Value"])
     return {k: v / CHILD_AGGREGATIONS for k, v in acc.items()}, copy
 
 

@@ -27,9 +27,10 @@ def test_counter_file_is_summed_per_phase_and_aggregation(tmp_path):
         2097152, "FETCH_SIZE", 524288.0)
     add("at::native::some_other_kernel<float, 4, 12, 2, true>()", 64, "FETCH_SIZE", 99.0)
     for _ in range(bench.CHILD_AGGREGATIONS):
-        add("void rofk::rof_rows_kernel<float, 4, 12, 0, true>(rofk::AggArgs)", 174080, "FETCH_SIZE", 10.0)      # groups
+        add("void rofk::rof_rows_kernel<float, 4, 12, 5, true>(rofk::AggArgs)", 174080, "FETCH_SIZE", 10.0)      # groups
         add("void rofk::rof_rows_kernel<float, 4, 12, 3, true>(rofk::AggArgs)", 9205760, "FETCH_SIZE", 1000.0)   # segments, streamed
-        add("void rofk::rof_rows_kernel<float, 4, 12, 2, true>(rofk::AggArgs)", 36012032, "FETCH_SIZE", 3000.0)  # rows
+        add("void rofk::rof_rows_kernel<float, 4, 12, 2, true>(rofk::AggArgs)", 36012032, "FETCH_SIZE", 2000.0)  # rows
+        add("void rofk::rof_rows_kernel<float, 4, 12, 4, true>(rofk::AggArgs)", 36012032, "FETCH_SIZE", 1000.0)  # rows, more in flight
         add("void rofk::rof_cluster_kernel<unsigned short, 8, 32, 1, false>(rofk::AggArgs)", 4096, "FETCH_SIZE", 500.0)
     path = tmp_path / "rof_counter_collection.csv"
     path.write_text("\n".join(rows) + "\n")
