@@ -149,6 +149,25 @@ def test_deterministic_run_to_run():
     assert torch.equal(a, b)                                 # no atomics: bitwise repeatable
 
 
+@pytest.mark.parametrize("feat,lanes", [(32, 8), (40, 10), (47, 12), (256, 64)])
+def test_gathers_in_flight_do_not_change_the_bits(feat, lanes):
+    """A feature matrix under 128 MB runs the instantiations with four (five at 10 lanes per row) row gathers in
+    flight, a larger one those with two; both add the same terms in the same order.  The same rows are aggregated
+    once packed and once as a view of a buffer whose row stride puts the matrix above 128 MB."""
+    indptr, indices, plan = _case("c1", 0, 3)
+    n = len(indptr) - 1
+    lay = _layout(plan, n, 3, min_consumers=2, lanes_per_row=lanes)    # three launches: groups, segments, rows
+    lay.set_degrees(torch.from_numpy(np.diff(indptr).astype(np.float32)).cuda())
+    x = torch.from_numpy(features(n, feat, seed=9)).cuda()
+    wide = (128 << 20) // (4 * n) + 8                                   # floats per row of the large buffer
+    assert n * wide * 4 >= (128 << 20) > n * feat * 4
+    big = torch.zeros((n, wide), device="cuda")
+    big[:, :feat] = x
+    a = lay.aggregate(x).clone()
+    b = lay.aggregate(big[:, :feat], feat_dim=feat).clone()
+    assert torch.equal(a, b)
+
+
 def test_empty_rows_and_isolated_nodes(oracle):
     indptr = np.array([0, 0, 2, 2, 3, 3, 3, 3, 3, 3, 3], dtype=np.int32)   # nodes 0,2,4.. have no in-edges
     indices = np.array([3, 1, 1], dtype=np.int32)
