@@ -151,7 +151,7 @@ def test_deterministic_run_to_run():
 
 @pytest.mark.parametrize("feat,lanes", [(32, 8), (40, 10), (47, 12), (256, 64)])
 def test_gathers_in_flight_do_not_change_the_bits(feat, lanes):
-    """A feature matrix under 128 MB runs the instantiations with four (five at 10 lanes per row) row gathers in
+    """A feature matrix under 96 MB runs the instantiations with four (five at 10 lanes per row) row gathers in
     flight, a larger one those with two; both add the same terms in the same order.  The same rows are aggregated
     once packed and once as a view of a buffer whose row stride puts the matrix above 128 MB."""
     indptr, indices, plan = _case("c1", 0, 3)
