@@ -49,6 +49,13 @@ int32_t default_cut(int32_t groups, int32_t elem_bytes) {
     const int32_t cut = groups <= 2 ? 128 : groups == 3 ? 256 : groups == 4 ? 384 : 640;
     return std::min(640, elem_bytes == 2 ? 2 * cut : cut);
 }
+// Segments are a quarter of the cut; 3/16 for bf16 rows of more than 256 bytes (G <= 2), whose partial rows are
+// streamed.  2^22-node R-MAT, 256 bf16 columns, cut 256: segments of 32 / 40 / 48 / 56 / 64 / 96 / 128 entries
+// 8.53 / 8.49 / 8.46 / 8.57 / 8.57 / 8.92 / 9.17 ms.  Narrower bf16 rows (128, 64 columns) and fp32 rows
+// (2^18 nodes x 256 floats: 24 / 28 / 32 / 40 entries 0.400 / 0.377 / 0.378 / 0.380 ms) stay at a quarter.
+int32_t default_segment(int32_t cut, int32_t groups, int32_t elem_bytes) {
+    return std::max(16, elem_bytes == 2 && groups <= 2 ? cut * 3 / 16 : cut / 4);
+}
 // Sharing groups costs one more launch (~4-6 us on MI355X), and on heavy-tailed graphs what it saves is cheap:
 // the sources of a popular group are themselves popular rows that sit in L2, while the partial rows that
 // replace them are read a few dozen times each.  Measured gain of the destination-row launch against the net
@@ -377,7 +384,7 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     const int32_t groups = std::max(1, 64 / lpr);
     const int64_t total = (int64_t)L->res_col.size() + (int64_t)L->group_dst.size();
     const int32_t hub_split = (o && o->hub_split > 0) ? o->hub_split : default_cut(groups, o ? o->elem_bytes : 4);
-    const int32_t segment = (o && o->segment > 0) ? o->segment : std::max(16, hub_split / 4);
+    const int32_t segment = (o && o->segment > 0) ? o->segment : default_segment(hub_split, groups, o ? o->elem_bytes : 4);
     L->hub_split = hub_split;
     L->segment = segment;
     const bool disable = o && o->disable_reuse;

@@ -201,11 +201,12 @@ def test_random_graphs_with_shared_neighbour_sets_through_clusters(oracle, seed)
     assert st["gathered_rows"] == total - nref - st["lds_reads"] <= len(ix)
 
 
-@pytest.mark.parametrize("lanes,elem,cut,seg", [(64, 4, 128, 32), (32, 4, 128, 32), (32, 2, 256, 64), (16, 4, 384, 96),
-                                                (12, 4, 640, 160), (8, 0, 640, 160)])
+@pytest.mark.parametrize("lanes,elem,cut,seg", [(64, 4, 128, 32), (32, 4, 128, 32), (32, 2, 256, 48), (16, 2, 640, 160),
+                                                (16, 4, 384, 96), (12, 4, 640, 160), (8, 0, 640, 160)])
 def test_long_rows_are_cut_by_width_and_their_segments_swept_by_source_id(lanes, elem, cut, seg):
     """Default cut by the rows a wavefront gathers at once (128 up to two, 384 at four, 640 from five on; doubled
-    for bf16 rows, whose partial rows are twice as wide), segments a quarter of it; the segment tasks come in the
+    for bf16 rows, whose partial rows are twice as wide), segments a quarter of it (3/16 for bf16 rows of more than
+    256 bytes); the segment tasks come in the
     order of the highest source id they gather (each task lists its sources by descending id), long tasks before
     packed ones."""
     ip, ix = make_workload("c4", 2)                          # 600 000 rows: enough segments to fill the machine
