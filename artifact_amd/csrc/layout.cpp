@@ -540,11 +540,12 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     // a run covers one whole tile of destinations (a workgroup packs 4 x `groups` short rows), so that the tile's
     // sources are fetched into one L2 only: measured on a block-structured graph of 4096-node blocks, 256
     // workgroups (= one tile at 4 rows per wavefront) are 11 % faster than 64 and 16 % faster than 16.  On
-    // graphs without that locality short runs balance the XCDs better (R-MAT: 16 is 2-6 % faster than 64, and
-    // 1..16 measure alike).
+    // graphs without that locality short runs balance the XCDs better (R-MAT, 2.4 M nodes: runs of 4 were 0-2 %
+    // faster than 16 at every width from 16 to 100 floats on two devices and equal on a third, 1 and 2 are 0.9 %
+    // slower than 4, 64 is 1-6 % slower; smaller graphs measure alike from 2 to 16).
     const int64_t tile_run = std::max<int64_t>(16, std::min<int64_t>(1024, tile_rows / (4 * groups)));
     L->local_sources = gathered > 0 && nearby * 2 >= gathered;
-    L->xcd_run = L->local_sources ? (int32_t)tile_run : 16;
+    L->xcd_run = L->local_sources ? (int32_t)tile_run : 4;
     L->n_slots = slots;
     L->n_segments = segments;
     L->gathered_rows = gathered;

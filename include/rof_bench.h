@@ -34,7 +34,7 @@ int rof_device_copy(void *dst, const void *src, size_t nbytes, void *stream);
 /* Launch tuning: how many consecutive workgroups of the partial-sum launches / of the destination-row launch
  * stay on one XCD (each XCD has its own L2, so runs of neighbouring destination rows share gathered rows
  * there).  run_launch2 = 0 (the default) lets every layout use its own choice: one tile of destinations per
- * run when at least half of the neighbours lie within 8192 ids of their row (block-structured graphs), 16
+ * run when at least half of the neighbours lie within 8192 ids of their row (block-structured graphs), 4
  * workgroups otherwise.  Process-wide; no upstream counterpart. */
 int rof_set_xcd_run(int run_launch1, int run_launch2);
 

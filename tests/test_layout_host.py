@@ -239,7 +239,7 @@ def test_xcd_run_follows_the_locality_of_the_graph():
     assert Layout.from_csr(ip, ix).export()["xcd_run"] == 256               # 4096-row tile / (4 wavefronts x 4 rows)
     assert Layout.from_csr(ip, ix, lanes_per_row=64).export()["xcd_run"] == 1024
     ip, ix = make_workload("c4", 3)                          # R-MAT, 300 000 nodes: 9 % of the neighbours are nearby
-    assert Layout.from_csr(ip, ix).export()["xcd_run"] == 16
+    assert Layout.from_csr(ip, ix).export()["xcd_run"] == 4
 
 
 def test_long_tasks_come_first_and_short_tasks_are_sorted_inside_tiles():
