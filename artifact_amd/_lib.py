@@ -19,7 +19,8 @@ SYMBOLS = (
     "rof_part_intersect_count", "rof_part_intersect_lists", "rof_greedy_max_reuse", "rof_reorganize",
     "rof_transpose_csr", "rof_plan_build", "rof_layout_from_v2", "rof_layout_from_v1", "rof_layout_from_parts",
     "rof_layout_export", "rof_layout_stats", "rof_layout_upload", "rof_layout_set_degrees",
-    "rof_plan_hub_patterns", "rof_plan_dynamic_greedy", "rof_column_sums", "rof_column_sums_workspace_bytes", "rof_layout_workspace_bytes", "rof_layout_free", "rof_aggregate", "rof_aggregate_epilogue", "rof_aggregate_noalloc", "rof_aggregate_timed", "rof_set_xcd_run", "rof_aggregate_launch_times", "rof_device_copy", "rof_set_lds_pad",
+    "rof_plan_hub_patterns", "rof_plan_dynamic_greedy", "rof_column_sums", "rof_column_sums_workspace_bytes", "rof_layout_workspace_bytes", "rof_layout_free", "rof_aggregate", "rof_aggregate_epilogue", "rof_aggregate_noalloc", "rof_aggregate_timed", "rof_aggregate_launch_times",
+    "rof_device_copy", "rof_device_read", "rof_layout_set_tuning", "rof_layout_get_tuning", "rof_layout_stats_n",
 )
 
 
@@ -31,7 +32,12 @@ class LayoutOpts(C.Structure):
     _fields_ = [("min_consumers", C.c_int32), ("disable_reuse", C.c_int32), ("hub_split", C.c_int32),
                 ("segment", C.c_int32), ("lanes_per_row", C.c_int32), ("entry_order", C.c_int32),
                 ("tile_rows", C.c_int32), ("elem_bytes", C.c_int32), ("local_groups", C.c_int32),
-                ("reserved", C.c_int32 * 3)]
+                ("share_scope", C.c_int32), ("reserved", C.c_int32 * 2)]
+
+
+class LaunchTuning(C.Structure):
+    _fields_ = [("xcd_run_partial", C.c_int32), ("xcd_run_dst", C.c_int32), ("wave_cap", C.c_int32),
+                ("lds_pad", C.c_int32), ("reserved", C.c_int32 * 4)]
 
 
 class Epilogue(C.Structure):
@@ -80,11 +86,13 @@ def lib():
     L.rof_aggregate_noalloc.argtypes = [vp, vp, ci, i64, vp, i64, ci, ci, C.POINTER(Epilogue), vp]
     L.rof_aggregate_timed.argtypes = [vp, vp, ci, i64, vp, i64, ci, ci, C.POINTER(Epilogue), vp, C.c_size_t, vp, ci,
                                       C.POINTER(C.c_float)]
-    L.rof_set_xcd_run.argtypes = [ci, ci]
+    L.rof_layout_set_tuning.argtypes = [vp, C.POINTER(LaunchTuning)]
+    L.rof_layout_get_tuning.argtypes = [vp, C.POINTER(LaunchTuning)]
+    L.rof_layout_stats_n.argtypes = [vp, vp, ci]
+    L.rof_device_read.argtypes = [vp, C.c_size_t, vp, vp]
     L.rof_column_sums_workspace_bytes.argtypes = [i64, ci]
     L.rof_column_sums_workspace_bytes.restype = C.c_size_t
     L.rof_column_sums.argtypes = [vp, ci, i64, i64, ci, vp, vp, C.c_size_t, vp]
-    L.rof_set_lds_pad.argtypes = [ci]
     L.rof_device_copy.argtypes = [vp, vp, C.c_size_t, vp]
     L.rof_aggregate_launch_times.argtypes = [vp, vp, ci, i64, vp, i64, ci, ci, C.POINTER(Epilogue), vp, C.c_size_t, vp, ci,
                                              C.POINTER(C.c_float * 2)]

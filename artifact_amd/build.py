@@ -3,7 +3,9 @@
     python -m artifact_amd.build
 
 hipcc cross-compiles for gfx950 without a GPU.  The library is loaded with ctypes
-(artifact_amd/_lib.py); nothing here links against PyTorch.
+(artifact_amd/_lib.py) and does not link against PyTorch.  `build_torch_module` then compiles the thin
+C++ module `artifact_amd/_ROF*.so` (csrc/rof_torch.cpp: upstream's seven `ROF` operators over the C ABI),
+which links against PyTorch and librof.so.
 """
 from __future__ import annotations
 
@@ -58,7 +60,38 @@ def build_library(verbose=True):
     return LIB
 
 
+def torch_module_path():
+    import sysconfig
+
+    return os.path.join(HERE, "_ROF" + sysconfig.get_config_var("EXT_SUFFIX"))
+
+
+def build_torch_module():
+    """csrc/rof_torch.cpp -> artifact_amd/_ROF<ext suffix>.so with g++ against the installed PyTorch's headers and
+    libraries (host code only: the kernels are in librof.so, found at run time next to the module)."""
+    import sysconfig
+
+    import torch
+    from torch.utils import cpp_extension
+
+    gxx = shutil.which("g++") or "g++"
+    tlib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    out = torch_module_path()
+    cmd = [gxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-w", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           "-DTORCH_EXTENSION_NAME=_ROF", "-DTORCH_API_INCLUDE_EXTENSION_H",
+           f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
+           "-I" + os.path.join(ROOT, "include")]
+    cmd += ["-I" + p for p in cpp_extension.include_paths()] + ["-I" + os.path.join(rocm, "include"),
+                                                                 "-I" + sysconfig.get_paths()["include"]]
+    cmd += [os.path.join(CSRC, "rof_torch.cpp"), "-o", out, "-L" + tlib, "-lc10", "-lc10_hip", "-ltorch", "-ltorch_cpu",
+            "-ltorch_hip", "-ltorch_python", "-L" + HERE, "-l:librof.so", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + tlib]
+    _run(cmd)
+    return out
+
+
 if __name__ == "__main__":
     build_library()
     print("built", LIB)
+    print("built", build_torch_module())
     sys.exit(0)

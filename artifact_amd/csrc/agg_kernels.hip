@@ -45,15 +45,7 @@
 #include "rof_bench.h"
 #include "rof_internal.h"
 
-namespace rofk {
-int g_xcd_run_a = 1, g_xcd_run_b = 0;   // 0: each layout's own choice for the destination-row launch
-int g_lds_pad = 0;
-}  // namespace rofk
-
 using rofk::AggArgs;
-using rofk::g_lds_pad;
-using rofk::g_xcd_run_a;
-using rofk::g_xcd_run_b;
 
 namespace {
 
@@ -116,6 +108,27 @@ __global__ void rof_copy_kernel(const float4 *__restrict__ src, float4 *__restri
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (; i < n16; i += stride) dst[i] = src[i];
+}
+
+// plain streaming read (every 16-byte piece once, four loads in flight per lane); the sums go to `sink` only so that
+// the loads cannot be dropped.  Gives the read rate the memory system sustains, against which gather traffic is put.
+__global__ __launch_bounds__(256) void rof_read_kernel(const float4 *__restrict__ src, int64_t n16, float *__restrict__ sink) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    for (; i + 3 * stride < n16; i += 4 * stride) {
+        const float4 p = src[i], q = src[i + stride], r = src[i + 2 * stride], t = src[i + 3 * stride];
+        a0 += p.x + p.y + p.z + p.w;
+        a1 += q.x + q.y + q.z + q.w;
+        a2 += r.x + r.y + r.z + r.w;
+        a3 += t.x + t.y + t.z + t.w;
+    }
+    for (; i < n16; i += stride) {
+        const float4 p = src[i];
+        a0 += p.x + p.y + p.z + p.w;
+    }
+    const float tot = (a0 + a1) + (a2 + a3);
+    if (tot == 1.2345e-30f) sink[0] = tot;   // practically never true; keeps the loads alive
 }
 
 // Column sums of a row-major [n, f] matrix (the bias gradient of a layer), in two launches with a fixed
@@ -307,19 +320,28 @@ const char *rof_strerror(int status) {
     }
 }
 
-int rof_version(void) { return 2; }
+int rof_version(void) { return ROF_ABI_VERSION; }
 
-// Tuning knobs used by the benchmark sweeps.
-int rof_set_lds_pad(int bytes) {
-    if (bytes < 0 || bytes > 64 * 1024) return ROF_ERR_ARG;
-    g_lds_pad = bytes;
+// Launch tuning of one layout, used by the benchmark sweeps.
+int rof_layout_set_tuning(rof_layout *L, const rof_launch_tuning *t) {
+    if (!L || !t) return ROF_ERR_ARG;
+    if (t->xcd_run_partial < 0 || t->xcd_run_dst < 0 || t->xcd_run_partial > 4096 || t->xcd_run_dst > 4096) return ROF_ERR_ARG;
+    if (t->wave_cap < -1 || t->wave_cap == 1 || t->wave_cap > 7) return ROF_ERR_ARG;
+    if (t->lds_pad < 0 || t->lds_pad > 64 * 1024) return ROF_ERR_ARG;
+    L->tune_xcd_run_partial = t->xcd_run_partial;
+    L->tune_xcd_run_dst = t->xcd_run_dst;
+    L->tune_wave_cap = t->wave_cap;
+    L->tune_lds_pad = t->lds_pad;
     return ROF_OK;
 }
 
-int rof_set_xcd_run(int run_a, int run_b) {
-    if (run_a < 1 || run_b < 0 || run_a > 4096 || run_b > 4096) return ROF_ERR_ARG;
-    g_xcd_run_a = run_a;
-    g_xcd_run_b = run_b;
+int rof_layout_get_tuning(const rof_layout *L, rof_launch_tuning *t) {
+    if (!L || !t) return ROF_ERR_ARG;
+    memset(t, 0, sizeof(*t));
+    t->xcd_run_partial = L->tune_xcd_run_partial;
+    t->xcd_run_dst = L->tune_xcd_run_dst;
+    t->wave_cap = L->tune_wave_cap;
+    t->lds_pad = L->tune_lds_pad;
     return ROF_OK;
 }
 
@@ -359,6 +381,15 @@ int rof_device_copy(void *dst, const void *src, size_t nbytes, void *stream) {
     return ROF_OK;
 }
 
+int rof_device_read(const void *src, size_t nbytes, float *sink, void *stream) {
+    if (!src || !sink || (nbytes & 15) || ((uintptr_t)src & 15)) return ROF_ERR_ARG;
+    if (nbytes == 0) return ROF_OK;
+    hipLaunchKernelGGL(rof_read_kernel, dim3(256 * 32), dim3(256), 0, (hipStream_t)stream, (const float4 *)src,
+                       (int64_t)(nbytes / 16), sink);
+    HIP_TRY(hipGetLastError());
+    return ROF_OK;
+}
+
 int rof_layout_upload(rof_layout *L, void *stream) {
     if (!L) return ROF_ERR_ARG;
     if (L->uploaded) return ROF_OK;
@@ -376,8 +407,11 @@ int rof_layout_upload(rof_layout *L, void *stream) {
     }
     HIP_TRY(hipStreamSynchronize(st));   // the host vectors may be released after this call
     L->uploaded = true;
-    void *unused = nullptr;   // set-up is also where this device's copy of the static scratch gets its address
-    return scratch_of_current_device(&unused);
+    // set-up is also where this device's copy of the static scratch gets its address; best effort here, because a
+    // caller who never uses rof_aggregate_noalloc must not see its failures (that entry point reports them itself)
+    void *unused = nullptr;
+    (void)scratch_of_current_device(&unused);
+    return ROF_OK;
 }
 
 int rof_layout_set_degrees(rof_layout *L, const float *deg, void *stream) {
@@ -452,6 +486,20 @@ static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64
     const bool off32 = rows_x < (1 << 24) && rows_p < (1 << 24) && ldx * esz < (1 << 24) && ldp * 4 < (1 << 24) &&
                        (rows_x + 1) * ldx * esz < ((int64_t)1 << 32) && (rows_p + 1) * ldp * 4 < ((int64_t)1 << 32);
 
+    // every launch of the call is checked before the first one is enqueued, so that a refusal leaves `out` untouched
+    {
+        const int lpr = rofk::rof_lanes_per_row(feat, vec);
+        const int cap = L->tune_wave_cap >= 0 ? L->tune_wave_cap
+                                              : dst_wave_cap(L, (int64_t)L->n * ldx * esz, (int64_t)feat * esz, ldx * esz);
+        const int64_t plain_lds = rofk::lds_request(false, lpr, vec, 0, cap, L->tune_lds_pad);
+        const int64_t cluster_lds = L->db.lg_blocks > 0
+                                        ? rofk::lds_request(true, lpr, vec, L->db.lg_max_rows, 0, L->tune_lds_pad) : 0;
+        if (plain_lds > rofk::kMaxLdsRequest || cluster_lds > rofk::kMaxLdsRequest) {
+            rof_set_device_error("rof_aggregate", "the LDS rows of the layout's clusters do not fit a workgroup's 64 KB at this "
+                                                  "feature width; build the layout for this width (lanes_per_row, elem_bytes)");
+            return ROF_ERR_UNSUPPORTED;
+        }
+    }
     AggArgs a;
     memset(&a, 0, sizeof(a));
     a.x = x;
@@ -460,6 +508,7 @@ static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64
     a.ldp = ldp;
     a.nsplit = L->n;
     a.feat = feat;
+    a.lds_pad = L->tune_lds_pad;
     int rc;
     // a feature matrix that the caches serve: more row gathers in flight in every launch (fp32 rows).  2^18-node
     // R-MAT graph against two in flight: 42 MB -8 %, 67 MB -7 %, 84 MB -2.8 %, 105 MB 0, 126 MB +1.9 %.
@@ -479,7 +528,7 @@ static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64
         a.ldo = ldp;
         a.n_wave = d.n_wave;
         a.n_tasks = d.n_tasks;
-        a.xcd_run = g_xcd_run_a;
+        a.xcd_run = L->tune_xcd_run_partial > 0 ? L->tune_xcd_run_partial : 1;
         a.vec_store = 1;
         const int phase = (int64_t)d.n_tasks * feat * 4 >= kStreamPartialBytes && vec > 1 ? 3 : deep ? 5 : 0;
         if ((rc = rofk::launch_rows(x_dtype != ROF_F32, a, phase, vec, off32, 0, st))) return rc;
@@ -495,7 +544,7 @@ static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64
         a.ldo = ldo;
         a.n_wave = L->db.n_wave;
         a.n_tasks = L->db.n_tasks;
-        a.xcd_run = g_xcd_run_b > 0 ? g_xcd_run_b : L->xcd_run;
+        a.xcd_run = L->tune_xcd_run_dst > 0 ? L->tune_xcd_run_dst : L->xcd_run;
         a.out_bf16 = out_dtype == ROF_BF16;
         a.vec_store = ((uintptr_t)out) % 4 == 0;   // pieces of a row are stored whole wherever they start on a dword
         a.bias = bias;
@@ -509,7 +558,8 @@ static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64
         const int phase = ((int64_t)L->n * feat * (a.out_bf16 ? 2 : 4) >= kStreamOutBytes && a.vec_store && vec > 1 &&
                            (!a.out_bf16 || ldo % 2 == 0)) ? 2 : deep ? 4 : 1;
         a.n_tasks = L->db.n_regular;   // the clustered destinations at the end of the list have a launch of their own
-        a.wave_cap = dst_wave_cap(L, (int64_t)L->n * ldx * esz, (int64_t)feat * esz, ldx * esz);
+        a.wave_cap = L->tune_wave_cap >= 0 ? L->tune_wave_cap
+                                           : dst_wave_cap(L, (int64_t)L->n * ldx * esz, (int64_t)feat * esz, ldx * esz);
         if ((rc = rofk::launch_rows(x_dtype != ROF_F32, a, phase, vec, off32, 0, st))) return rc;
         a.wave_cap = 0;
         if (L->db.lg_blocks > 0) {

@@ -23,11 +23,6 @@
 
 namespace rofk {
 
-// process-wide launch tuning of the benchmark interface (rof_set_xcd_run, rof_set_lds_pad in rof_bench.h);
-// defined in agg_kernels.hip
-extern int g_xcd_run_a, g_xcd_run_b;
-extern int g_lds_pad;   // bytes of unused LDS requested per workgroup: caps the workgroups resident per CU
-
 struct AggArgs {
     const void *x;         // feature rows
     int64_t ldx;
@@ -45,6 +40,7 @@ struct AggArgs {
     int32_t n_blocks;          // logical workgroups
     int32_t xcd_run;           // consecutive logical workgroups kept on one XCD
     int32_t wave_cap;          // host side only: at most this many wavefronts per SIMD (0: as many as fit)
+    int32_t lds_pad;           // host side only: bytes of unused LDS requested per workgroup (benchmark tuning)
     int32_t vec_store;         // output rows start on 4-byte boundaries: whole-vector stores
     const float *bias;         // destination-row launch only: added to every output row (null: none)
     int32_t relu;              // destination-row launch only: clamp the output at zero
@@ -556,6 +552,18 @@ inline int rof_lanes_per_row(int feat, int vec) {
     return 64;
 }
 
+// Dynamic LDS one workgroup of a launch asks for: the rows of the workgroup-local groups of a cluster launch
+// (`lds_rows` rows of lpr * vec columns plus 4 floats of padding; none: 0 bytes) on top of the benchmark interface's
+// padding.  A cap on the wavefronts per SIMD (= workgroups of 4 wavefronts per CU) of an ordinary launch is put into
+// effect by asking for so much unused LDS that no more workgroups fit into the CU's 160 KB.
+constexpr int64_t kMaxLdsRequest = 64 * 1024;
+inline int64_t lds_request(bool cluster, int lpr, int vec, int lds_rows, int wave_cap, int lds_pad) {
+    int64_t lds = (int64_t)lds_pad + (cluster ? (int64_t)lds_rows * (lpr * vec + 4) * 4 : 0);
+    if (!cluster && wave_cap >= 2 && wave_cap < 8)
+        lds = std::max<int64_t>(lds, (kLdsPerCu / (wave_cap + 1) + 2048) / 2048 * 2048);
+    return lds;
+}
+
 // CLUSTER: a.n_blocks clusters (one workgroup each) that need `lds_rows` LDS rows; otherwise the tasks [0, n_tasks)
 // of `a`, the first n_wave of them long.
 template <typename XT, int VEC, int PHASE, bool OFF32, bool CLUSTER>
@@ -568,13 +576,8 @@ int launch_lpr(const AggArgs &a0, int lpr, int lds_rows, hipStream_t st) {
         a.n_blocks = (int32_t)((waves + kWavesPerBlock - 1) / kWavesPerBlock);
     }
     if (a.n_blocks == 0) return ROF_OK;
-    // LDS rows of the workgroup-local groups (none: 0 bytes) on top of the benchmark interface's padding.  A cap
-    // on the wavefronts per SIMD (= workgroups of 4 wavefronts per CU) is put into effect by asking for so much
-    // unused LDS that no more workgroups fit into the CU's 160 KB.
-    int64_t lds = (int64_t)g_lds_pad + (CLUSTER ? (int64_t)lds_rows * (lpr * VEC + 4) * 4 : 0);
-    if (!CLUSTER && a.wave_cap >= 2 && a.wave_cap < 8)
-        lds = std::max<int64_t>(lds, (kLdsPerCu / (a.wave_cap + 1) + 2048) / 2048 * 2048);
-    if (lds > 64 * 1024) return ROF_ERR_UNSUPPORTED;
+    const int64_t lds = lds_request(CLUSTER, lpr, VEC, lds_rows, a.wave_cap, a.lds_pad);
+    if (lds > kMaxLdsRequest) return ROF_ERR_UNSUPPORTED;   // (aggregate_impl checks every launch before the first one)
     const int64_t span = (int64_t)kXcds * a.xcd_run;
     const int64_t grid = (a.n_blocks + span - 1) / span * span;
     dim3 gr((unsigned)grid), bl(64 * kWavesPerBlock);

@@ -121,7 +121,6 @@ struct TaskList {   // tasks in natural order, before sorting
 struct Clusters {
     ivec tasks;                       // destination tasks of the cluster section, cluster by cluster
     ivec task_first{0};               // per cluster: its range in `tasks`
-    int32_t cut = 0;                  // rows up to this many entries counted as short when the clusters were formed
     ivec lg_ptr{0}, lg_task_ptr{0}, lg_col;   // per workgroup: its local groups; per local group: its sources
     int32_t max_rows = 0;
     // destination -> (group, LDS row) pairs served from LDS
@@ -135,49 +134,55 @@ int32_t short_cut(const int64_t T, const int64_t over, int32_t groups) {
 }
 
 // Long tasks first (descending), then the short tasks tile by tile, each tile descending, and last the tasks of
-// `placed` in their given order (the clustered short tasks, may be null).  `groups`: short tasks that share a
-// wavefront.  With `band` (one key per task: the highest source id it gathers) both kinds are ordered by descending
-// key instead.
-void order_tasks(const ivec &ptr, int64_t tile_rows, int32_t groups, const ivec *band, const ivec *placed, int32_t fixed_cut,
+// `placed` in their given order (the clustered short tasks, may be null; they run in a launch of their own, one lane
+// group each whatever their length, so the cut between long and short tasks is taken from the other tasks alone).
+// `groups`: short tasks that share a wavefront.  With `band` (one key per task: the highest source id it gathers)
+// both kinds are ordered by descending key instead.
+void order_tasks(const ivec &ptr, int64_t tile_rows, int32_t groups, const ivec *band, const ivec *placed,
                  ivec &order, int32_t &n_wave) {
     int64_t T = (int64_t)ptr.size() - 1;
     order.clear();
     order.reserve(T);
-    int64_t over = 0;
-    for (int64_t t = 0; t < T; ++t) over += ptr[t + 1] - ptr[t] > kShortRow;
-    // (`placed` tasks were chosen as short ones against `fixed_cut`, which then has to be the cut used here)
-    const int32_t cut = fixed_cut > 0 ? fixed_cut : short_cut(T, over, groups);
+    std::vector<char> taken;
+    if (placed && !placed->empty()) {
+        taken.assign(T, 0);
+        for (int32_t t : *placed) taken[t] = 1;
+    }
+    auto free_task = [&taken](int64_t t) { return taken.empty() || !taken[t]; };
+    int64_t over = 0, mine = 0;
+    for (int64_t t = 0; t < T; ++t)
+        if (free_task(t)) {
+            ++mine;
+            over += ptr[t + 1] - ptr[t] > kShortRow;
+        }
+    const int32_t cut = short_cut(mine, over, groups);
     ivec longs;
     for (int64_t t = 0; t < T; ++t)
-        if (ptr[t + 1] - ptr[t] > cut) longs.push_back((int32_t)t);
+        if (free_task(t) && ptr[t + 1] - ptr[t] > cut) longs.push_back((int32_t)t);
     if (band && cut == kShortRow) {   // a launch too small to fill the machine keeps the longest-first order
         ivec shorts;
         for (int64_t t = 0; t < T; ++t)
-            if (ptr[t + 1] - ptr[t] <= cut) shorts.push_back((int32_t)t);
+            if (free_task(t) && ptr[t + 1] - ptr[t] <= cut) shorts.push_back((int32_t)t);
         auto higher = [band](int32_t x, int32_t y) { return (*band)[x] > (*band)[y]; };
         std::stable_sort(longs.begin(), longs.end(), higher);
         std::stable_sort(shorts.begin(), shorts.end(), higher);
         n_wave = (int32_t)longs.size();
         order = longs;
         order.insert(order.end(), shorts.begin(), shorts.end());
+        if (placed) order.insert(order.end(), placed->begin(), placed->end());
         return;
     }
     std::stable_sort(longs.begin(), longs.end(),
                      [&ptr](int32_t x, int32_t y) { return ptr[x + 1] - ptr[x] > ptr[y + 1] - ptr[y]; });
     n_wave = (int32_t)longs.size();
     order = longs;
-    std::vector<char> taken;
-    if (placed && !placed->empty()) {
-        taken.assign(T, 0);
-        for (int32_t t : *placed) taken[t] = 1;
-    }
     std::vector<ivec> bucket(cut + 1);
     for (int64_t t0 = 0; t0 < T; t0 += tile_rows) {
         int64_t t1 = std::min(T, t0 + tile_rows);
         for (auto &b : bucket) b.clear();
         for (int64_t t = t0; t < t1; ++t) {
             int32_t len = ptr[t + 1] - ptr[t];
-            if (len <= cut && (taken.empty() || !taken[t])) bucket[len].push_back((int32_t)t);
+            if (len <= cut && free_task(t)) bucket[len].push_back((int32_t)t);
         }
         for (int32_t len = cut; len >= 0; --len) order.insert(order.end(), bucket[len].begin(), bucket[len].end());
     }
@@ -195,8 +200,7 @@ void finalize_phase(const TaskList &tl, int64_t tile_rows, int32_t groups, bool 
             band[t] = first < tl.ptr[t + 1] ? tl.col[first] : -1;
         }
     }
-    order_tasks(tl.ptr, tile_rows, groups, by_band ? &band : nullptr, cl ? &cl->tasks : nullptr,
-                (cl && !cl->tasks.empty()) ? cl->cut : 0, order, ph.n_wave);
+    order_tasks(tl.ptr, tile_rows, groups, by_band ? &band : nullptr, cl ? &cl->tasks : nullptr, order, ph.n_wave);
     ph.n_tasks = (int32_t)T;
     ph.n_regular = ph.n_tasks;
     if (cl && !cl->tasks.empty()) {
@@ -387,6 +391,7 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     const int32_t segment = (o && o->segment > 0) ? o->segment : default_segment(hub_split, groups, o ? o->elem_bytes : 4);
     L->hub_split = hub_split;
     L->segment = segment;
+    if (o && (o->share_scope < 0 || o->share_scope > 1)) return ROF_ERR_ARG;
     const bool disable = o && o->disable_reuse;
     const int32_t min_consumers = o ? o->min_consumers : 0;
     const int32_t entry_order = o ? o->entry_order : 0;
@@ -409,10 +414,12 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     Clusters cl;
     cl.of_node.assign(n, -1);
     const int32_t local_groups = o ? o->local_groups : 0;
+    const int32_t share_scope = o ? o->share_scope : 0;
     ivec served(G, 0);   // consumers of each group that read it from LDS
-    if (!disable && min_consumers == 0 && local_groups >= 0 && G > 0) {
-        ivec full_len(n);
-        int64_t over = 0;
+    ivec full_len;       // entries of every destination with every group expanded
+    int64_t over = 0;    // destinations whose task, as cut by hub_split, is a long one
+    if (G > 0) {
+        full_len.resize(n);
         for (int32_t v = 0; v < n; ++v) {
             int64_t len = L->res_ptr[v + 1] - L->res_ptr[v];
             for (int32_t j = ng_ptr[v]; j < ng_ptr[v + 1]; ++j) len += L->group_ptr[ng[j] + 1] - L->group_ptr[ng[j]];
@@ -420,14 +427,18 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
             const int64_t task_len = len > hub_split ? (len + segment - 1) / segment : len;
             over += task_len > kShortRow;
         }
+    }
+    // share_scope 1: only rows that will be cut into segments read shared groups from the workspace
+    auto in_scope = [&](int32_t v) { return share_scope != 1 || full_len[v] > hub_split; };
+    if (!disable && min_consumers == 0 && local_groups >= 0 && G > 0) {
         // sharing only shortens rows, so a row that is short now stays short, and rows above the segment cut are
         // no candidates
         const int32_t cut = short_cut(n, over, groups);
-        cl.cut = cut;
-        // LDS rows per workgroup: 16 KB at the width this layout is built for, at most 32 rows (a kernel that is
-        // launched at a greater width than that still stays within the 64 KB a workgroup may ask for)
+        // LDS rows per workgroup: 16 KB at the width this layout is built for, at most 31 rows: the widest row any
+        // launch can ask for is that of bf16 features at 64 lanes, (64 * 8 + 4) * 4 = 2064 bytes, and 31 of those
+        // still fit the 64 KB a workgroup may request (32 would not)
         const int32_t row_bytes = lpr * 16 * ((o && o->elem_bytes == 2) ? 2 : 1);
-        const int32_t max_rows = std::max(4, std::min(32, (16 << 10) / row_bytes));
+        const int32_t max_rows = std::max(4, std::min(31, (16 << 10) / row_bytes));
         build_clusters(L, ng_ptr, ng, full_len, std::min(cut, hub_split), groups, max_rows, local_groups > 0 ? local_groups : kMinClusterSaving,
                        local_groups == 0, cl);
         for (int32_t v = 0; v < n; ++v)
@@ -452,10 +463,19 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
         if (min_consumers > 0) return cnt >= min_consumers;
         return (cnt - 1) * len > cnt + 1;
     };
+    // consumers of each group that would read it from the workspace
+    ivec scoped(G, 0);
+    for (int64_t g = 0; g < G; ++g) {
+        if (share_scope != 1) {
+            scoped[g] = L->group_dst_ptr[g + 1] - L->group_dst_ptr[g] - served[g];
+            continue;
+        }
+        for (int32_t j = L->group_dst_ptr[g]; j < L->group_dst_ptr[g + 1]; ++j) scoped[g] += in_scope(L->group_dst[j]);
+    }
     // a plan whose sharing would not repay its extra launch is executed with every group folded back
     int64_t saved = 0;
     for (int64_t g = 0; g < G; ++g) {
-        int64_t cnt = L->group_dst_ptr[g + 1] - L->group_dst_ptr[g] - served[g], len = L->group_ptr[g + 1] - L->group_ptr[g];
+        int64_t cnt = scoped[g], len = L->group_ptr[g + 1] - L->group_ptr[g];
         if (worth(cnt, len)) saved += (cnt - 1) * len - cnt;
     }
     const bool too_small = min_consumers == 0 && (saved * lpr * 16 < kMinSavedBytes ||   // a lane holds 16 bytes of a row
@@ -465,7 +485,7 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     TaskList tg, ts, tb;
     for (int64_t g = 0; g < G; ++g) {
         if (too_small) break;
-        if (!worth(L->group_dst_ptr[g + 1] - L->group_dst_ptr[g] - served[g], L->group_ptr[g + 1] - L->group_ptr[g])) continue;
+        if (!worth(scoped[g], L->group_ptr[g + 1] - L->group_ptr[g])) continue;
         slot_of[g] = (int32_t)slots++;
         tg.begin_task(slot_of[g]);
         tg.col.insert(tg.col.end(), L->group_col.begin() + L->group_ptr[g], L->group_col.begin() + L->group_ptr[g + 1]);
@@ -489,14 +509,15 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
                 row.push_back(cl.row[j]);
                 ++nlds;
             }
+        const bool reads_workspace = ng_ptr[v + 1] > ng_ptr[v] && in_scope(v);
         for (int32_t j = ng_ptr[v]; j < ng_ptr[v + 1]; ++j)
-            if (local_row[ng[j]] < 0 && slot_of[ng[j]] >= 0) {
+            if (local_row[ng[j]] < 0 && slot_of[ng[j]] >= 0 && reads_workspace) {
                 row.push_back(n + slot_of[ng[j]]);
                 ++refs;
             }
         for (int32_t j = ng_ptr[v]; j < ng_ptr[v + 1]; ++j) {
             int32_t g = ng[j];
-            if (local_row[g] < 0 && slot_of[g] < 0)
+            if (local_row[g] < 0 && (slot_of[g] < 0 || !reads_workspace))
                 row.insert(row.end(), L->group_col.begin() + L->group_ptr[g], L->group_col.begin() + L->group_ptr[g + 1]);
         }
         if (nlds)
@@ -786,6 +807,15 @@ int rof_layout_export(const rof_layout *L, rof_bag **out) {
         return ROF_ERR_ALLOC;
     }
     *out = bag;
+    return ROF_OK;
+}
+
+int rof_layout_stats_n(const rof_layout *L, int64_t *stats, int count) {
+    if (!L || !stats || count < 0) return ROF_ERR_ARG;
+    int64_t s[20];
+    int rc = rof_layout_stats(L, s);
+    if (rc) return rc;
+    for (int i = 0; i < count; ++i) stats[i] = i < 20 ? s[i] : 0;
     return ROF_OK;
 }
 

@@ -59,10 +59,11 @@ def lanes_per_row(feat_dim, bf16=False):
 
 
 ENTRY_ORDERS = {"descending": 0, "plan": 1, "ascending": 2}
+SHARE_SCOPES = {"all": 0, "long_rows": 1}
 
 
 def _opts(min_consumers=0, disable_reuse=False, hub_split=0, segment=0, lanes_per_row=0, entry_order="descending",
-          tile_rows=0, elem_bytes=0, local_groups=0):
+          tile_rows=0, elem_bytes=0, local_groups=0, share_scope="all"):
     o = LayoutOpts()
     o.min_consumers = int(min_consumers)
     o.disable_reuse = int(bool(disable_reuse))
@@ -73,6 +74,7 @@ def _opts(min_consumers=0, disable_reuse=False, hub_split=0, segment=0, lanes_pe
     o.tile_rows = int(tile_rows)
     o.elem_bytes = int(elem_bytes)
     o.local_groups = int(local_groups)
+    o.share_scope = SHARE_SCOPES[share_scope]
     return o
 
 
@@ -173,6 +175,19 @@ class Layout:
         s = (C.c_int64 * 20)()
         check(_lib.lib().rof_layout_stats(self._h, s))
         return {k: int(s[i]) for i, k in enumerate(STAT_NAMES)}
+
+    def set_tuning(self, xcd_run_partial=0, xcd_run_dst=0, wave_cap=-1, lds_pad=0):
+        """Launch tuning of this layout (rof_layout_set_tuning in include/rof_bench.h); the defaults are the
+        library's own choices."""
+        t = _lib.LaunchTuning(int(xcd_run_partial), int(xcd_run_dst), int(wave_cap), int(lds_pad))
+        check(_lib.lib().rof_layout_set_tuning(self._h, C.byref(t)))
+        return self
+
+    def tuning(self):
+        t = _lib.LaunchTuning()
+        check(_lib.lib().rof_layout_get_tuning(self._h, C.byref(t)))
+        return {"xcd_run_partial": t.xcd_run_partial, "xcd_run_dst": t.xcd_run_dst, "wave_cap": t.wave_cap,
+                "lds_pad": t.lds_pad}
 
     def algorithmic_bytes(self, feat_dim, in_bytes=4):
         """Bytes one aggregation must move at least once per use, as counted for the roofline:

@@ -138,6 +138,12 @@ def build_input_info(indptr, indices, part_size=3, device="cuda", warps_per_bloc
     return info
 
 
+def _layout_arg(layout):
+    """The prebuilt layout of a plan container as a keyword argument, when there is one: upstream's signature has no
+    such argument, and an operator module without it (the compiled one) re-lays the plan tensors out itself."""
+    return {} if layout is None else {"layout": layout}
+
+
 class ROF_GCNConvFunc(torch.autograd.Function):
     """reuse_conv.py:30-92: dispatch on kernel_type, same plan forward and backward, five gradients."""
 
@@ -165,7 +171,7 @@ class ROF_GCNConvFunc(torch.autograd.Function):
         if kernel_type == "ROF_v2":
             return ROF.reuse_forward_v2(x, weight, ii.uniqpart_column_index, ii.degrees, ii.uniqpart_pointers,
                                         ii.part2Node_ptr, ii.part2Node_col, ii.partSize, ii.dimWorker,
-                                        ii.warpPerBlock, layout=ctx.layout)[0]
+                                        ii.warpPerBlock, **_layout_arg(ctx.layout))[0]
         raise NotImplementedError
 
     @staticmethod
@@ -185,7 +191,7 @@ class ROF_GCNConvFunc(torch.autograd.Function):
         elif ctx.kernel_type == "ROF_v2":
             d_input, d_weight = ROF.reuse_backward_v2(grad_output, x, weight, uniqpart_column_index, degrees,
                                                       uniqpart_pointers, part2Node_ptr, part2Node_col, ps, dw, wpb,
-                                                      layout=ctx.layout)
+                                                      **_layout_arg(ctx.layout))
         else:
             raise NotImplementedError
         return d_input, d_weight, None, None, None

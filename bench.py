@@ -234,7 +234,7 @@ def build_layouts(d, n, ps, lpr, in_bytes, args, want_forced=True):
 
     v2 = (d["uniqpart_column_index"], d["uniqpart_pointers"], d["part2Node_ptr"], d["part2Node_col"], n, ps)
     common = dict(hub_split=args.hub_split, segment=args.segment, lanes_per_row=lpr, entry_order=args.entry_order,
-                  tile_rows=args.tile_rows, elem_bytes=in_bytes)
+                  tile_rows=args.tile_rows, elem_bytes=in_bytes, share_scope=args.share_scope)
     reuse = Layout.from_v2(*v2, min_consumers=args.min_consumers, **common)
     plain = Layout.from_v2(*v2, disable_reuse=True, **common)
     # when the cost model folds every group back (the plan saves too little), also time the plan with its
@@ -263,6 +263,13 @@ def make_features(name, n, feat, bf16, dev):
     return x, x32, ld
 
 
+def apply_tuning(lay, args):
+    """Launch tuning from the command line (all defaults: the library's own choices)."""
+    if lay is not None and (args.xcd_run or args.xcd_run_partial or args.lds_pad > 0 or args.wave_cap >= 0):
+        lay.set_tuning(xcd_run_partial=args.xcd_run_partial, xcd_run_dst=args.xcd_run, wave_cap=args.wave_cap,
+                       lds_pad=max(0, args.lds_pad))
+
+
 def traffic_child(args):
     """Body of a counter run (this script under `rocprofv3 --pmc ...`): the default layout of the workload, one
     calibration copy of COPY_BYTES and a few aggregations, nothing else on the GPU."""
@@ -281,6 +288,7 @@ def traffic_child(args):
     d, _, _ = load_or_build(name, ps, args.cache_dir)
     n = len(d["indptr"]) - 1
     reuse, _, _ = build_layouts(d, n, ps, lanes_per_row(feat, bf16), 2 if bf16 else 4, args, want_forced=False)
+    apply_tuning(reuse, args)
     reuse.upload()
     if normalized:
         reuse.set_degrees(torch.from_numpy(np.diff(d["indptr"]).astype(np.float32)).to(dev))
@@ -317,6 +325,29 @@ def read_counter_csv(path):
     return {k: v / CHILD_AGGREGATIONS for k, v in acc.items()}, copy
 
 
+def run_group(cmd, cwd, env, limit_s):
+    """Run `cmd` as the leader of a process group of its own and return (exit status, output).  On a time-out the
+    whole group is killed -- the profiler and the Python process it started -- so that no GPU holder outlives us."""
+    import signal
+
+    p = subprocess.Popen(cmd, cwd=cwd, env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, start_new_session=True)
+    try:
+        out, _ = p.communicate(timeout=limit_s)
+        return p.returncode, out.decode(errors="replace")
+    except subprocess.TimeoutExpired:
+        try:
+            os.killpg(p.pid, signal.SIGKILL)
+        except ProcessLookupError:
+            pass
+        out, _ = p.communicate()
+        return -9, out.decode(errors="replace") + f"\n[killed after {limit_s} s]"
+    finally:
+        try:   # whatever happened: nothing of the group is left behind
+            os.killpg(p.pid, signal.SIGKILL)
+        except (ProcessLookupError, PermissionError):
+            pass
+
+
 def measure_traffic(args, passthrough):
     """HBM-side bytes per launch from rocprofv3 counter runs of this script (one counter set per run, as the
     hardware collects them), started as child processes *before* this process initialises the GPU.
@@ -333,14 +364,13 @@ def measure_traffic(args, passthrough):
     try:
         for tag, counters in (("fetch", ["FETCH_SIZE"]), ("write", ["WRITE_SIZE"]), ("tcc", ["TCC_HIT_sum", "TCC_MISS_sum"])):
             out_dir = os.path.join(tmp, tag)
-            cmd = ["timeout", "-s", "KILL", "240", prof, "--pmc", *counters, "-d", out_dir, "-o", "rof", "-f", "csv",
+            cmd = [prof, "--pmc", *counters, "-d", out_dir, "-o", "rof", "-f", "csv",
                    "--", sys.executable, os.path.abspath(__file__), "--traffic-child", *passthrough]
-            log(f"[bench] counter run: {' '.join(cmd[4:])}")
-            r = subprocess.run(cmd, cwd="/tmp", env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, timeout=300)
+            log(f"[bench] counter run: {' '.join(cmd)}")
+            rc, text = run_group(cmd, "/tmp", env, 240)
             files = glob.glob(os.path.join(out_dir, "**", "*counter_collection.csv"), recursive=True)
-            if r.returncode != 0 or not files:
-                return {"error": f"rocprofv3 --pmc {' '.join(counters)} failed (rc {r.returncode}): "
-                                 + r.stdout.decode(errors="replace")[-300:]}
+            if rc != 0 or not files:
+                return {"error": f"rocprofv3 --pmc {' '.join(counters)} failed (rc {rc}): " + text[-300:]}
             rows_per_phase, copy_values = read_counter_csv(files[0])
             copy.update(copy_values)
             per.update(rows_per_phase)
@@ -366,6 +396,50 @@ def measure_traffic(args, passthrough):
                                 "tcc_hit_rate": hit / (hit + miss) if hit is not None and miss else None,
                                 "tcc_miss_x_128B": miss * 128.0 if miss is not None else None}
     return res
+
+
+def read_calibration(L, dev):
+    """What plain streaming reaches on this device, as yardsticks for the gather launches' fetch rate: reads of a
+    buffer far beyond the caches (2 GiB: HBM), reads of a buffer that the 256 MB Infinity Cache holds but the L2s do
+    not (128 MiB, read repeatedly), and a 1 GiB device-to-device copy (read + write).  GB/s, HIP events on the
+    current stream, best of three."""
+    import ctypes
+
+    import torch
+
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    sink = torch.zeros(1, dtype=torch.float32, device=dev)
+    big = torch.empty((2 << 30) // 4, dtype=torch.float32, device=dev).normal_()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+    def rate(fn, nbytes, reps):
+        best = 0.0
+        for _ in range(3):
+            e0.record()
+            for _ in range(reps):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            best = max(best, nbytes * reps / (e0.elapsed_time(e1) * 1e-3) / 1e9)
+        return best
+
+    def read(buf, nbytes):
+        return lambda: _check_rc(L.rof_device_read(ctypes.c_void_p(buf.data_ptr()), nbytes, ctypes.c_void_p(sink.data_ptr()), st))
+
+    res = {"hbm_stream_read_GBs": rate(read(big, 2 << 30), 2 << 30, 4),
+           "infinity_cache_read_GBs": rate(read(big, 128 << 20), 128 << 20, 64)}
+    half = big[: (1 << 30) // 4]
+    other = big[(1 << 30) // 4:]
+    res["copy_read_plus_write_GBs"] = rate(lambda: _check_rc(L.rof_device_copy(
+        ctypes.c_void_p(other.data_ptr()), ctypes.c_void_p(half.data_ptr()), 1 << 30, st)), 2 << 30, 4)
+    del big, half, other
+    return res
+
+
+def _check_rc(rc):
+    from artifact_amd import _lib
+
+    _lib.check(rc)
 
 
 def restrided(t):
@@ -425,13 +499,17 @@ def main():
     ap.add_argument("--quick", action="store_true", help="only the headline timing: no counters, sweep, model step or CPU leg")
     ap.add_argument("--traffic-child", action="store_true", help=argparse.SUPPRESS)
     ap.add_argument("--xcd-run", type=int, default=0, help="launch tuning: workgroups per XCD run, destination rows")
-    ap.add_argument("--xcd-run-partial", type=int, default=1, help="same for the partial-sum launches")
+    ap.add_argument("--xcd-run-partial", type=int, default=0, help="same for the partial-sum launches")
+    ap.add_argument("--wave-cap", type=int, default=-1,
+                    help="launch tuning: wavefronts per SIMD of the destination-row launch (0 = all, 2..7; -1 = the library's rule)")
     ap.add_argument("--padded-output", action="store_true",
                     help="store the output in rows of the input's stride (47 floats in rows of 48, rof_epilogue."
                          "pad_columns) instead of the packed [N, feat] tensor the operator API returns")
     ap.add_argument("--hub-split", type=int, default=0, help="layout tuning: rows longer than this are segmented")
     ap.add_argument("--segment", type=int, default=0, help="layout tuning: entries per segment")
     ap.add_argument("--min-consumers", type=int, default=0, help="layout tuning: share groups with >= this many consumers")
+    ap.add_argument("--share-scope", default="all", choices=["all", "long_rows"],
+                    help="layout tuning: which consumers read shared groups from the workspace")
     ap.add_argument("--lds-pad", type=int, default=-1, help="launch tuning: unused LDS bytes per workgroup")
     ap.add_argument("--entry-order", default="descending", choices=["descending", "plan", "ascending"],
                     help="layout tuning: order of the gathered rows inside a task")
@@ -455,7 +533,7 @@ def main():
     normalized = name != "c3"
     bf16 = name == "c5"
     default_opts = (not (args.hub_split or args.segment or args.tile_rows or args.xcd_run
-                         or args.xcd_run_partial != 1 or args.lds_pad >= 0)
+                         or args.xcd_run_partial or args.lds_pad >= 0 or args.wave_cap >= 0 or args.share_scope != "all")
                     and args.search == "upstream" and args.entry_order == "descending")
 
     # ---- host side first: graph and plan (cached on disk), then the counter runs in child processes; this
@@ -483,10 +561,6 @@ def main():
     L = _lib.lib()   # raises if the HIP library is missing
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
-    if args.xcd_run or args.xcd_run_partial != 1:
-        _lib.check(L.rof_set_xcd_run(args.xcd_run_partial, args.xcd_run))
-    if args.lds_pad >= 0:
-        _lib.check(L.rof_set_lds_pad(args.lds_pad))
     dev = torch.device("cuda:0")
 
     indptr, indices = d["indptr"], d["indices"]
@@ -514,6 +588,7 @@ def main():
             f"candidates")
     deg = torch.from_numpy(np.diff(indptr).astype(np.float32)).to(dev)
 
+    calibration = None if args.quick else read_calibration(L, dev)
     x, x32, ld = make_features(name, n, feat, bf16, dev)
     in_bytes = 2 if bf16 else 4
     lpr = lanes_per_row(feat, bf16)
@@ -521,6 +596,7 @@ def main():
     reuse, plain, forced = build_layouts(d, n, ps, lpr, in_bytes, args)
     t_layout = time.time() - t0
     for lay in (reuse, plain) + ((forced,) if forced else ()):
+        apply_tuning(lay, args)
         lay.upload()
         if normalized:
             lay.set_degrees(deg)
@@ -732,7 +808,13 @@ def main():
         tb = t["bytes"] if t and ms > 0 else None
         return {
             "bound": "hbm", "kernel": label,
-            # achieved / frac: HBM-side bytes the launch really moved (profiler counters) over its duration
+            # What `traffic` counts: the fills and write-backs of the L2s (FETCH_SIZE / WRITE_SIZE), i.e. everything
+            # that crosses from the XCDs to the memory side.  The 256 MB Infinity Cache sits behind those counters, so
+            # a part of it never reaches HBM: `frac` is an upper bound of the HBM fraction, and only for a feature
+            # matrix several times that cache (the 2^22-node bf16 workload) is it close to one.
+            "traffic_kind": "L2 fills + write-backs (served by HBM and by the Infinity Cache behind the counters)",
+            "achievable_read_GBs": calibration,
+            # achieved / frac: memory-side bytes the launch really moved (profiler counters) over its duration
             "achieved": tb / (ms * 1e-3) / 1e9 if tb else None, "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": tb / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS if tb else None,
             "traffic": tb, "traffic_read": t["read_bytes"] if t else None, "traffic_written": t["written_bytes"] if t else None,

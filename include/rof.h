@@ -3,8 +3,7 @@
  * Every entry point is extern "C", takes plain pointers and sizes, returns 0 or a negative
  * rof_status, never throws and never exits the process.  State lives in the handles it returns;
  * the only process-wide state is the static device scratch of rof_aggregate_noalloc (one copy per
- * GPU) and the launch-tuning settings of the benchmark interface in rof_bench.h, which are not meant
- * to be changed while other threads launch.  Host-side functions are safe to call concurrently on
+ * GPU).  Host-side functions are safe to call concurrently on
  * different handles; device-side functions enqueue on the hipStream_t they are given and do not
  * synchronise.
  *
@@ -34,7 +33,13 @@ typedef enum {
 
 const char *rof_strerror(int status);
 const char *rof_last_device_error(void); /* thread-local text of the last HIP failure */
-int rof_version(void);   /* 2: rof_layout_opts has local_groups, rof_layout_stats fills 20 counters */
+/* Version of this interface.  A caller compiled against another value of ROF_ABI_VERSION than rof_version() returns
+ * must not pass structs or fixed-size arrays to the library: 2 grew rof_layout_opts from 32 to 48 bytes and the array
+ * of rof_layout_stats from 16 to 20 counters; 3 added rof_layout_stats_n (which takes the caller's count, so later
+ * counters no longer change a signature) and moved the launch tuning of rof_bench.h from process-wide settings into
+ * the layout.  Structs keep reserved fields so that they can gain members without growing. */
+#define ROF_ABI_VERSION 3
+int rof_version(void);
 
 /* ------------------------------------------------------------------------------------------
  * Host side 1: the reuse-plan builder.  Stays on the CPU (OpenMP); every array is bit-exact
@@ -146,7 +151,12 @@ typedef struct {
                              /* same groups are placed in one workgroup, which sums those groups once into LDS;      */
                              /* 0 = on: a cluster must save 8 row gathers and an eighth of its rows' gathers, and all  */
                              /* clusters together 64 MB of gathers; k > 0 = every cluster that saves k; -1 = off      */
-    int32_t reserved[3];
+    int32_t share_scope;     /* which consumers read a shared group from the workspace: 0 = every consumer; 1 = only rows   */
+                             /* long enough to be cut into segments (more than hub_split entries with every group           */
+                             /* expanded): their partial-row reads happen in the swept launch, whose working set is small,   */
+                             /* while every other consumer gets the group's sources folded back into its row.  The tests of  */
+                             /* min_consumers / the cost model then count the consumers in scope only.                      */
+    int32_t reserved[2];
 } rof_layout_opts;
 
 /* v2 tensors: replaces the plan arguments of reuse_forward_v2 / reuse_backward_v2
@@ -185,6 +195,8 @@ int rof_layout_export(const rof_layout *layout, rof_bag **out);
  * per workgroup that sums it) [17] reads of them [18] workgroups that hold clustered destinations [19] LDS rows the
  * destination-row launch asks for per workgroup. */
 int rof_layout_stats(const rof_layout *layout, int64_t stats[20]);
+/* The first `count` of those counters (fewer than the library knows: the rest is dropped; more: zero-filled). */
+int rof_layout_stats_n(const rof_layout *layout, int64_t *stats, int count);
 
 /* Copy the schedule to the current HIP device (idempotent). */
 int rof_layout_upload(rof_layout *layout, void *stream);

@@ -1,8 +1,7 @@
 /* rof_bench.h -- benchmark and tuning interface of librof.so: timing helpers that bracket the aggregation with
- * HIP events on the launch stream, a plain copy kernel for calibrating profiler byte counters, and two process-wide
- * launch-tuning settings.  None of it has a counterpart in upstream and none of it is needed to use the library
- * (rof.h); bench.py and the tuning sweeps use it.  The two settings are plain globals read by every launch: set
- * them before launching from other threads, not while.
+ * HIP events on the launch stream, plain copy and read kernels for calibrating profiler byte counters, and the
+ * launch-tuning settings of a layout.  None of it has a counterpart in upstream and none of it is needed to use the
+ * library (rof.h); bench.py and the tuning sweeps use it.
  */
 #ifndef ROF_BENCH_H_
 #define ROF_BENCH_H_
@@ -31,16 +30,35 @@ int rof_aggregate_launch_times(const rof_layout *layout, const void *x, int x_dt
  * No upstream counterpart. */
 int rof_device_copy(void *dst, const void *src, size_t nbytes, void *stream);
 
-/* Launch tuning: how many consecutive workgroups of the partial-sum launches / of the destination-row launch
- * stay on one XCD (each XCD has its own L2, so runs of neighbouring destination rows share gathered rows
- * there).  run_launch2 = 0 (the default) lets every layout use its own choice: one tile of destinations per
- * run when at least half of the neighbours lie within 8192 ids of their row (block-structured graphs), 4
- * workgroups otherwise.  Process-wide; no upstream counterpart. */
-int rof_set_xcd_run(int run_launch1, int run_launch2);
+/* Plain streaming read of nbytes (a multiple of 16, pointer 16-byte aligned) of device memory; `sink` is one float
+ * of device memory that is practically never written.  Timed over a buffer far larger than the caches it gives the
+ * read rate the memory system sustains on this device, the yardstick for the gather launches' fetch rate.
+ * No upstream counterpart. */
+int rof_device_read(const void *src, size_t nbytes, float *sink, void *stream);
 
-/* Launch tuning: request `bytes` (0..65536) of unused LDS per workgroup, which caps how many workgroups
- * share a CU (160 KB LDS each) and with it the number of row gathers in flight.  Process-wide. */
-int rof_set_lds_pad(int bytes);
+/* Launch tuning of one layout.  Every field has a "library decides" value, which is what a new layout holds; the
+ * settings belong to the layout (no process-wide state) and are read by every aggregation that uses it, so change
+ * them only while no other thread launches with the same layout.  No upstream counterpart.
+ *   xcd_run_partial / xcd_run_dst: how many consecutive workgroups of the partial-sum launches / of the
+ *     destination-row launch stay on one XCD (each XCD has its own L2, so runs of neighbouring destination rows
+ *     share gathered rows there).  0 = the library's choice: 1 for the partial-sum launches; for the destination
+ *     rows one tile of destinations per run when at least half of the neighbours lie within 8192 ids of their row
+ *     (block-structured graphs), 4 workgroups otherwise.
+ *   wave_cap: wavefronts per SIMD of the destination-row launch, 2..7; 0 = as many as fit; -1 = the library's
+ *     choice from the size of the feature matrix, the row bytes and the row stride.
+ *   lds_pad: bytes (0..65536) of unused LDS requested per workgroup in every launch, which caps how many
+ *     workgroups share a CU and with it the number of row gathers in flight. */
+typedef struct {
+    int32_t xcd_run_partial;
+    int32_t xcd_run_dst;
+    int32_t wave_cap;
+    int32_t lds_pad;
+    int32_t reserved[4];
+} rof_launch_tuning;
+
+int rof_layout_set_tuning(rof_layout *layout, const rof_launch_tuning *tuning);
+/* The settings as stored (the "library decides" values are returned as such). */
+int rof_layout_get_tuning(const rof_layout *layout, rof_launch_tuning *tuning);
 
 #ifdef __cplusplus
 }

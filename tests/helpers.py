@@ -46,6 +46,22 @@ def close_fp32(got, want64, mag=None, rtol=1e-5, atol=1e-6, extra=None, what="")
     assert not bad.any(), f"{what}: {int(bad.sum())} elements off, max err {err.max():.3e}"
 
 
+def strict_excess(got, want64, rtol=1e-5, atol=1e-6):
+    """(elements beyond the strict bar atol + rtol*|want|, largest error as a multiple of that bar)."""
+    err = np.abs(np.asarray(got, dtype=np.float64) - np.asarray(want64, dtype=np.float64))
+    strict = atol + rtol * np.abs(np.asarray(want64, dtype=np.float64))
+    return int((err > strict).sum()), float((err / strict).max()) if err.size else 0.0
+
+
+def summation_error(got, want64, mag):
+    """Largest error in units of the sum of the absolute values of the terms (the quantity that bounds the
+    re-association error of an fp32 sum: about sqrt(terms) * 2^-24 for a sequential sum of random terms)."""
+    err = np.abs(np.asarray(got, dtype=np.float64) - np.asarray(want64, dtype=np.float64))
+    mag = np.asarray(mag, dtype=np.float64)
+    ok = mag > 0
+    return float((err[ok] / mag[ok]).max()) if ok.any() else 0.0
+
+
 def toy_csr():
     indptr = np.zeros(11, dtype=np.int32)
     idx = []
@@ -196,3 +212,112 @@ def check_plan_invariants(ipd, isrc, ps, plan, discard=True):
     for p in np.nonzero(flag)[0]:
         k = flag[p] - 1
         assert np.array_equal(new[pp[p]:pp[p + 1]], cc[cp[k]:cp[k + 1]])
+
+
+# ---- the randomised schedule cases of tests/test_gpu_random_schedules.py (the GPU test runs them; the CPU suite
+# measures on the same inputs how far fp32 arithmetic in upstream's own order is from float64)
+LANES = [0, 4, 8, 10, 12, 16, 20, 32, 64]
+
+
+def random_csr(rng, n, ps):
+    """Rows of 0..40 neighbours, a few hubs of up to n, and rows made of one to three of a few shared
+    neighbour sets of `ps` ids each (each set inside its own id range, so the sets stay whole when a row is cut
+    into parts and the plan builder finds parts to share); columns sorted and unique per row."""
+    kind = rng.random(n)
+    deg = np.where(kind < 0.15, 0, rng.integers(1, 41, n))
+    hubs = rng.choice(n, max(1, n // 200), replace=False)
+    deg[hubs] = rng.integers(n // 4, n + 1, len(hubs))
+    kind[hubs] = 0.5
+    sets = max(1, min(n // (2 * ps), n // 50 + 1))
+    width = n // sets
+    shared = [j * width + np.sort(rng.choice(width, ps, replace=False)) for j in range(sets)]
+    rows = []
+    for v in range(n):
+        if kind[v] > 0.6:
+            rows.append(np.concatenate([shared[j] for j in np.sort(rng.choice(sets, min(sets, int(rng.integers(1, 4))),
+                                                                              replace=False))]))
+            continue
+        rows.append(np.unique(rng.choice(n, min(int(deg[v]), n), replace=False)))
+    ip = np.r_[0, np.cumsum([len(r) for r in rows])].astype(np.int32)
+    ix = (np.concatenate(rows) if ip[-1] else np.zeros(0)).astype(np.int32)
+    return ip, ix
+
+
+def bf16_round(a):
+    """float32 -> nearest-even bfloat16 -> float32 (the rounding torch's .to(bfloat16) performs on finite values)."""
+    u = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
+    return ((u + 0x7fff + ((u >> 16) & 1)) & np.uint32(0xffff0000)).astype(np.uint32).view(np.float32)
+
+
+
+
+def random_schedule_case(seed):
+    """Inputs and options of one randomised case (graph, schedule options, width, stride, types, epilogue)."""
+    rng = np.random.default_rng(seed)
+    n = int(rng.integers(12, 3000))
+    ps = int(rng.integers(2, 6))
+    ip, ix = random_csr(rng, n, ps)
+    opts = dict(hub_split=int(rng.choice([0, 8, 33, 100])), segment=int(rng.choice([0, 1, 5, 16])),
+                lanes_per_row=int(rng.choice(LANES)), entry_order=str(rng.choice(["descending", "plan", "ascending"])),
+                tile_rows=int(rng.choice([0, 64])), elem_bytes=int(rng.choice([0, 2, 4])),
+                local_groups=int(rng.choice([0, 0, 1, 30, -1])))
+    if seed % 3 == 2:        # (chosen from the seed, not drawn: the cases keep the inputs they always had)
+        opts["share_scope"] = "long_rows"
+    use_plan = rng.random() < 0.6
+    min_consumers = int(rng.choice([0, 2, 3])) if use_plan else 0
+    feat = int(rng.choice([1, 2, 3, 5, 8, 17, 32, 47, 64, 100, 129, 256, 300]))
+    ld = feat + int(rng.choice([0, 0, 1, 3, 8]))
+    bf16_in, bf16_out = rng.random() < 0.35, rng.random() < 0.3
+    normalized = rng.random() < 0.6
+    bias = rng.standard_normal(feat).astype(np.float32) if rng.random() < 0.5 else None
+    relu = rng.random() < 0.5
+    self_weight = float(rng.choice([0.0, 0.0, 0.7, -1.25]))
+    pad = bool(rng.random() < 0.4)                         # rows taken as whole vectors where the stride allows it
+    x = rng.standard_normal((n, feat)).astype(np.float32)
+    if bf16_in:
+        x = bf16_round(x)
+    deg = rng.integers(1, 50, n).astype(np.float32)        # the degrees are an input of their own (cu:254)
+    return dict(n=n, ps=ps, ip=ip, ix=ix, opts=opts, use_plan=use_plan, min_consumers=min_consumers, feat=feat, ld=ld,
+                bf16_in=bf16_in, bf16_out=bf16_out, normalized=normalized, bias=bias, relu=relu,
+                self_weight=self_weight, pad=pad, x=x, deg=deg)
+
+
+def closed_form_case(oracle, c):
+    """float64 closed form of one randomised case and the sum of the absolute values of its terms:
+    out[v] = relu( rs(deg v) * sum_u rs(deg u) x[u]  +  self_weight * x[v]  +  bias )."""
+    n, ip, ix, feat = c["n"], c["ip"], c["ix"], c["feat"]
+    rs = oracle.rsqrt_rn(c["deg"]).astype(np.float64) if c["normalized"] else np.ones(n)
+    x64 = c["x"].astype(np.float64)
+    rows = np.repeat(np.arange(n), np.diff(ip))
+    want, mag = np.zeros((n, feat)), np.zeros((n, feat))
+    np.add.at(want, rows, x64[ix] * rs[ix, None])
+    np.add.at(mag, rows, np.abs(x64[ix]) * rs[ix, None])
+    want, mag = want * rs[:, None], mag * rs[:, None]
+    want, mag = want + c["self_weight"] * x64, mag + abs(c["self_weight"]) * np.abs(x64)
+    if c["bias"] is not None:
+        want, mag = want + c["bias"], mag + np.abs(c["bias"])
+    if c["relu"]:
+        want = np.maximum(want, 0.0)
+    return want, mag
+
+
+def reference_order_fp32(oracle, c):
+    """The layer of one randomised case in fp32, summed the way the upstream GNNA kernel sums it: every row in
+    parts of `ps` neighbours in CSR order (oracle/agg_oracle.c, reuse_conv_kernel.cu:205-286), then the epilogue in
+    the order the library applies it (own row, bias, ReLU), each step rounded to fp32."""
+    n, ps, ip, ix = c["n"], c["ps"], c["ip"], c["ix"]
+    part_ptr, part2node = [0], []
+    for v in range(n):
+        for q in range(ip[v], ip[v + 1], ps):
+            part_ptr.append(min(q + ps, ip[v + 1]))
+            part2node.append(v)
+    agg = oracle.agg_parts(c["x"], c["deg"], ix, np.asarray(part_ptr, dtype=np.int32),
+                           np.asarray(part2node, dtype=np.int32), normalized=c["normalized"])
+    r = agg.astype(np.float64)
+    if c["self_weight"] != 0.0:
+        r = (np.float32(c["self_weight"]).astype(np.float64) * c["x"].astype(np.float64) + r).astype(np.float32).astype(np.float64)
+    if c["bias"] is not None:
+        r = (r + c["bias"].astype(np.float64)).astype(np.float32).astype(np.float64)
+    if c["relu"]:
+        r = np.maximum(r, 0.0)
+    return r

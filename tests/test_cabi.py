@@ -45,8 +45,8 @@ def test_no_torch_types_in_signatures():
 
 def test_benchmark_entry_points_are_not_in_the_product_header():
     text = open(os.path.join(ROOT, "include", "rof.h")).read()
-    for name in ("rof_aggregate_timed", "rof_aggregate_launch_times", "rof_device_copy", "rof_set_xcd_run",
-                 "rof_set_lds_pad"):
+    for name in ("rof_aggregate_timed", "rof_aggregate_launch_times", "rof_device_copy", "rof_device_read",
+                 "rof_layout_set_tuning", "rof_layout_get_tuning"):
         assert name not in text
 
 
@@ -63,8 +63,9 @@ def test_error_codes_and_messages():
     assert L.rof_aggregate(None, None, 0, 0, None, 0, 1, 1, None, 0, None) == -1
     assert L.rof_aggregate_noalloc(None, None, 0, 0, None, 0, 1, 1, None, None) == -1
     assert L.rof_layout_workspace_bytes(None, 4) == 0
-    assert L.rof_set_xcd_run(0, 1) == -1
-    assert L.rof_set_xcd_run(1, 0) == 0                      # 0 for the destination-row launch: per-layout choice
+    assert L.rof_layout_set_tuning(None, None) == -1 and L.rof_layout_get_tuning(None, None) == -1
+    assert L.rof_layout_stats_n(None, None, 4) == -1
+    assert L.rof_version() == 3
     ep = _lib.Epilogue(None, 1, 0, 0.5)
     assert L.rof_aggregate_epilogue(None, None, 0, 0, None, 0, 1, 1, C.byref(ep), None, 0, None) == -1
     assert L.rof_column_sums(None, 0, 4, 10, 4, None, None, 0, None) == -1          # no output
@@ -76,6 +77,7 @@ def test_error_codes_and_messages():
     assert L.rof_plan_hub_patterns(None, None, 0, 0, 16, 8, C.byref(h)) == -1
     assert L.rof_plan_dynamic_greedy(None, None, None, None, 0, 0, 3, C.byref(h)) == -1
     assert C.sizeof(_lib.Epilogue) == 32 and C.sizeof(_lib.LayoutOpts) == 48         # the structs of include/rof.h
+    assert C.sizeof(_lib.LaunchTuning) == 32                                         # and of include/rof_bench.h
     with pytest.raises(_lib.RofError, match="invalid argument"):
         _lib.check(-1)
 

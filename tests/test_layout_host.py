@@ -186,9 +186,16 @@ def test_random_graphs_with_shared_neighbour_sets_through_clusters(oracle, seed)
     plan = R.build_plan(ip, ix, ps, t.indptr, t.indices)
     opts = dict(lanes_per_row=int(rng.choice([4, 8, 12, 16, 32, 64])), local_groups=int(rng.choice([1, 4, 8, 30])),
                 hub_split=int(rng.choice([0, 24, 100])), segment=int(rng.choice([0, 8])),
-                elem_bytes=int(rng.choice([2, 4])), entry_order=str(rng.choice(["descending", "plan", "ascending"])))
+                elem_bytes=int(rng.choice([2, 4])), entry_order=str(rng.choice(["descending", "plan", "ascending"])),
+                share_scope=str(rng.choice(["all", "long_rows"])), min_consumers=int(rng.choice([0, 0, 2])))
     lay = _v2(plan, n, ps, **opts)
     ex, st = lay.export(), lay.stats()
+    if opts["share_scope"] == "long_rows" and st["materialised_groups"]:
+        # only rows that are cut into segments may reference a shared group: the references sit in segment tasks
+        # (or in a row that sharing shortened below the cut), never in a row that was short to begin with
+        b_ref_rows = ex["b_task_out"][(ex["b_task_nref"] > 0) & (np.diff(ex["b_task_ptr"]) > ex["b_task_nref"])]
+        cut = opts["hub_split"] or {4: 640, 8: 640, 12: 640, 16: 384, 32: 128, 64: 128}[opts["lanes_per_row"]] * (2 if opts["elem_bytes"] == 2 else 1)
+        assert all(np.diff(ip)[v] > min(cut, 640) for v in b_ref_rows), opts
     x = rng.standard_normal((n, 2))
     w = rng.uniform(0.5, 2.0, n)
     got = emulate_schedule(ex, n, x, lambda c: w[c], lambda v: w[v], st["partial_rows"])
