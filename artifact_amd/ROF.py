@@ -70,8 +70,8 @@ def _layout_parts(column_index, part_pointers, part2Node, num_nodes, part_size):
 
     def build():
         host = _host(column_index, part_pointers, part2Node)
-        return LayoutFamily(lambda lpr, eb: Layout.from_parts(*host, num_nodes, part_size, lanes_per_row=lpr,
-                                                              elem_bytes=eb))
+        return LayoutFamily(lambda lpr, eb, rb=0, **kw: Layout.from_parts(*host, num_nodes, part_size, lanes_per_row=lpr,
+                                                                          elem_bytes=eb, row_bytes=rb, **kw))
 
     return _cached(key, build, (column_index, part_pointers, part2Node))
 
@@ -82,8 +82,9 @@ def _layout_v1(column_index, part_pointers, part2Node, flag, cache_ptr, cache_co
     def build():
         host = _host(column_index, part_pointers, part2Node, flag, cache_ptr, cache_col)
         # every cache row is materialised (min_consumers=-1) so that slot g of the workspace is cache row g
-        return LayoutFamily(lambda lpr, eb: Layout.from_v1(*host, num_nodes, part_size, min_consumers=-1,
-                                                           lanes_per_row=lpr, elem_bytes=eb))
+        return LayoutFamily(lambda lpr, eb, rb=0, **kw: Layout.from_v1(*host, num_nodes, part_size, min_consumers=-1,
+                                                                       lanes_per_row=lpr, elem_bytes=eb, row_bytes=rb,
+                                                                       **kw))
 
     return _cached(key, build, (column_index, part_pointers, part2Node, flag, cache_ptr, cache_col))
 
@@ -93,8 +94,8 @@ def _layout_v2(ucol, uptr, dptr, dcol, num_nodes, part_size):
 
     def build():
         host = _host(ucol, uptr, dptr, dcol)
-        return LayoutFamily(lambda lpr, eb: Layout.from_v2(*host, num_nodes, part_size, lanes_per_row=lpr,
-                                                           elem_bytes=eb))
+        return LayoutFamily(lambda lpr, eb, rb=0, **kw: Layout.from_v2(*host, num_nodes, part_size, lanes_per_row=lpr,
+                                                                       elem_bytes=eb, row_bytes=rb, **kw))
 
     return _cached(key, build, (ucol, uptr, dptr, dcol))
 

@@ -20,7 +20,7 @@ SYMBOLS = (
     "rof_transpose_csr", "rof_plan_build", "rof_layout_from_v2", "rof_layout_from_v1", "rof_layout_from_parts",
     "rof_layout_export", "rof_layout_stats", "rof_layout_upload", "rof_layout_set_degrees",
     "rof_plan_hub_patterns", "rof_plan_dynamic_greedy", "rof_column_sums", "rof_column_sums_workspace_bytes", "rof_layout_workspace_bytes", "rof_layout_free", "rof_aggregate", "rof_aggregate_epilogue", "rof_aggregate_noalloc", "rof_aggregate_timed", "rof_aggregate_launch_times",
-    "rof_device_copy", "rof_device_read", "rof_layout_set_tuning", "rof_layout_get_tuning", "rof_layout_stats_n",
+    "rof_device_copy", "rof_device_read", "rof_layout_set_tuning", "rof_layout_get_tuning", "rof_layout_stats_n", "rof_layout_calibrate",
 )
 
 
@@ -32,12 +32,12 @@ class LayoutOpts(C.Structure):
     _fields_ = [("min_consumers", C.c_int32), ("disable_reuse", C.c_int32), ("hub_split", C.c_int32),
                 ("segment", C.c_int32), ("lanes_per_row", C.c_int32), ("entry_order", C.c_int32),
                 ("tile_rows", C.c_int32), ("elem_bytes", C.c_int32), ("local_groups", C.c_int32),
-                ("share_scope", C.c_int32), ("reserved", C.c_int32 * 2)]
+                ("share_scope", C.c_int32), ("row_bytes", C.c_int32), ("reserved", C.c_int32 * 1)]
 
 
 class LaunchTuning(C.Structure):
     _fields_ = [("xcd_run_partial", C.c_int32), ("xcd_run_dst", C.c_int32), ("wave_cap", C.c_int32),
-                ("lds_pad", C.c_int32), ("reserved", C.c_int32 * 4)]
+                ("lds_pad", C.c_int32), ("deep", C.c_int32), ("reserved", C.c_int32 * 3)]
 
 
 class Epilogue(C.Structure):
@@ -89,6 +89,8 @@ def lib():
     L.rof_layout_set_tuning.argtypes = [vp, C.POINTER(LaunchTuning)]
     L.rof_layout_get_tuning.argtypes = [vp, C.POINTER(LaunchTuning)]
     L.rof_layout_stats_n.argtypes = [vp, vp, ci]
+    L.rof_layout_calibrate.argtypes = [vp, vp, ci, i64, vp, i64, ci, ci, C.POINTER(Epilogue), vp, C.c_size_t, vp, ci, ci,
+                                       C.POINTER(LaunchTuning)]
     L.rof_device_read.argtypes = [vp, C.c_size_t, vp, vp]
     L.rof_column_sums_workspace_bytes.argtypes = [i64, ci]
     L.rof_column_sums_workspace_bytes.restype = C.c_size_t

@@ -328,10 +328,12 @@ int rof_layout_set_tuning(rof_layout *L, const rof_launch_tuning *t) {
     if (t->xcd_run_partial < 0 || t->xcd_run_dst < 0 || t->xcd_run_partial > 4096 || t->xcd_run_dst > 4096) return ROF_ERR_ARG;
     if (t->wave_cap < -1 || t->wave_cap == 1 || t->wave_cap > 7) return ROF_ERR_ARG;
     if (t->lds_pad < 0 || t->lds_pad > 64 * 1024) return ROF_ERR_ARG;
+    if (t->deep < -1 || t->deep > 1) return ROF_ERR_ARG;
     L->tune_xcd_run_partial = t->xcd_run_partial;
     L->tune_xcd_run_dst = t->xcd_run_dst;
     L->tune_wave_cap = t->wave_cap;
     L->tune_lds_pad = t->lds_pad;
+    L->tune_deep = t->deep;
     return ROF_OK;
 }
 
@@ -342,6 +344,7 @@ int rof_layout_get_tuning(const rof_layout *L, rof_launch_tuning *t) {
     t->xcd_run_dst = L->tune_xcd_run_dst;
     t->wave_cap = L->tune_wave_cap;
     t->lds_pad = L->tune_lds_pad;
+    t->deep = L->tune_deep;
     return ROF_OK;
 }
 
@@ -395,6 +398,9 @@ int rof_layout_upload(rof_layout *L, void *stream) {
     if (L->uploaded) return ROF_OK;
     hipStream_t st = (hipStream_t)stream;
     HIP_TRY(hipGetDevice(&L->device));
+    int lds_per_cu = 0;   // what an occupancy cap by LDS request has to be measured against
+    if (hipDeviceGetAttribute(&lds_per_cu, hipDeviceAttributeMaxSharedMemoryPerMultiprocessor, L->device) == hipSuccess)
+        L->lds_per_cu = lds_per_cu;
     int rc;
     if ((rc = upload_phase(L->g, L->dg, false, st, &L->device_bytes)) ||
         (rc = upload_phase(L->s, L->ds, false, st, &L->device_bytes)) ||
@@ -491,9 +497,9 @@ static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64
         const int lpr = rofk::rof_lanes_per_row(feat, vec);
         const int cap = L->tune_wave_cap >= 0 ? L->tune_wave_cap
                                               : dst_wave_cap(L, (int64_t)L->n * ldx * esz, (int64_t)feat * esz, ldx * esz);
-        const int64_t plain_lds = rofk::lds_request(false, lpr, vec, 0, cap, L->tune_lds_pad);
+        const int64_t plain_lds = rofk::lds_request(false, lpr, vec, 0, cap, L->tune_lds_pad, L->lds_per_cu);
         const int64_t cluster_lds = L->db.lg_blocks > 0
-                                        ? rofk::lds_request(true, lpr, vec, L->db.lg_max_rows, 0, L->tune_lds_pad) : 0;
+                                        ? rofk::lds_request(true, lpr, vec, L->db.lg_max_rows, 0, L->tune_lds_pad, L->lds_per_cu) : 0;
         if (plain_lds > rofk::kMaxLdsRequest || cluster_lds > rofk::kMaxLdsRequest) {
             rof_set_device_error("rof_aggregate", "the LDS rows of the layout's clusters do not fit a workgroup's 64 KB at this "
                                                   "feature width; build the layout for this width (lanes_per_row, elem_bytes)");
@@ -509,10 +515,11 @@ static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64
     a.nsplit = L->n;
     a.feat = feat;
     a.lds_pad = L->tune_lds_pad;
+    a.lds_per_cu = L->lds_per_cu;
     int rc;
     // a feature matrix that the caches serve: more row gathers in flight in every launch (fp32 rows).  2^18-node
     // R-MAT graph against two in flight: 42 MB -8 %, 67 MB -7 %, 84 MB -2.8 %, 105 MB 0, 126 MB +1.9 %.
-    const bool deep = x_dtype == ROF_F32 && (int64_t)L->n * ldx * esz < kServedMatrixBytes;
+    const bool deep = x_dtype == ROF_F32 && (L->tune_deep >= 0 ? L->tune_deep == 1 : (int64_t)L->n * ldx * esz < kServedMatrixBytes);
     // launches 1 and 2: partial-sum rows (shared groups, then segments of long rows)
     const rof_phase_dev *partial[2] = {&L->dg, &L->ds};
     for (int i = 0; i < 2 && (launches & 1); ++i) {
@@ -644,6 +651,73 @@ int rof_aggregate_timed(const rof_layout *L, const void *x, int x_dtype, int64_t
     HIP_TRY(hipEventElapsedTime(&ms, e.ev[0], e.ev[1]));
     *ms_per_call = ms / iters;
     return rc;
+}
+
+int rof_layout_calibrate(rof_layout *L, const void *x, int x_dtype, int64_t ldx, void *out, int64_t ldo, int feat,
+                         int normalized, const rof_epilogue *ep, void *workspace, size_t workspace_bytes, void *stream,
+                         int rounds, int iters, rof_launch_tuning *chosen) {
+    if (!L || rounds < 1 || iters < 1) return ROF_ERR_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    EventSet e;
+    int rc = e.create(2);
+    if (rc) return rc;
+    // one timing of the whole call under the layout's current settings; < 0: failed
+    auto timed = [&](float *ms) -> int {
+        float best = -1.f;
+        for (int r = 0; r < rounds; ++r) {
+            HIP_TRY(hipEventRecord(e.ev[0], st));
+            int status = ROF_OK;
+            for (int i = 0; i < iters && status == ROF_OK; ++i)
+                status = aggregate_with(L, x, x_dtype, ldx, out, ldo, feat, normalized, ep, workspace, workspace_bytes, st, 3);
+            HIP_TRY(hipEventRecord(e.ev[1], st));
+            HIP_TRY(hipEventSynchronize(e.ev[1]));
+            if (status != ROF_OK) return status;
+            float t = 0.f;
+            HIP_TRY(hipEventElapsedTime(&t, e.ev[0], e.ev[1]));
+            if (best < 0.f || t < best) best = t;
+        }
+        *ms = best / iters;
+        return ROF_OK;
+    };
+    const rof_launch_tuning before = {L->tune_xcd_run_partial, L->tune_xcd_run_dst, L->tune_wave_cap, L->tune_lds_pad,
+                                      L->tune_deep, {0, 0, 0}};
+    float t = 0.f;
+    if ((rc = aggregate_with(L, x, x_dtype, ldx, out, ldo, feat, normalized, ep, workspace, workspace_bytes, st, 3)) ||
+        (rc = timed(&t))) {   // warm-up, then the settings the size rules give
+        return rc;
+    }
+    float best = t;
+    // one setting after the other; a candidate replaces the incumbent only if it is measurably faster (1 %)
+    auto sweep = [&](int32_t *field, const int32_t *values, int count) -> int {
+        int32_t keep = *field;
+        for (int i = 0; i < count; ++i) {
+            if (values[i] == keep) continue;
+            *field = values[i];
+            float ms = 0.f;
+            int status = timed(&ms);
+            if (status == ROF_ERR_UNSUPPORTED) continue;   // e.g. a cap whose LDS request does not fit beside the padding
+            if (status != ROF_OK) {
+                *field = keep;
+                return status;
+            }
+            if (ms < best * 0.99f) {
+                best = ms;
+                keep = values[i];
+            }
+        }
+        *field = keep;
+        return ROF_OK;
+    };
+    const int32_t caps[] = {0, 7, 6}, deeps[] = {0, 1}, runs[] = {4, 16, L->xcd_run};
+    if ((rc = sweep(&L->tune_wave_cap, caps, 3)) || (x_dtype == ROF_F32 && (rc = sweep(&L->tune_deep, deeps, 2))) ||
+        (rc = sweep(&L->tune_xcd_run_dst, runs, 3))) {
+        L->tune_wave_cap = before.wave_cap;
+        L->tune_deep = before.deep;
+        L->tune_xcd_run_dst = before.xcd_run_dst;
+        return rc;
+    }
+    if (chosen) rof_layout_get_tuning(L, chosen);
+    return ROF_OK;
 }
 
 int rof_aggregate_launch_times(const rof_layout *L, const void *x, int x_dtype, int64_t ldx, void *out, int64_t ldo,

@@ -41,6 +41,7 @@ struct AggArgs {
     int32_t xcd_run;           // consecutive logical workgroups kept on one XCD
     int32_t wave_cap;          // host side only: at most this many wavefronts per SIMD (0: as many as fit)
     int32_t lds_pad;           // host side only: bytes of unused LDS requested per workgroup (benchmark tuning)
+    int32_t lds_per_cu;        // host side only: LDS bytes of one CU on the layout's device (queried at upload)
     int32_t vec_store;         // output rows start on 4-byte boundaries: whole-vector stores
     const float *bias;         // destination-row launch only: added to every output row (null: none)
     int32_t relu;              // destination-row launch only: clamp the output at zero
@@ -66,7 +67,7 @@ __device__ __forceinline__ uint32_t rof_bf16_bits(float f) {
 constexpr int kGathersInFlight = 2;
 constexpr int kWavesPerBlock = 4;
 constexpr int kXcds = 8;
-constexpr int64_t kLdsPerCu = 160 * 1024;
+constexpr int64_t kLdsPerCu = 160 * 1024;   // gfx950; the launch path uses what the device reports at upload
 
 template <typename XT, int VEC>
 struct RowLoad;
@@ -557,10 +558,14 @@ inline int rof_lanes_per_row(int feat, int vec) {
 // padding.  A cap on the wavefronts per SIMD (= workgroups of 4 wavefronts per CU) of an ordinary launch is put into
 // effect by asking for so much unused LDS that no more workgroups fit into the CU's 160 KB.
 constexpr int64_t kMaxLdsRequest = 64 * 1024;
-inline int64_t lds_request(bool cluster, int lpr, int vec, int lds_rows, int wave_cap, int lds_pad) {
+inline int64_t lds_request(bool cluster, int lpr, int vec, int lds_rows, int wave_cap, int lds_pad, int64_t lds_per_cu) {
     int64_t lds = (int64_t)lds_pad + (cluster ? (int64_t)lds_rows * (lpr * vec + 4) * 4 : 0);
-    if (!cluster && wave_cap >= 2 && wave_cap < 8)
-        lds = std::max<int64_t>(lds, (kLdsPerCu / (wave_cap + 1) + 2048) / 2048 * 2048);
+    // more than 1 / (cap + 1) of the CU's LDS per workgroup: cap + 1 workgroups no longer fit, cap still do
+    // (a device whose CU had so little LDS that the request would exceed a workgroup's 64 KB runs uncapped)
+    if (!cluster && wave_cap >= 2 && wave_cap < 8) {
+        const int64_t want = ((lds_per_cu > 0 ? lds_per_cu : kLdsPerCu) / (wave_cap + 1) + 2048) / 2048 * 2048;
+        if (want <= kMaxLdsRequest) lds = std::max<int64_t>(lds, want);
+    }
     return lds;
 }
 
@@ -576,7 +581,7 @@ int launch_lpr(const AggArgs &a0, int lpr, int lds_rows, hipStream_t st) {
         a.n_blocks = (int32_t)((waves + kWavesPerBlock - 1) / kWavesPerBlock);
     }
     if (a.n_blocks == 0) return ROF_OK;
-    const int64_t lds = lds_request(CLUSTER, lpr, VEC, lds_rows, a.wave_cap, a.lds_pad);
+    const int64_t lds = lds_request(CLUSTER, lpr, VEC, lds_rows, a.wave_cap, a.lds_pad, a.lds_per_cu);
     if (lds > kMaxLdsRequest) return ROF_ERR_UNSUPPORTED;   // (aggregate_impl checks every launch before the first one)
     const int64_t span = (int64_t)kXcds * a.xcd_run;
     const int64_t grid = (a.n_blocks + span - 1) / span * span;

@@ -38,23 +38,46 @@ const int64_t kWavesToFill = 2 * 8192;   // two rounds of 256 CUs x 32 wavefront
 // and the launch sweeps the matrix once from top to bottom, so a row gathered for one destination is still in
 // L2 when the next destinations need it.  The effect is large -- rotating each row's list by a random offset,
 // which keeps every task monotone but puts the tasks out of phase, costs 25 % on the 2.4 M-node workload -- and
-// it is why the cut is low: measured optima with G rows per wavefront are cut / segment = 96-128 / 32 at G = 1
-// (-12 % against a cut of 1024), 256 / 64 at G = 2 (-18 % against 8192), 640-1024 / 160 at G = 5 (-7 % against
-// 5457).  Every segment writes and re-reads one partial row (fp32, so twice a gathered row when those are bf16),
-// which is what stops finer cuts: at G = 2 the best cut is 128 / 32 for fp32 rows (-10 % against 256 / 64) and
-// 256 / 64 for bf16 rows; at G = 4 256-512; at G = 8 and 16 640-1024 (256 is 10-30 % slower there).
+// it is why the cut is low.  Every segment writes and re-reads one partial row (fp32, so twice a gathered row when
+// those are bf16), which is what stops finer cuts.  The table below is measured (MI355X, R-MAT graphs of 2^18 to
+// 2.4 M nodes and average degrees 8 to 48, cut / segment from 64 / 16 to 8192 / 2048; G = rows a wavefront gathers
+// per instruction), the figures are the cost of the neighbouring choices against the one taken:
+//   fp32, G = 1, rows of 1024 bytes or more: 128 / 32 when the caches can hold the matrix (2^18 nodes x 256 floats:
+//     256 / 64 +7 %, 1024 / 256 +15 %), else 256 / 32 (128 / 32 0 ... +7 %, 512 / 128 +7 ... +8 %);
+//   fp32, G = 1, narrower rows (160 floats): 1024 / 128 on matrices beyond the caches (128 / 32 +2 ... +34 %,
+//     512 / 64 -2 ... +4 %, 2048 / 512 +4 ... +13 %), 128 / 32 on smaller ones (1024 / 128 +11 %);
+//   fp32, G = 2 ... 3 (100 floats): 1024 / 128 beyond the caches (128 / 32 +2 ... +26 %, 256 / 64 +1 ... +5 %),
+//     128 / 32 on smaller matrices (1024 / 128 +3 %);
+//   fp32, G = 4 (64 floats): 1024 / 128 (384 / 96 0 ... +6 %, 128 / 32 +1 ... +19 %);
+//   fp32, G >= 5: 640 / 160 (1024 / 256 -2 ... +2 %, 256 / 64 +4 ... +7 %, 5457 +7 % on the 2.4 M-node workload);
+//   bf16, G <= 2 (256 columns): 256 / 48 (2^22 nodes: -18 % against 8192; segments of 32 / 40 / 48 / 56 / 64 / 96 /
+//     128 entries 8.53 / 8.49 / 8.46 / 8.57 / 8.57 / 8.92 / 9.17 ms); G = 3: 512 / 128; G >= 4 (128 columns):
+//     1280 / 320 (640 / 160 -1 ... +4 %, 2560 / 640 0 ... +4 %).
+// No rule of sizes gets every graph right (the same width wants 128 / 32 on one graph and 1024 / 128 on another),
+// which is what the timed choice between candidate layouts is for (LayoutFamily(autotune=True)).
 // (Giving long rows a whole workgroup instead -- four wavefronts combined through LDS -- was measured as well:
 // no faster than segments on any workload, so it is not built in.)
-int32_t default_cut(int32_t groups, int32_t elem_bytes) {
-    const int32_t cut = groups <= 2 ? 128 : groups == 3 ? 256 : groups == 4 ? 384 : 640;
-    return std::min(640, elem_bytes == 2 ? 2 * cut : cut);
-}
-// Segments are a quarter of the cut; 3/16 for bf16 rows of more than 256 bytes (G <= 2), whose partial rows are
-// streamed.  2^22-node R-MAT, 256 bf16 columns, cut 256: segments of 32 / 40 / 48 / 56 / 64 / 96 / 128 entries
-// 8.53 / 8.49 / 8.46 / 8.57 / 8.57 / 8.92 / 9.17 ms.  Narrower bf16 rows (128, 64 columns) and fp32 rows
-// (2^18 nodes x 256 floats: 24 / 28 / 32 / 40 entries 0.400 / 0.377 / 0.378 / 0.380 ms) stay at a quarter.
-int32_t default_segment(int32_t cut, int32_t groups, int32_t elem_bytes) {
-    return std::max(16, elem_bytes == 2 && groups <= 2 ? cut * 3 / 16 : cut / 4);
+const int64_t kCachedMatrixBytes = 256 << 20;   // the Infinity Cache
+void default_cut(int32_t groups, int32_t elem_bytes, int64_t row_bytes, int64_t matrix_bytes, int32_t &cut, int32_t &segment) {
+    if (elem_bytes == 2) {
+        cut = groups <= 2 ? 256 : groups == 3 ? 512 : 1280;
+        segment = groups <= 2 ? cut * 3 / 16 : cut / 4;
+        return;
+    }
+    const bool cached = matrix_bytes <= kCachedMatrixBytes;
+    if (groups == 1 && row_bytes >= 1024) {
+        cut = cached ? 128 : 256;
+        segment = 32;
+    } else if (groups <= 3) {
+        cut = cached ? 128 : 1024;
+        segment = cached ? 32 : 128;
+    } else if (groups == 4) {
+        cut = 1024;
+        segment = 128;
+    } else {
+        cut = 640;
+        segment = 160;
+    }
 }
 // Sharing groups costs one more launch (~4-6 us on MI355X), and on heavy-tailed graphs what it saves is cheap:
 // the sources of a popular group are themselves popular rows that sit in L2, while the partial rows that
@@ -387,8 +410,14 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     if (lpr > 64) lpr = 64;
     const int32_t groups = std::max(1, 64 / lpr);
     const int64_t total = (int64_t)L->res_col.size() + (int64_t)L->group_dst.size();
-    const int32_t hub_split = (o && o->hub_split > 0) ? o->hub_split : default_cut(groups, o ? o->elem_bytes : 4);
-    const int32_t segment = (o && o->segment > 0) ? o->segment : default_segment(hub_split, groups, o ? o->elem_bytes : 4);
+    const int32_t elem_bytes = (o && o->elem_bytes == 2) ? 2 : 4;
+    const int64_t row_bytes = (o && o->row_bytes > 0) ? o->row_bytes : (int64_t)lpr * 16;
+    int32_t rule_cut = 0, rule_segment = 0;
+    default_cut(groups, elem_bytes, row_bytes, (int64_t)n * row_bytes, rule_cut, rule_segment);
+    const int32_t hub_split = (o && o->hub_split > 0) ? o->hub_split : rule_cut;
+    // (a caller's cut with the library's segment: the rule's share of the rule's cut)
+    const int32_t segment = (o && o->segment > 0) ? o->segment
+                                                  : std::max<int32_t>(16, (int64_t)hub_split * rule_segment / rule_cut);
     L->hub_split = hub_split;
     L->segment = segment;
     if (o && (o->share_scope < 0 || o->share_scope > 1)) return ROF_ERR_ARG;
@@ -761,6 +790,7 @@ int rof_layout_export(const rof_layout *L, rof_bag **out) {
         put("res_col", L->res_col);
         bag->arr["canonical"].assign(1, L->canonical ? 1u : 0u);
         bag->arr["xcd_run"].assign(1, (uint32_t)L->xcd_run);
+        bag->arr["long_row_cut"] = {(uint32_t)L->hub_split, (uint32_t)L->segment};   // as chosen for this layout
         // v2 tensors: groups first, then every node's residual list re-chunked by part_size
         // (reuse_search_ext.h:537-636)
         const int ps = L->part_size;

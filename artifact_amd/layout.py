@@ -20,7 +20,7 @@ STAT_NAMES = ("nodes", "edges", "groups", "materialised_groups", "gathered_rows"
               "hub_segments", "tasks_a", "tasks_b", "device_bytes", "part_size", "wave_tasks_a", "wave_tasks_b",
               "canonical", "gathered_rows_a", "local_groups", "lds_reads", "cluster_workgroups", "lds_rows")
 
-EXPORT_NAMES = ("group_ptr", "group_col", "group_dst_ptr", "group_dst", "res_ptr", "res_col", "canonical", "xcd_run",
+EXPORT_NAMES = ("group_ptr", "group_col", "group_dst_ptr", "group_dst", "res_ptr", "res_col", "canonical", "xcd_run", "long_row_cut",
                 "uniqpart_column_index", "uniqpart_pointers", "part2Node_ptr", "part2Node_col",
                 "g_task_ptr", "g_task_nref", "g_task_out", "g_col", "s_task_ptr", "s_task_nref", "s_task_out", "s_col",
                 "b_task_ptr", "b_task_nref", "b_task_out", "b_col", "b_task_nlds", "b_lg_ptr", "b_lg_task_ptr", "b_lg_col", "b_lg_task_first",
@@ -63,7 +63,7 @@ SHARE_SCOPES = {"all": 0, "long_rows": 1}
 
 
 def _opts(min_consumers=0, disable_reuse=False, hub_split=0, segment=0, lanes_per_row=0, entry_order="descending",
-          tile_rows=0, elem_bytes=0, local_groups=0, share_scope="all"):
+          tile_rows=0, elem_bytes=0, local_groups=0, share_scope="all", row_bytes=0):
     o = LayoutOpts()
     o.min_consumers = int(min_consumers)
     o.disable_reuse = int(bool(disable_reuse))
@@ -75,29 +75,107 @@ def _opts(min_consumers=0, disable_reuse=False, hub_split=0, segment=0, lanes_pe
     o.elem_bytes = int(elem_bytes)
     o.local_groups = int(local_groups)
     o.share_scope = SHARE_SCOPES[share_scope]
+    o.row_bytes = int(row_bytes)
     return o
 
 
-class LayoutFamily:
-    """Layouts of one plan, one per width class (lanes per row, element size): how finely long rows are cut
-    depends on how many rows a wavefront gathers at once and on how wide a partial-sum row is against a gathered
-    one, i.e. on the feature width and type the layout will be used with."""
+# (cut, segment) candidates that an autotuned family times against the rule's choice, by element size
+CUT_CANDIDATES = {4: ((128, 32), (512, 64), (1024, 128)), 2: ((256, 48), (640, 160), (1280, 320))}
 
-    def __init__(self, build):
-        self._build = build            # callable(lanes_per_row[, elem_bytes]) -> Layout
+
+def autotune_default():
+    """Whether layout families time their candidates by default: the environment variable ROF_AUTOTUNE=1."""
+    import os
+
+    return os.environ.get("ROF_AUTOTUNE", "0") not in ("", "0", "false", "no")
+
+
+class LayoutFamily:
+    """Layouts of one plan, one per width class (lanes per row, element size, and at one row per wavefront whether a
+    row has 1024 bytes): how finely long rows are cut depends on how many rows a wavefront gathers at once and on how
+    wide a partial-sum row is against a gathered one, i.e. on the feature width and type the layout will be used with.
+
+    `build(lanes_per_row, elem_bytes, row_bytes, **overrides)` returns a Layout (builders that take only the first
+    one or two arguments are accepted; they cannot be autotuned).  With `autotune` the first use of a width class on a
+    GPU builds the rule's layout and the candidates of CUT_CANDIDATES, times one aggregation of random rows of that
+    width with each (HIP events, two rounds in turn), keeps the fastest and lets it choose its launch settings by
+    timing too (`Layout.calibrate`); `chosen[key]` records what was taken.  That costs a few layout builds and a few
+    dozen aggregations per width class, once."""
+
+    def __init__(self, build, autotune=None):
+        self._build = build
         self._by_lpr = {}
+        self.autotune = autotune_default() if autotune is None else bool(autotune)
+        self.chosen = {}
         try:
             import inspect
 
-            self._two = len(inspect.signature(build).parameters) >= 2
+            params = inspect.signature(build).parameters.values()
+            self._nargs = sum(p.kind in (p.POSITIONAL_ONLY, p.POSITIONAL_OR_KEYWORD) for p in params)
+            self._kw = any(p.kind == p.VAR_KEYWORD for p in params)
         except (TypeError, ValueError):
-            self._two = False
+            self._nargs, self._kw = 1, False
 
-    def get(self, feat_dim, bf16=False):
-        key = (lanes_per_row(feat_dim, bf16), 2 if bf16 else 4)
+    def _make(self, key, **over):
+        lpr, eb, rb = key
+        if self._nargs >= 3:
+            return self._build(lpr, eb, rb, **over)
+        return self._build(lpr, eb) if self._nargs == 2 else self._build(lpr)
+
+    def get(self, feat_dim, bf16=False, normalized=True):
+        lpr, eb = lanes_per_row(feat_dim, bf16), 2 if bf16 else 4
+        # one row per wavefront covers widths from 81 floats up: rows of 1024 bytes and more are their own class
+        rb = (1024 if feat_dim * eb >= 1024 else 512) if (lpr == 64 and eb == 4) else 0
+        key = (lpr, eb, rb)
         lay = self._by_lpr.get(key)
         if lay is None:
-            lay = self._by_lpr[key] = self._build(*key) if self._two else self._build(key[0])
+            lay = self._make(key)
+            if self.autotune and self._nargs >= 3 and self._kw:
+                lay = self._autotune(key, lay, int(feat_dim), bool(bf16), bool(normalized))
+            self._by_lpr[key] = lay
+        return lay
+
+    def _autotune(self, key, first, feat, bf16, normalized):
+        import torch
+
+        if not torch.cuda.is_available():
+            return first
+        n = first.num_nodes
+        mult = 8 if bf16 else 4
+        ld = -(-feat // mult) * mult
+        x = torch.randn((n, ld), device="cuda").to(torch.bfloat16 if bf16 else torch.float32)[:, :feat]
+        out = torch.empty((n, feat), dtype=torch.float32, device="cuda")
+        ex = first.export()
+        rule = (ex["hub_split"], ex["segment"])
+        longest = int(np.diff(ex["b_task_ptr"]).max()) if len(ex["b_task_ptr"]) > 1 else 0
+        del ex
+        cands = {rule: first}
+        if first.stats()["hub_segments"] or longest > min(c for c, _ in CUT_CANDIDATES[key[1]]):
+            for cut, seg in CUT_CANDIDATES[key[1]]:
+                if (cut, seg) not in cands:
+                    cands[(cut, seg)] = self._make(key, hub_split=cut, segment=seg)
+        if normalized:
+            deg = torch.ones(n, dtype=torch.float32, device="cuda")
+            for lay in cands.values():
+                lay.set_degrees(deg)
+        for lay in cands.values():
+            lay.aggregate(x, normalized=normalized, out=out, feat_dim=feat)
+        ms = {k: [] for k in cands}
+        for _ in range(2):
+            for k, lay in cands.items():
+                ms[k].append(lay.aggregate_timed(x, 3, normalized=normalized, out=out, feat_dim=feat)[0])
+        ms = {k: min(v) for k, v in ms.items()}
+        best = min(ms, key=ms.get)
+        if ms[best] > 0.99 * ms[rule]:      # the rule's choice unless a candidate is measurably faster
+            best = rule
+        for k, lay in cands.items():
+            if k != best:
+                lay.close()
+        lay = cands[best]
+        tuning = lay.calibrate(x, normalized=normalized, out=out, feat_dim=feat)
+        lay._deg_key = None                  # the degrees used for timing were placeholders
+        self.chosen[key] = {"cut": best[0], "segment": best[1], "rule": rule, "ms": {f"{c}/{s}": v for (c, s), v in ms.items()},
+                            "tuning": tuning}
         return lay
 
     def close(self):
@@ -167,6 +245,7 @@ class Layout:
         r = bag_take(h, EXPORT_NAMES, dtype=np.int32)
         r["canonical"] = bool(r["canonical"][0])
         r["xcd_run"] = int(r["xcd_run"][0])
+        r["hub_split"], r["segment"] = (int(v) for v in r.pop("long_row_cut"))
         r["b_shape"] = dict(zip(("n_wave", "n_regular", "lg_blocks", "lg_max_rows"),
                                 (int(v) for v in r["b_shape"])))
         return r
@@ -176,10 +255,10 @@ class Layout:
         check(_lib.lib().rof_layout_stats(self._h, s))
         return {k: int(s[i]) for i, k in enumerate(STAT_NAMES)}
 
-    def set_tuning(self, xcd_run_partial=0, xcd_run_dst=0, wave_cap=-1, lds_pad=0):
+    def set_tuning(self, xcd_run_partial=0, xcd_run_dst=0, wave_cap=-1, lds_pad=0, deep=-1):
         """Launch tuning of this layout (rof_layout_set_tuning in include/rof_bench.h); the defaults are the
         library's own choices."""
-        t = _lib.LaunchTuning(int(xcd_run_partial), int(xcd_run_dst), int(wave_cap), int(lds_pad))
+        t = _lib.LaunchTuning(int(xcd_run_partial), int(xcd_run_dst), int(wave_cap), int(lds_pad), int(deep))
         check(_lib.lib().rof_layout_set_tuning(self._h, C.byref(t)))
         return self
 
@@ -187,7 +266,7 @@ class Layout:
         t = _lib.LaunchTuning()
         check(_lib.lib().rof_layout_get_tuning(self._h, C.byref(t)))
         return {"xcd_run_partial": t.xcd_run_partial, "xcd_run_dst": t.xcd_run_dst, "wave_cap": t.wave_cap,
-                "lds_pad": t.lds_pad}
+                "lds_pad": t.lds_pad, "deep": t.deep}
 
     def algorithmic_bytes(self, feat_dim, in_bytes=4):
         """Bytes one aggregation must move at least once per use, as counted for the roofline:
@@ -344,6 +423,23 @@ class Layout:
                                              workspace.numel() * workspace.element_size(), C.c_void_p(st), int(iters),
                                              C.byref(ms)))
         return float(ms.value), out
+
+    def calibrate(self, x, normalized=True, out=None, feat_dim=None, workspace=None, pad_columns=False, rounds=3, iters=3):
+        """Choose this layout's launch settings (wavefront cap, gathers in flight, XCD run) by timing the aggregation
+        on these operands (rof_layout_calibrate); returns the settings now in force."""
+        import torch
+
+        dt, f, out, workspace = self._args(x, out, feat_dim, workspace)
+        st = torch.cuda.current_stream().cuda_stream
+        self.upload(st)
+        t = _lib.LaunchTuning()
+        check(_lib.lib().rof_layout_calibrate(self._h, C.c_void_p(x.data_ptr()), dt, x.stride(0),
+                                              C.c_void_p(out.data_ptr()), out.stride(0), f, int(bool(normalized)),
+                                              self._plain_epilogue(x, out, f, pad_columns),
+                                              C.c_void_p(workspace.data_ptr()),
+                                              workspace.numel() * workspace.element_size(), C.c_void_p(st),
+                                              int(rounds), int(iters), C.byref(t)))
+        return self.tuning()
 
     def launch_times(self, x, iters, normalized=True, out=None, feat_dim=None, workspace=None, pad_columns=False):
         """(ms of the partial-sum launch, ms of the destination-row launch), HIP-event means over `iters`."""

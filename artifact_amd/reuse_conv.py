@@ -82,8 +82,8 @@ class ROF_inputInfo:
             n, ps = len(z["row_pointers"]) - 1, int(z["partSize"])
             v2 = tuple(np.array(z[k]) for k in ("uniqpart_column_index", "uniqpart_pointers", "part2Node_ptr",
                                                  "part2Node_col"))
-            info.layouts["ROF_v2"] = LayoutFamily(lambda lpr, eb: Layout.from_v2(
-                *v2, n, ps, lanes_per_row=lpr, elem_bytes=eb, **layout_opts))
+            info.layouts["ROF_v2"] = LayoutFamily(lambda lpr, eb, rb=0, **kw: Layout.from_v2(
+                *v2, n, ps, lanes_per_row=lpr, elem_bytes=eb, row_bytes=rb, **{**layout_opts, **kw}))
         return info
 
     def __getstate__(self):
@@ -98,10 +98,12 @@ class ROF_inputInfo:
 
 
 def build_input_info(indptr, indices, part_size=3, device="cuda", warps_per_block=4, plan=None, search="upstream",
-                     hubs=16384, **layout_opts):
+                     hubs=16384, autotune=None, **layout_opts):
     """CSR (symmetric graph, in-neighbours = out-neighbours) -> ROF_inputInfo, following the glue of
     ROF_main.py:71-178: plan on the CPU, arrays cast to int32, degrees = diff(indptr) as float32.
-    `layout_opts` (min_consumers, disable_reuse, hub_split, segment) go to the device layout.
+    `layout_opts` (min_consumers, disable_reuse, hub_split, segment) go to the device layout; `autotune=True` lets
+    the layout family choose the cut of long rows and the launch settings of every width class by timing candidates
+    on the GPU at first use (LayoutFamily; None: the environment variable ROF_AUTOTUNE).
     search="hub_patterns" (not upstream) fills the v2 tensors from reuse_search_ext.hub_pattern_plan with
     `hubs` hubs in blocks of `part_size`, search="dynamic_greedy" from reuse_search_ext.dynamic_greedy_plan; the
     GNNA / v1 tensors then describe the graph without reuse."""
@@ -131,9 +133,9 @@ def build_input_info(indptr, indices, part_size=3, device="cuda", warps_per_bloc
                          t(plan["column_index_cache"]), t(plan["uniqpart_column_index"]), t(plan["uniqpart_pointers"]),
                          t(plan["part2Node_ptr"]), t(plan["part2Node_col"]))
     if torch.device(device).type == "cuda":
-        info.layouts["ROF_v2"] = LayoutFamily(lambda lpr, eb: Layout.from_v2(
+        info.layouts["ROF_v2"] = LayoutFamily(lambda lpr, eb, rb=0, **kw: Layout.from_v2(
             plan["uniqpart_column_index"], plan["uniqpart_pointers"], plan["part2Node_ptr"], plan["part2Node_col"], n,
-            part_size, lanes_per_row=lpr, elem_bytes=eb, **layout_opts))
+            part_size, lanes_per_row=lpr, elem_bytes=eb, row_bytes=rb, **{**layout_opts, **kw}), autotune=autotune)
     info.plan = plan
     return info
 

@@ -155,9 +155,9 @@ def model_step(name, d, n, ps, deg, dev, timed):
     from artifact_amd.layout import Layout, LayoutFamily
     from artifact_amd.reuse_conv import ROF_GCNConv, ROF_GINConv
 
-    fam = LayoutFamily(lambda lpr, eb: Layout.from_v2(d["uniqpart_column_index"], d["uniqpart_pointers"],
+    fam = LayoutFamily(lambda lpr, eb, rb=0, **kw: Layout.from_v2(d["uniqpart_column_index"], d["uniqpart_pointers"],
                                                       d["part2Node_ptr"], d["part2Node_col"], n, ps,
-                                                      lanes_per_row=lpr, elem_bytes=eb))
+                                                      lanes_per_row=lpr, elem_bytes=eb, row_bytes=rb, **kw))
     dummy = torch.zeros(1, dtype=torch.int32, device=dev)   # the plan tensors are not read when a layout is attached
     info = types.SimpleNamespace(degrees=deg, layouts={"ROF_v2": fam}, partSize=ps, warpPerBlock=4,
                                  **{k: dummy for k in ("column_index", "part_pointers", "part2Node",
@@ -234,7 +234,8 @@ def build_layouts(d, n, ps, lpr, in_bytes, args, want_forced=True):
 
     v2 = (d["uniqpart_column_index"], d["uniqpart_pointers"], d["part2Node_ptr"], d["part2Node_col"], n, ps)
     common = dict(hub_split=args.hub_split, segment=args.segment, lanes_per_row=lpr, entry_order=args.entry_order,
-                  tile_rows=args.tile_rows, elem_bytes=in_bytes, share_scope=args.share_scope)
+                  tile_rows=args.tile_rows, elem_bytes=in_bytes, share_scope=args.share_scope,
+                  row_bytes=args.row_bytes)
     reuse = Layout.from_v2(*v2, min_consumers=args.min_consumers, **common)
     plain = Layout.from_v2(*v2, disable_reuse=True, **common)
     # when the cost model folds every group back (the plan saves too little), also time the plan with its
@@ -245,7 +246,7 @@ def build_layouts(d, n, ps, lpr, in_bytes, args, want_forced=True):
     return reuse, plain, forced
 
 
-def make_features(name, n, feat, bf16, dev):
+def make_features(name, n, feat, bf16, dev, packed=False):
     """Feature rows as the dense update leaves them: N(0,1) fp32 (uniform(-1,1) -> bf16 for c5) in rows
     allocated up to a multiple of 4 (8) elements.  Returns (view [n, feat], fp32 host copy, row stride)."""
     import torch
@@ -253,7 +254,7 @@ def make_features(name, n, feat, bf16, dev):
     from artifact_amd.graphgen import features
 
     mult = 8 if bf16 else 4
-    ld = (feat + mult - 1) // mult * mult
+    ld = feat if packed else (feat + mult - 1) // mult * mult   # packed: rows `feat` elements apart, as a gradient arrives
     x32 = features(n, feat, seed=2000 + (int(name[1]) if name[1].isdigit() else 6), kind="uniform" if bf16 else "normal")
     xbuf = torch.zeros((n, ld), dtype=torch.bfloat16 if bf16 else torch.float32, device=dev)
     xbuf[:, :feat] = torch.from_numpy(x32).to(dev)
@@ -287,12 +288,13 @@ def traffic_child(args):
     bf16, normalized = name == "c5", name != "c3"
     d, _, _ = load_or_build(name, ps, args.cache_dir)
     n = len(d["indptr"]) - 1
+    args.row_bytes = feat * (2 if bf16 else 4)
     reuse, _, _ = build_layouts(d, n, ps, lanes_per_row(feat, bf16), 2 if bf16 else 4, args, want_forced=False)
     apply_tuning(reuse, args)
     reuse.upload()
     if normalized:
         reuse.set_degrees(torch.from_numpy(np.diff(d["indptr"]).astype(np.float32)).to(dev))
-    x, _, ld = make_features(name, n, feat, bf16, dev)
+    x, _, ld = make_features(name, n, feat, bf16, dev, args.packed_input)
     pad = args.padded_output and ld != feat
     out = torch.empty((n, ld if pad else feat), dtype=torch.float32, device=dev)[:, :feat]
     a = torch.empty(COPY_BYTES // 4, dtype=torch.float32, device=dev).normal_()
@@ -505,9 +507,15 @@ def main():
     ap.add_argument("--padded-output", action="store_true",
                     help="store the output in rows of the input's stride (47 floats in rows of 48, rof_epilogue."
                          "pad_columns) instead of the packed [N, feat] tensor the operator API returns")
+    ap.add_argument("--packed-input", action="store_true",
+                    help="gather rows that are `feat` elements apart (47 floats = 188 bytes), the way the backward pass "
+                         "meets its gradient, instead of rows in a stride that is a multiple of 16 bytes")
     ap.add_argument("--hub-split", type=int, default=0, help="layout tuning: rows longer than this are segmented")
     ap.add_argument("--segment", type=int, default=0, help="layout tuning: entries per segment")
     ap.add_argument("--min-consumers", type=int, default=0, help="layout tuning: share groups with >= this many consumers")
+    ap.add_argument("--autotune", action="store_true",
+                    help="also time the layout that LayoutFamily(autotune=True) picks (candidate cuts of long rows and "
+                         "launch settings chosen by timing) against the size rules' choice")
     ap.add_argument("--share-scope", default="all", choices=["all", "long_rows"],
                     help="layout tuning: which consumers read shared groups from the workspace")
     ap.add_argument("--lds-pad", type=int, default=-1, help="launch tuning: unused LDS bytes per workgroup")
@@ -549,6 +557,8 @@ def main():
             passthrough += ["--feat", str(args.feat)]
         if args.padded_output:
             passthrough += ["--padded-output"]
+        if args.packed_input:
+            passthrough += ["--packed-input"]
         if args.min_consumers:
             passthrough += ["--min-consumers", str(args.min_consumers)]
         traffic = measure_traffic(args, passthrough)
@@ -589,9 +599,10 @@ def main():
     deg = torch.from_numpy(np.diff(indptr).astype(np.float32)).to(dev)
 
     calibration = None if args.quick else read_calibration(L, dev)
-    x, x32, ld = make_features(name, n, feat, bf16, dev)
+    x, x32, ld = make_features(name, n, feat, bf16, dev, args.packed_input)
     in_bytes = 2 if bf16 else 4
     lpr = lanes_per_row(feat, bf16)
+    args.row_bytes = feat * in_bytes
     t0 = time.time()
     reuse, plain, forced = build_layouts(d, n, ps, lpr, in_bytes, args)
     t_layout = time.time() - t0
@@ -660,6 +671,29 @@ def main():
     max_diff = float((out - out_plain).abs().max())
 
     extra = {}
+    if args.autotune:
+        # the cut of long rows and the launch settings chosen by timing candidates (LayoutFamily(autotune=True)) against
+        # the size rules' choice, timed in turn
+        from artifact_amd.layout import LayoutFamily
+
+        v2 = (d["uniqpart_column_index"], d["uniqpart_pointers"], d["part2Node_ptr"], d["part2Node_col"], n, ps)
+        t0 = time.time()
+        fam = LayoutFamily(lambda lpr_, eb, rb=0, **kw: Layout.from_v2(*v2, lanes_per_row=lpr_, elem_bytes=eb, row_bytes=rb, **kw),
+                           autotune=True)
+        tuned = fam.get(feat, bf16, normalized)
+        t_tune = time.time() - t0
+        if normalized:
+            tuned.set_degrees(deg)
+        tuned.aggregate(x, normalized, out=out_plain, feat_dim=feat, pad_columns=pad)
+        ev_t, ev_d = [], []
+        for _ in range(4):
+            ev_t.append(tuned.aggregate_timed(x, per, normalized, out=out_plain, feat_dim=feat, pad_columns=pad)[0])
+            ev_d.append(reuse.aggregate_timed(x, per, normalized, out=out, feat_dim=feat, pad_columns=pad)[0])
+        extra["autotune"] = {"chosen": {f"{k}": v for k, v in fam.chosen.items()}, "seconds": t_tune,
+                             "event_ms": float(np.median(ev_t)), "rule_event_ms": float(np.median(ev_d)),
+                             "speedup_over_rule": float(np.median(ev_d) / np.median(ev_t)),
+                             "max_abs_diff_vs_rule": float((out - out_plain).abs().max())}
+        fam.close()
     if not args.no_sweep and not args.feat and args.search == "upstream":
         extra["part_size_sweep"] = part_size_sweep(name, (2, 3, 4, 5), {ps: d}, n, e, x, deg, normalized, feat, lpr,
                                                    in_bytes, args, out_plain)

@@ -134,9 +134,11 @@ typedef struct {
     int32_t min_consumers;   /* a group is materialised iff it has >= this many consumers; 0 = cost model; -1 = all */
     int32_t disable_reuse;   /* 1: expand every group back into its consumers' rows (the comparator)      */
     int32_t hub_split;       /* rows with more entries than this are gathered in segments one launch earlier;  */
-                             /* 0 = by the rows a wavefront gathers at once (G = 64 / lanes_per_row): 128 for   */
-                             /* G <= 2, 256 for 3, 384 for 4, 640 from 5 on; doubled for bfloat16 rows; <= 640  */
-    int32_t segment;         /* entries per segment; 0 = a quarter of hub_split                                */
+                             /* 0 = by the rows a wavefront gathers at once (G = 64 / lanes_per_row) and the    */
+                             /* row bytes: float32 rows 128 / 256 (matrix within / beyond 256 MB) at G = 1 and   */
+                             /* >= 1024 bytes; otherwise up to G = 3 128 within and 1024 beyond 256 MB; 1024 at   */
+                             /* G = 4; 640 from 5 on; bfloat16 rows 256 for G <= 2, 512 at 3, 1280 above          */
+    int32_t segment;         /* entries per segment; 0 = an eighth to a quarter of hub_split (see layout.cpp)   */
     int32_t lanes_per_row;   /* lanes one gathered row occupies in the kernel that will use this layout:   */
                              /* smallest of 4,8,10,12,16,20,32,64 >= ceil(feat_dim / 4) (fp32) or / 8      */
                              /* (bf16); 0 = 16.  Steers the default hub_split and the sharing gate.        */
@@ -156,7 +158,10 @@ typedef struct {
                              /* expanded): their partial-row reads happen in the swept launch, whose working set is small,   */
                              /* while every other consumer gets the group's sources folded back into its row.  The tests of  */
                              /* min_consumers / the cost model then count the consumers in scope only.                      */
-    int32_t reserved[2];
+    int32_t row_bytes;       /* bytes of one gathered row (feat_dim x element size) in the kernel that will use this layout; */
+                             /* 0 = unknown (taken as 16 x lanes_per_row).  Steers the default hub_split and segment: at one  */
+                             /* row per wavefront, rows of 1024 bytes or more are cut finer than narrower ones.                */
+    int32_t reserved[1];
 } rof_layout_opts;
 
 /* v2 tensors: replaces the plan arguments of reuse_forward_v2 / reuse_backward_v2
@@ -180,6 +185,7 @@ int rof_layout_from_parts(const int32_t *column_index, const int32_t *part_point
 
 /* Canonical arrays of the layout (host copies, int32 viewed as uint32):
  *   "group_ptr"[G+1] "group_col"  "group_dst_ptr"[G+1] "group_dst"  "res_ptr"[N+1] "res_col"
+ * "xcd_run"[1] and "long_row_cut"[2] (hub_split, segment) as chosen for this layout;
  * the schedule of the three launches ("g_*", "s_*", "b_*": task_ptr, task_nref, task_out, col; for the destination
  * rows also "b_task_nlds", "b_lg_ptr", "b_lg_task_ptr", "b_lg_col", "b_lg_task_first" and "b_shape" = long tasks, tasks of
  * the ordinary launch, clusters, LDS rows per cluster)

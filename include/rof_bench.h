@@ -46,6 +46,7 @@ int rof_device_read(const void *src, size_t nbytes, float *sink, void *stream);
  *     (block-structured graphs), 4 workgroups otherwise.
  *   wave_cap: wavefronts per SIMD of the destination-row launch, 2..7; 0 = as many as fit; -1 = the library's
  *     choice from the size of the feature matrix, the row bytes and the row stride.
+ *   deep: see below.
  *   lds_pad: bytes (0..65536) of unused LDS requested per workgroup in every launch, which caps how many
  *     workgroups share a CU and with it the number of row gathers in flight. */
 typedef struct {
@@ -53,10 +54,25 @@ typedef struct {
     int32_t xcd_run_dst;
     int32_t wave_cap;
     int32_t lds_pad;
-    int32_t reserved[4];
+    int32_t deep;          /* row gathers in flight per lane group: -1 = the library's choice (more of them when the */
+                           /* caches serve the whole fp32 feature matrix), 0 = two, 1 = four (five at 10 lanes per   */
+                           /* row) wherever such an instantiation exists (fp32 rows, 32-bit offsets)                 */
+    int32_t reserved[3];
 } rof_launch_tuning;
 
 int rof_layout_set_tuning(rof_layout *layout, const rof_launch_tuning *tuning);
+
+/* Choose the launch tuning of a layout by timing instead of by the size rules: runs the aggregation on the caller's
+ * operands (arguments as rof_aggregate_epilogue; `out` receives the same, correct result every time, since no setting
+ * changes a bit) with the wavefront cap of the destination-row launch at 8 / 7 / 6, with two and four row gathers in
+ * flight where both exist, and with XCD runs of 4 / 16 / one tile, one setting after the other, keeping each
+ * winner (`rounds` timings of `iters` calls per candidate, the fastest counts; HIP events on `stream`, which the call
+ * synchronises).  The winners are stored in the layout (and returned in *chosen when not NULL) and hold until
+ * rof_layout_set_tuning changes them; they were measured for this width, stride and type, so calibrate the layout
+ * with the operands it will be used with.  Costs about (8 candidates x rounds x iters) aggregations. */
+int rof_layout_calibrate(rof_layout *layout, const void *x, int x_dtype, int64_t ldx, void *out, int64_t ldo,
+                         int feat_dim, int normalized, const rof_epilogue *epilogue, void *workspace,
+                         size_t workspace_bytes, void *stream, int rounds, int iters, rof_launch_tuning *chosen);
 /* The settings as stored (the "library decides" values are returned as such). */
 int rof_layout_get_tuning(const rof_layout *layout, rof_launch_tuning *tuning);
 

@@ -473,11 +473,14 @@ def test_rows_taken_as_whole_vectors_give_the_same_columns(oracle, feat, bf16_in
 
 
 @pytest.mark.parametrize("feat,bf16,build_lanes", [(64, False, 16), (47, False, 12), (3, False, 4), (300, False, 64),
-                                                   (256, True, 32), (100, True, 16), (64, False, 64), (520, False, 4)])
+                                                   (256, True, 32), (100, True, 16), (64, False, 64), (520, False, 4),
+                                                   (520, True, 4), (512, True, 0)])
 def test_groups_summed_in_lds_by_the_workgroup_of_their_consumers(oracle, feat, bf16, build_lanes):
     """Planted reuse: destinations that share groups sit in one workgroup, which sums the groups once into LDS
     (local_groups=8: kept whatever the plan saves in total; the default needs 64 MB of saved gathers).  Widths cover one and several feature chunks per row (the LDS rows are rewritten per
-    chunk), the scalar instantiation, bf16 rows, and layouts built for another width than they are run at."""
+    chunk), the scalar instantiation, bf16 rows, and layouts built for another width than they are run at -- among them
+    the widest LDS rows there are (bf16 rows at 64 lanes: 2064 bytes each) under a layout built for narrow rows or
+    for the default width, which gets the most LDS rows per cluster (31 x 2064 bytes fit a workgroup's 64 KB)."""
     indptr, indices, plan = _case("hr", 6, 3)
     n = len(indptr) - 1
     x = features(n, feat, seed=31)
@@ -512,3 +515,81 @@ def test_groups_summed_in_lds_by_the_workgroup_of_their_consumers(oracle, feat, 
     again = torch.empty_like(fused)
     lay.aggregate_noalloc(xt, again, normalized=True, bias=bias, relu=True, self_weight=0.5)
     assert torch.equal(again, fused)
+
+
+def test_a_call_whose_launches_do_not_all_fit_is_refused_before_the_first_launch():
+    """A cluster launch whose LDS rows do not fit a workgroup's 64 KB (forced here with the benchmark interface's
+    unused-LDS setting) is refused with ROF_ERR_UNSUPPORTED before anything is enqueued: the output keeps what it
+    held, and the same layout works again once the setting is back."""
+    indptr, indices, plan = _case("hr", 6, 3)
+    n = len(indptr) - 1
+    lay = _layout(plan, n, 3, lanes_per_row=16, local_groups=8)
+    assert lay.stats()["cluster_workgroups"] > 0
+    xt = torch.from_numpy(features(n, 64, seed=1)).cuda()
+    good = lay.aggregate(xt, normalized=False)
+    out = torch.full((n, 64), float("nan"), device="cuda")
+    lay.set_tuning(lds_pad=64 * 1024)
+    with pytest.raises(RofError, match="unsupported"):
+        lay.aggregate(xt, normalized=False, out=out)
+    torch.cuda.synchronize()
+    assert torch.isnan(out).all()                            # no launch of the refused call has run
+    assert lay.tuning()["lds_pad"] == 64 * 1024
+    lay.set_tuning()
+    assert torch.equal(lay.aggregate(xt, normalized=False, out=out), good)
+    for bad in (dict(wave_cap=1), dict(wave_cap=8), dict(xcd_run_dst=-1), dict(lds_pad=-4)):
+        with pytest.raises(RofError):
+            lay.set_tuning(**bad)
+
+
+@pytest.mark.parametrize("tuning", [dict(wave_cap=0), dict(wave_cap=5), dict(xcd_run_dst=16, xcd_run_partial=4),
+                                    dict(lds_pad=8192), dict(deep=0), dict(deep=1)])
+def test_launch_tuning_of_a_layout_changes_no_bit(tuning):
+    indptr, indices, plan = _case("c4", 6, 3)
+    n = len(indptr) - 1
+    xt = torch.from_numpy(features(n, 47, seed=2)).cuda()
+    deg = torch.from_numpy(np.diff(indptr).astype(np.float32)).cuda()
+    lay = _layout(plan, n, 3, min_consumers=2, lanes_per_row=12, hub_split=64)
+    lay.set_degrees(deg)
+    want = lay.aggregate(xt, normalized=True)
+    other = _layout(plan, n, 3, min_consumers=2, lanes_per_row=12, hub_split=64)   # a second layout keeps its own settings
+    other.set_degrees(deg)
+    lay.set_tuning(**tuning)
+    assert torch.equal(lay.aggregate(xt, normalized=True), want)
+    assert other.tuning() == dict(xcd_run_partial=0, xcd_run_dst=0, wave_cap=-1, lds_pad=0, deep=-1)
+    assert torch.equal(other.aggregate(xt, normalized=True), want)
+
+
+def test_calibration_and_autotuning_choose_by_timing_and_change_no_bit(oracle):
+    """rof_layout_calibrate times the launch settings on the caller's operands and stores the winners in the layout;
+    an autotuning family also times candidate cuts of the long rows.  Whatever they pick, the sums are those of the
+    float64 closed form and the launch settings alone change no bit."""
+    from artifact_amd.layout import LayoutFamily
+
+    indptr, indices, plan = _case("c4", 5, 3)
+    n = len(indptr) - 1
+    feat = 100
+    x = features(n, feat, seed=9)
+    xt = torch.from_numpy(x).cuda()
+    deg = np.diff(indptr).astype(np.float32)
+    degt = torch.from_numpy(deg).cuda()
+    lay = _layout(plan, n, 3, lanes_per_row=32, row_bytes=400)
+    lay.set_degrees(degt)
+    want = lay.aggregate(xt, normalized=True)
+    out = torch.full((n, feat), float("nan"), device="cuda")
+    chosen = lay.calibrate(xt, normalized=True, out=out, rounds=2, iters=2)
+    assert set(chosen) == {"xcd_run_partial", "xcd_run_dst", "wave_cap", "lds_pad", "deep"} and chosen == lay.tuning()
+    assert chosen["wave_cap"] in (-1, 0, 6, 7) and chosen["deep"] in (-1, 0, 1) and chosen["lds_pad"] == 0
+    assert torch.equal(out, want) and torch.equal(lay.aggregate(xt, normalized=True), want)
+
+    v2 = (plan["uniqpart_column_index"], plan["uniqpart_pointers"], plan["part2Node_ptr"], plan["part2Node_col"], n, 3)
+    fam = LayoutFamily(lambda lpr, eb, rb=0, **kw: Layout.from_v2(*v2, lanes_per_row=lpr, elem_bytes=eb, row_bytes=rb, **kw),
+                       autotune=True)
+    tuned = fam.get(feat, False)
+    (key, rec), = fam.chosen.items()
+    assert key == (32, 4, 0) and (rec["cut"], rec["segment"]) in {tuple(rec["rule"]), (128, 32), (512, 64), (1024, 128)}
+    assert f"{rec['cut']}/{rec['segment']}" in rec["ms"] and len(rec["ms"]) >= 2
+    assert fam.get(feat, False) is tuned                          # timed once per width class
+    tuned.set_degrees(degt)                                      # (the timing ran on placeholder degrees)
+    got = tuned.aggregate(xt, normalized=True).cpu().numpy()
+    _close(got, oracle.closed_form(indptr, indices, x, deg), oracle.closed_form(indptr, indices, np.abs(x), deg))
+    fam.close()

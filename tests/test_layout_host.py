@@ -208,17 +208,19 @@ def test_random_graphs_with_shared_neighbour_sets_through_clusters(oracle, seed)
     assert st["gathered_rows"] == total - nref - st["lds_reads"] <= len(ix)
 
 
-@pytest.mark.parametrize("lanes,elem,cut,seg", [(64, 4, 128, 32), (32, 4, 128, 32), (32, 2, 256, 48), (16, 2, 640, 160),
-                                                (16, 4, 384, 96), (12, 4, 640, 160), (8, 0, 640, 160)])
-def test_long_rows_are_cut_by_width_and_their_segments_swept_by_source_id(lanes, elem, cut, seg):
-    """Default cut by the rows a wavefront gathers at once (128 up to two, 384 at four, 640 from five on; doubled
-    for bf16 rows, whose partial rows are twice as wide), segments a quarter of it (3/16 for bf16 rows of more than
-    256 bytes); the segment tasks come in the
-    order of the highest source id they gather (each task lists its sources by descending id), long tasks before
-    packed ones."""
+@pytest.mark.parametrize("lanes,elem,row,cut,seg", [(64, 4, 0, 256, 32), (64, 4, 1024, 256, 32), (64, 4, 640, 1024, 128),
+                                                    (32, 4, 0, 1024, 128), (20, 4, 0, 128, 32), (16, 4, 0, 1024, 128),
+                                                    (12, 4, 0, 640, 160), (8, 0, 0, 640, 160),
+                                                    (32, 2, 0, 256, 48), (20, 2, 0, 512, 128), (16, 2, 0, 1280, 320)])
+def test_long_rows_are_cut_by_width_and_their_segments_swept_by_source_id(lanes, elem, row, cut, seg):
+    """Default cut and segment by the rows a wavefront gathers at once, the bytes of a row and whether the caches
+    can hold the matrix (the measured table in csrc/layout.cpp; this 600 000-row matrix is beyond them at 32 lanes
+    and more); the segment tasks come in the order of the highest source id they gather (each task lists its sources
+    by descending id), long tasks before packed ones."""
     ip, ix = make_workload("c4", 2)                          # 600 000 rows: enough segments to fill the machine
     n = len(ip) - 1
-    lay = Layout.from_csr(ip, ix, lanes_per_row=lanes, elem_bytes=elem)
+    lay = Layout.from_csr(ip, ix, lanes_per_row=lanes, elem_bytes=elem, row_bytes=row)
+    assert (lay.export()["hub_split"], lay.export()["segment"]) == (cut, seg)
     ex, st = lay.export(), lay.stats()
     deg = np.diff(ip)
     assert st["hub_segments"] == int(np.ceil(deg[deg > cut] / seg).sum())
@@ -231,12 +233,40 @@ def test_long_rows_are_cut_by_width_and_their_segments_swept_by_source_id(lanes,
         assert (np.diff(s_col[s_ptr[t]:s_ptr[t + 1]]) < 0).all()
     first = s_col[s_ptr[:-1]]
     nw = st["wave_tasks_a"]
+    groups = max(1, 64 // lanes)
+    if nw + (len(s_len) - nw + groups - 1) // groups < 2 * 8192:
+        # too few segment tasks to fill the machine twice: such a launch is bound by its longest task and runs
+        # longest first, with the lower cut between wavefront-wide and packed tasks
+        assert nw == int((s_len > 32).sum()) and (np.diff(s_len[:nw]) <= 0).all()
+        return
     assert (np.diff(first[:nw]) <= 0).all() and (np.diff(first[nw:]) <= 0).all()
     assert nw == int((s_len > 64).sum()) and (s_len[:nw] > 64).all()
     # with the plan's own order inside tasks there is no sweep: segments come longest first
-    ex2 = Layout.from_csr(ip, ix, lanes_per_row=lanes, elem_bytes=elem, entry_order="plan").export()
+    ex2 = Layout.from_csr(ip, ix, lanes_per_row=lanes, elem_bytes=elem, row_bytes=row, entry_order="plan").export()
     first2 = ex2["s_col"][ex2["s_task_ptr"][:-1]]
     assert not (np.diff(first2[:nw]) <= 0).all() or nw < 2 or not (np.diff(first2[nw:]) <= 0).all()
+
+
+def test_a_cluster_never_needs_more_lds_rows_than_fit_at_the_widest_launch():
+    """A layout may be run at another width than it was built for; the widest LDS row there is (bf16 features at 64
+    lanes: (64 * 8 + 4) * 4 = 2064 bytes) times the rows of any cluster stays within the 64 KB a workgroup may ask
+    for, also for the default width, which gets the most rows."""
+    ip, ix = make_workload("hr", 6)
+    n = len(ip) - 1
+    plan = R.build_plan(ip, ix, 3)
+    for lanes, elem in ((0, 0), (4, 4), (4, 2), (16, 4), (64, 2)):
+        ex = _v2(plan, n, 3, lanes_per_row=lanes, elem_bytes=elem, local_groups=1).export()
+        assert 0 < ex["b_shape"]["lg_max_rows"] <= 31 and ex["b_shape"]["lg_max_rows"] * 2064 <= 64 * 1024
+
+
+def test_small_matrices_keep_the_fine_cut():
+    """A matrix that the 256 MB Infinity Cache can hold is cut at 128 / 32 up to three rows per wavefront (the
+    2^18-node workload at 256 floats is exactly 256 MB), whatever the row bytes."""
+    ip, ix = make_workload("c2", 0)
+    for lanes, row, want in ((64, 640, (128, 32)), (64, 1000, (128, 32)), (32, 0, (128, 32)), (20, 0, (128, 32)),
+                             (16, 0, (1024, 128)), (64, 1024, (128, 32)), (64, 2048, (256, 32))):
+        ex = Layout.from_csr(ip, ix, lanes_per_row=lanes, row_bytes=row).export()
+        assert (ex["hub_split"], ex["segment"]) == want, (lanes, row)
 
 
 def test_xcd_run_follows_the_locality_of_the_graph():
