@@ -708,9 +708,9 @@ int rof_layout_calibrate(rof_layout *L, const void *x, int x_dtype, int64_t ldx,
         *field = keep;
         return ROF_OK;
     };
-    const int32_t caps[] = {0, 7, 6}, deeps[] = {0, 1}, runs[] = {4, 16, L->xcd_run};
+    const int32_t caps[] = {0, 7, 6}, deeps[] = {0, 1}, runs[] = {4, 16, 256, L->xcd_run};
     if ((rc = sweep(&L->tune_wave_cap, caps, 3)) || (x_dtype == ROF_F32 && (rc = sweep(&L->tune_deep, deeps, 2))) ||
-        (rc = sweep(&L->tune_xcd_run_dst, runs, 3))) {
+        (rc = sweep(&L->tune_xcd_run_dst, runs, 4))) {
         L->tune_wave_cap = before.wave_cap;
         L->tune_deep = before.deep;
         L->tune_xcd_run_dst = before.xcd_run_dst;

@@ -65,11 +65,11 @@ int rof_layout_set_tuning(rof_layout *layout, const rof_launch_tuning *tuning);
 /* Choose the launch tuning of a layout by timing instead of by the size rules: runs the aggregation on the caller's
  * operands (arguments as rof_aggregate_epilogue; `out` receives the same, correct result every time, since no setting
  * changes a bit) with the wavefront cap of the destination-row launch at 8 / 7 / 6, with two and four row gathers in
- * flight where both exist, and with XCD runs of 4 / 16 / one tile, one setting after the other, keeping each
+ * flight where both exist, and with XCD runs of 4 / 16 / 256 / one tile, one setting after the other, keeping each
  * winner (`rounds` timings of `iters` calls per candidate, the fastest counts; HIP events on `stream`, which the call
  * synchronises).  The winners are stored in the layout (and returned in *chosen when not NULL) and hold until
  * rof_layout_set_tuning changes them; they were measured for this width, stride and type, so calibrate the layout
- * with the operands it will be used with.  Costs about (8 candidates x rounds x iters) aggregations. */
+ * with the operands it will be used with.  Costs about (9 candidates x rounds x iters) aggregations. */
 int rof_layout_calibrate(rof_layout *layout, const void *x, int x_dtype, int64_t ldx, void *out, int64_t ldo,
                          int feat_dim, int normalized, const rof_epilogue *epilogue, void *workspace,
                          size_t workspace_bytes, void *stream, int rounds, int iters, rof_launch_tuning *chosen);
