@@ -16,11 +16,17 @@ from helpers import close_fp32                             # noqa: E402
 
 
 @pytest.fixture(scope="module")
-def big():
+def big_plan():
     ip, ix = make_workload("c4")
     plan = R.build_plan(ip, ix, 3)
     n = len(ip) - 1
-    args = (plan["uniqpart_column_index"], plan["uniqpart_pointers"], plan["part2Node_ptr"], plan["part2Node_col"], n, 3)
+    return ip, ix, n, (plan["uniqpart_column_index"], plan["uniqpart_pointers"], plan["part2Node_ptr"],
+                       plan["part2Node_col"], n, 3)
+
+
+@pytest.fixture(scope="module")
+def big(big_plan):
+    ip, ix, n, args = big_plan
     return ip, ix, n, Layout.from_v2(*args, min_consumers=3), Layout.from_v2(*args, disable_reuse=True)
 
 
@@ -111,3 +117,32 @@ def test_full_size_hub_pattern_plan(big):
     lay.set_degrees(degt)
     plain.set_degrees(degt)
     assert torch.allclose(lay.aggregate(x, feat_dim=47), plain.aggregate(x, feat_dim=47), rtol=1e-5, atol=2e-6)
+
+
+def test_full_size_default_and_long_rows_scope(big, big_plan):
+    """The layouts a caller gets without options (the cost model folds this plan: the schedule of the reuse-disabled
+    layout, built for the width it runs at) and with sharing restricted to the long rows, at full size: exact integer
+    sums, and the normalised layer against the reuse-disabled layout."""
+    from artifact_amd.layout import lanes_per_row
+
+    ip, ix, n, reuse, plain = big
+    dev = "cuda"
+    args = big_plan[3]
+    opts = dict(lanes_per_row=lanes_per_row(47), row_bytes=188)
+    default = Layout.from_v2(*args, **opts)
+    scoped = Layout.from_v2(*args, min_consumers=3, share_scope="long_rows", **opts)
+    st = scoped.stats()
+    assert default.stats()["materialised_groups"] == 0 and 0 < st["materialised_groups"] < reuse.stats()["materialised_groups"]
+    deg = np.diff(ip).astype(np.float32)
+    degt = torch.from_numpy(deg).to(dev)
+    g = torch.Generator(device=dev).manual_seed(11)
+    x = torch.randn((n, 48), device=dev, generator=g)[:, :47]
+    plain.set_degrees(degt)
+    want = plain.aggregate(x, feat_dim=47).clone()
+    ones = torch.ones((n, 4), device=dev)
+    for lay in (default, scoped):
+        assert np.array_equal(lay.aggregate(ones, normalized=False).cpu().numpy(), np.repeat(deg[:, None], 4, axis=1))
+        lay.set_degrees(degt)
+        got = lay.aggregate(x, feat_dim=47)
+        assert torch.allclose(got, want, rtol=1e-5, atol=2e-6)
+        lay.close()
