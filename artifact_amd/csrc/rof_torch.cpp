@@ -63,17 +63,21 @@ struct Plan {
     int64_t nodes = 0;
     std::vector<torch::Tensor> host;   // the plan tensors on the host (int32, contiguous)
     std::vector<torch::Tensor> keep;   // the device tensors whose addresses are the cache key
-    std::map<int, std::unique_ptr<Layout>> by_lanes;
+    std::map<int, std::unique_ptr<Layout>> by_lanes;   // by width class: 2 * lanes per row + (rows of >= 1024 bytes)
 
     Layout &get(int64_t feat) {
         const int lpr = lanes_per_row(feat);
-        std::unique_ptr<Layout> &slot = by_lanes[lpr];
+        // one row per wavefront covers every width from 81 floats up: rows of 1024 bytes and more are a class of
+        // their own (they are cut finer), like in the Python layer's LayoutFamily
+        const int row_bytes = lpr == 64 ? (feat * 4 >= 1024 ? 1024 : 512) : 0;
+        std::unique_ptr<Layout> &slot = by_lanes[lpr * 2 + (row_bytes == 1024)];
         if (slot) return *slot;
         slot.reset(new Layout);
         rof_layout_opts o;
         memset(&o, 0, sizeof(o));
         o.lanes_per_row = lpr;
         o.elem_bytes = 4;
+        o.row_bytes = row_bytes;
         auto p = [this](size_t i) { return host[i].numel() ? host[i].data_ptr<int32_t>() : nullptr; };
         int rc;
         if (kind == 0) {
@@ -88,9 +92,11 @@ struct Plan {
             rc = rof_layout_from_v2(p(0), host[1].data_ptr<int32_t>(), host[2].data_ptr<int32_t>(), p(3),
                                     host[1].numel() - 1, (int32_t)nodes, part_size, &o, &slot->h);
         }
-        if (rc != ROF_OK) by_lanes.erase(lpr);
-        rof_check(rc, "re-laying out the plan");
-        return *slot;
+        if (rc != ROF_OK) {
+            by_lanes.erase(lpr * 2 + (row_bytes == 1024));
+            rof_check(rc, "re-laying out the plan");
+        }
+        return *by_lanes[lpr * 2 + (row_bytes == 1024)];
     }
 };
 

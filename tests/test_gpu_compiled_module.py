@@ -40,7 +40,7 @@ def _call(kind, ii, *lead):
                    ii.partSize, dw, wpb)
 
 
-@pytest.mark.parametrize("fout", [47, 32, 3])
+@pytest.mark.parametrize("fout", [47, 32, 3, 100, 300])
 def test_forward_of_all_three_kernel_types(oracle, ROF, fout):
     ip, ix, n, info, x, w = _setup(fout=fout)
     xt, wt = torch.from_numpy(x).to(DEV), torch.from_numpy(w).to(DEV)
