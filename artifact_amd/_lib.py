@@ -91,7 +91,7 @@ def lib():
     L.rof_layout_stats_n.argtypes = [vp, vp, ci]
     L.rof_layout_calibrate.argtypes = [vp, vp, ci, i64, vp, i64, ci, ci, C.POINTER(Epilogue), vp, C.c_size_t, vp, ci, ci,
                                        C.POINTER(LaunchTuning)]
-    L.rof_device_read.argtypes = [vp, C.c_size_t, vp, vp]
+    L.rof_device_read.argtypes = [vp, C.c_size_t, ci, vp, vp]
     L.rof_column_sums_workspace_bytes.argtypes = [i64, ci]
     L.rof_column_sums_workspace_bytes.restype = C.c_size_t
     L.rof_column_sums.argtypes = [vp, ci, i64, i64, ci, vp, vp, C.c_size_t, vp]

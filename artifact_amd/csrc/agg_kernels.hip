@@ -114,14 +114,17 @@ __global__ void rof_copy_kernel(const float4 *__restrict__ src, float4 *__restri
 // dropped.  Gives the read rate the memory side sustains, against which gather traffic is put.  (Measured shapes on
 // MI355X: 2048 workgroups of 256 lanes with one load per lane and trip reach 6.5 TB/s from HBM and 6.8-6.9 TB/s from
 // the Infinity Cache; unrolling to 2 ... 8 loads in flight per lane or 8192 / 32768 workgroups: 5.4-5.9 and 6.4-6.7.)
-__global__ __launch_bounds__(256) void rof_read_kernel(const float4 *__restrict__ src, int64_t n16, float *__restrict__ sink) {
-    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+__global__ __launch_bounds__(256) void rof_read_kernel(const float4 *__restrict__ src, int64_t n16, int repeat,
+                                                       float *__restrict__ sink) {
+    const int64_t first = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     float a = 0.f;
+    for (int r = 0; r < repeat; ++r) {   // repeat > 1: the same buffer again (a buffer small enough stays in L2)
 #pragma unroll 1
-    for (; i < n16; i += stride) {
-        const float4 p = src[i];
-        a += p.x + p.y + p.z + p.w;
+        for (int64_t i = first; i < n16; i += stride) {
+            const float4 p = src[i];
+            a += p.x + p.y + p.z + p.w;
+        }
     }
     if (a == 1.2345e-30f) sink[0] = a;   // practically never true; keeps the loads alive
 }
@@ -379,11 +382,11 @@ int rof_device_copy(void *dst, const void *src, size_t nbytes, void *stream) {
     return ROF_OK;
 }
 
-int rof_device_read(const void *src, size_t nbytes, float *sink, void *stream) {
-    if (!src || !sink || (nbytes & 15) || ((uintptr_t)src & 15)) return ROF_ERR_ARG;
+int rof_device_read(const void *src, size_t nbytes, int repeat, float *sink, void *stream) {
+    if (!src || !sink || repeat < 1 || (nbytes & 15) || ((uintptr_t)src & 15)) return ROF_ERR_ARG;
     if (nbytes == 0) return ROF_OK;
     hipLaunchKernelGGL(rof_read_kernel, dim3(2048), dim3(256), 0, (hipStream_t)stream, (const float4 *)src,
-                       (int64_t)(nbytes / 16), sink);
+                       (int64_t)(nbytes / 16), repeat, sink);
     HIP_TRY(hipGetLastError());
     return ROF_OK;
 }

@@ -403,8 +403,8 @@ def measure_traffic(args, passthrough):
 def read_calibration(L, dev):
     """What plain streaming reaches on this device, as yardsticks for the gather launches' fetch rate: reads of a
     buffer far beyond the caches (2 GiB: HBM), reads of a buffer that the 256 MB Infinity Cache holds but the L2s do
-    not (128 MiB, read repeatedly), and a 1 GiB device-to-device copy (read + write).  GB/s, HIP events on the
-    current stream, best of three."""
+    not (128 MiB, read repeatedly), reads that the L2s serve (16 MiB, read 128 times in one launch), and
+    a 1 GiB device-to-device copy (read + write).  GB/s, HIP events on the current stream, best of three."""
     import ctypes
 
     import torch
@@ -425,11 +425,15 @@ def read_calibration(L, dev):
             best = max(best, nbytes * reps / (e0.elapsed_time(e1) * 1e-3) / 1e9)
         return best
 
-    def read(buf, nbytes):
-        return lambda: _check_rc(L.rof_device_read(ctypes.c_void_p(buf.data_ptr()), nbytes, ctypes.c_void_p(sink.data_ptr()), st))
+    def read(buf, nbytes, repeat=1):
+        return lambda: _check_rc(L.rof_device_read(ctypes.c_void_p(buf.data_ptr()), nbytes, repeat,
+                                                   ctypes.c_void_p(sink.data_ptr()), st))
 
     res = {"hbm_stream_read_GBs": rate(read(big, 2 << 30), 2 << 30, 4),
-           "infinity_cache_read_GBs": rate(read(big, 128 << 20), 128 << 20, 64)}
+           "infinity_cache_read_GBs": rate(read(big, 128 << 20), 128 << 20, 64),
+           # 16 MiB read 128 times in one launch: a workgroup reads the same pieces every time, so each XCD's 4 MB L2
+           # holds its eighth of the buffer after the first pass
+           "l2_read_GBs": rate(read(big, 16 << 20, 128), (16 << 20) * 128, 4)}
     half = big[: (1 << 30) // 4]
     other = big[(1 << 30) // 4:]
     res["copy_read_plus_write_GBs"] = rate(lambda: _check_rc(L.rof_device_copy(

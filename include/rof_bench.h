@@ -30,11 +30,12 @@ int rof_aggregate_launch_times(const rof_layout *layout, const void *x, int x_dt
  * No upstream counterpart. */
 int rof_device_copy(void *dst, const void *src, size_t nbytes, void *stream);
 
-/* Plain streaming read of nbytes (a multiple of 16, pointer 16-byte aligned) of device memory; `sink` is one float
- * of device memory that is practically never written.  Timed over a buffer far larger than the caches it gives the
- * read rate the memory system sustains on this device, the yardstick for the gather launches' fetch rate.
+/* Plain streaming read of nbytes (a multiple of 16, pointer 16-byte aligned) of device memory, `repeat` times over in
+ * one launch; `sink` is one float of device memory that is practically never written.  Timed over a buffer far
+ * larger than the caches it gives the read rate the memory system sustains on this device, the yardstick for the
+ * gather launches' fetch rate; over a buffer of a few MB read many times, the rate of the L2s.
  * No upstream counterpart. */
-int rof_device_read(const void *src, size_t nbytes, float *sink, void *stream);
+int rof_device_read(const void *src, size_t nbytes, int repeat, float *sink, void *stream);
 
 /* Launch tuning of one layout.  Every field has a "library decides" value, which is what a new layout holds; the
  * settings belong to the layout (no process-wide state) and are read by every aggregation that uses it, so change
