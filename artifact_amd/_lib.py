@@ -20,7 +20,7 @@ SYMBOLS = (
     "rof_transpose_csr", "rof_plan_build", "rof_layout_from_v2", "rof_layout_from_v1", "rof_layout_from_parts",
     "rof_layout_export", "rof_layout_stats", "rof_layout_upload", "rof_layout_set_degrees",
     "rof_plan_hub_patterns", "rof_plan_dynamic_greedy", "rof_column_sums", "rof_column_sums_workspace_bytes", "rof_layout_workspace_bytes", "rof_layout_free", "rof_aggregate", "rof_aggregate_epilogue", "rof_aggregate_noalloc", "rof_aggregate_timed", "rof_aggregate_launch_times",
-    "rof_device_copy", "rof_device_read", "rof_layout_set_tuning", "rof_layout_get_tuning", "rof_layout_stats_n", "rof_layout_calibrate",
+    "rof_device_copy", "rof_device_read", "rof_device_gather", "rof_layout_set_tuning", "rof_layout_get_tuning", "rof_layout_stats_n", "rof_layout_calibrate",
 )
 
 
@@ -92,6 +92,7 @@ def lib():
     L.rof_layout_calibrate.argtypes = [vp, vp, ci, i64, vp, i64, ci, ci, C.POINTER(Epilogue), vp, C.c_size_t, vp, ci, ci,
                                        C.POINTER(LaunchTuning)]
     L.rof_device_read.argtypes = [vp, C.c_size_t, ci, vp, vp]
+    L.rof_device_gather.argtypes = [vp, u32, ci, ci, vp, vp, C.POINTER(C.c_uint64)]
     L.rof_column_sums_workspace_bytes.argtypes = [i64, ci]
     L.rof_column_sums_workspace_bytes.restype = C.c_size_t
     L.rof_column_sums.argtypes = [vp, ci, i64, i64, ci, vp, vp, C.c_size_t, vp]

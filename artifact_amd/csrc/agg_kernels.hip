@@ -129,6 +129,29 @@ __global__ __launch_bounds__(256) void rof_read_kernel(const float4 *__restrict_
     if (a == 1.2345e-30f) sink[0] = a;   // practically never true; keeps the loads alive
 }
 
+// nothing but row gathers: every lane group of LPR lanes fetches pseudo-random rows of LPR * 16 bytes from a table of
+// rows_mask + 1 rows, two in flight, and adds them up.  The rate it reaches from a table that the L2s hold, that the
+// Infinity Cache holds, or that only HBM holds is the yardstick for the aggregation launches, whose gathers are of
+// exactly this shape (plus indices, weights and stores).
+template <int LPR>
+__global__ __launch_bounds__(256) void rof_gather_kernel(const char *__restrict__ table, uint32_t rows_mask, int iters,
+                                                         float *__restrict__ sink) {
+    const int lane = threadIdx.x & 63, sub = lane / LPR, li = lane % LPR;
+    if (lane >= (64 / LPR) * LPR) return;   // lanes left over when LPR does not divide 64
+    uint32_t s = (blockIdx.x * 256u + (threadIdx.x & ~63u)) * 2654435761u + sub * 40503u + 12345u;
+    float a = 0.f;
+    for (int it = 0; it < iters; ++it) {
+        s = s * 1664525u + 1013904223u;
+        const uint32_t r0 = (s >> 8) & rows_mask;
+        s = s * 1664525u + 1013904223u;
+        const uint32_t r1 = (s >> 8) & rows_mask;
+        const rofk::rof_f4 p = *reinterpret_cast<const rofk::rof_f4 *>(table + (size_t)r0 * (LPR * 16) + li * 16);
+        const rofk::rof_f4 q = *reinterpret_cast<const rofk::rof_f4 *>(table + (size_t)r1 * (LPR * 16) + li * 16);
+        a += (p.x + p.y + p.z + p.w) + (q.x + q.y + q.z + q.w);
+    }
+    if (a == 1.2345e-30f) sink[0] = a;   // practically never true; keeps the loads alive
+}
+
 // Column sums of a row-major [n, f] matrix (the bias gradient of a layer), in two launches with a fixed
 // order of summation.  A workgroup owns a run of rows; its four wavefronts take every fourth row of the run,
 // 64 lanes across 64 consecutive columns, so each load instruction reads one contiguous piece of a row.
@@ -388,6 +411,27 @@ int rof_device_read(const void *src, size_t nbytes, int repeat, float *sink, voi
     hipLaunchKernelGGL(rof_read_kernel, dim3(2048), dim3(256), 0, (hipStream_t)stream, (const float4 *)src,
                        (int64_t)(nbytes / 16), repeat, sink);
     HIP_TRY(hipGetLastError());
+    return ROF_OK;
+}
+
+int rof_device_gather(const void *table, uint32_t rows, int lanes_per_row, int iters, float *sink, void *stream,
+                      uint64_t *gathered_rows) {
+    if (!table || !sink || iters < 1 || rows == 0 || (rows & (rows - 1)) || ((uintptr_t)table & 15)) return ROF_ERR_ARG;
+    const dim3 grid(256 * 32), block(256);
+    hipStream_t st = (hipStream_t)stream;
+    switch (lanes_per_row) {
+        case 4: hipLaunchKernelGGL(rof_gather_kernel<4>, grid, block, 0, st, (const char *)table, rows - 1, iters, sink); break;
+        case 8: hipLaunchKernelGGL(rof_gather_kernel<8>, grid, block, 0, st, (const char *)table, rows - 1, iters, sink); break;
+        case 10: hipLaunchKernelGGL(rof_gather_kernel<10>, grid, block, 0, st, (const char *)table, rows - 1, iters, sink); break;
+        case 12: hipLaunchKernelGGL(rof_gather_kernel<12>, grid, block, 0, st, (const char *)table, rows - 1, iters, sink); break;
+        case 16: hipLaunchKernelGGL(rof_gather_kernel<16>, grid, block, 0, st, (const char *)table, rows - 1, iters, sink); break;
+        case 20: hipLaunchKernelGGL(rof_gather_kernel<20>, grid, block, 0, st, (const char *)table, rows - 1, iters, sink); break;
+        case 32: hipLaunchKernelGGL(rof_gather_kernel<32>, grid, block, 0, st, (const char *)table, rows - 1, iters, sink); break;
+        case 64: hipLaunchKernelGGL(rof_gather_kernel<64>, grid, block, 0, st, (const char *)table, rows - 1, iters, sink); break;
+        default: return ROF_ERR_UNSUPPORTED;
+    }
+    HIP_TRY(hipGetLastError());
+    if (gathered_rows) *gathered_rows = (uint64_t)grid.x * 4 * (64 / lanes_per_row) * 2 * (uint64_t)iters;
     return ROF_OK;
 }
 

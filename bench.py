@@ -396,11 +396,12 @@ def measure_traffic(args, passthrough):
         hit, miss = per.get(("TCC_HIT_sum", phase)), per.get(("TCC_MISS_sum", phase))
         res["launch"][phase] = {"read_bytes": rd, "written_bytes": wr, "bytes": rd + wr,
                                 "tcc_hit_rate": hit / (hit + miss) if hit is not None and miss else None,
-                                "tcc_miss_x_128B": miss * 128.0 if miss is not None else None}
+                                "tcc_miss_x_128B": miss * 128.0 if miss is not None else None,
+                                "tcc_hit_x_128B": hit * 128.0 if hit is not None else None}
     return res
 
 
-def read_calibration(L, dev):
+def read_calibration(L, dev, gather_lanes=0):
     """What plain streaming reaches on this device, as yardsticks for the gather launches' fetch rate: reads of a
     buffer far beyond the caches (2 GiB: HBM), reads of a buffer that the 256 MB Infinity Cache holds but the L2s do
     not (128 MiB, read repeatedly), reads that the L2s serve (16 MiB, read 128 times in one launch), and
@@ -434,6 +435,22 @@ def read_calibration(L, dev):
            # 16 MiB read 128 times in one launch: a workgroup reads the same pieces every time, so each XCD's 4 MB L2
            # holds its eighth of the buffer after the first pass
            "l2_read_GBs": rate(read(big, 16 << 20, 128), (16 << 20) * 128, 4)}
+    if gather_lanes in (4, 8, 10, 12, 16, 20, 32, 64):
+        # nothing but gathers of rows as wide as the workload's (16 bytes per lane), pseudo-random, two in flight: from
+        # a table that the L2s hold, that the Infinity Cache holds, and that only HBM holds; GB/s of gathered row bytes
+        row = 16 * gather_lanes
+        got = ctypes.c_uint64()
+        gres = {"row_bytes": row}
+        for tag, table_bytes, iters in (("l2", 1 << 20, 1000), ("infinity_cache", 48 << 20, 250), ("hbm", 2 << 30, 250)):
+            rows = 1 << int(np.floor(np.log2(table_bytes // row)))
+
+            def gather(rows=rows, iters=iters):
+                _check_rc(L.rof_device_gather(ctypes.c_void_p(big.data_ptr()), rows, gather_lanes, iters,
+                                              ctypes.c_void_p(sink.data_ptr()), st, ctypes.byref(got)))
+
+            gather()
+            gres[tag + "_GBs"] = rate(gather, got.value * row, 1)
+        res["row_gathers"] = gres
     half = big[: (1 << 30) // 4]
     other = big[(1 << 30) // 4:]
     res["copy_read_plus_write_GBs"] = rate(lambda: _check_rc(L.rof_device_copy(
@@ -602,7 +619,7 @@ def main():
             f"candidates")
     deg = torch.from_numpy(np.diff(indptr).astype(np.float32)).to(dev)
 
-    calibration = None if args.quick else read_calibration(L, dev)
+    calibration = None if args.quick else read_calibration(L, dev, lanes_per_row(feat, bf16))
     x, x32, ld = make_features(name, n, feat, bf16, dev, args.packed_input)
     in_bytes = 2 if bf16 else 4
     lpr = lanes_per_row(feat, bf16)
@@ -841,6 +858,24 @@ def main():
                                        + traffic["error"])
     tl = traffic.get("launch", {})
 
+    def gather_model(t, ms):
+        """The launch against what nothing-but-gathers reaches on this device: its L2 hits priced at the rate of row
+        gathers that the L2s serve, its L2 misses at the rate of row gathers from HBM (and from the Infinity Cache),
+        in 128-byte lines (a gathered row of R bytes occupies ceil(R / 128) lines).  An estimate, not a bound: misses
+        with locality (the swept launch) or served by the Infinity Cache come faster than random rows from HBM, stores
+        are priced like gathers.  A launch close to it does little else than wait for its lines."""
+        g = (calibration or {}).get("row_gathers")
+        if not g or not t or not t.get("tcc_hit_x_128B") or not t.get("tcc_miss_x_128B") or ms <= 0:
+            return None
+        per_row = -(-g["row_bytes"] // 128) * 128.0 / g["row_bytes"]      # line bytes fetched per useful byte
+        hit_b, miss_b = t["tcc_hit_x_128B"], t["tcc_miss_x_128B"]
+        ms_of = lambda tag: (hit_b / (g["l2_GBs"] * per_row) + miss_b / (g[tag] * per_row)) / 1e9 * 1e3
+        return {"row_bytes": g["row_bytes"], "l2_hit_bytes": hit_b, "l2_miss_bytes": miss_b,
+                "line_GBs": {"l2": g["l2_GBs"] * per_row, "infinity_cache": g["infinity_cache_GBs"] * per_row,
+                             "hbm": g["hbm_GBs"] * per_row},
+                "model_ms_misses_from_hbm": ms_of("hbm_GBs"), "model_ms_misses_from_infinity_cache": ms_of("infinity_cache_GBs"),
+                "measured_ms": ms, "measured_over_model_hbm": ms / ms_of("hbm_GBs")}
+
     def roof(phase, label, alg_bytes, ms):
         t = tl.get(phase)
         tb = t["bytes"] if t and ms > 0 else None
@@ -858,6 +893,7 @@ def main():
             "traffic": tb, "traffic_read": t["read_bytes"] if t else None, "traffic_written": t["written_bytes"] if t else None,
             "tcc_hit_rate": t.get("tcc_hit_rate") if t else None,
             "tcc_miss_x_128B": t.get("tcc_miss_x_128B") if t else None,
+            "gather_model": gather_model(t, ms),
             "ms_per_launch": ms,
             # the model figure: one gathered row per edge whether or not a cache served it; exceeds the HBM peak
             # when rows gathered many times come from L2 / Infinity Cache

@@ -37,6 +37,15 @@ int rof_device_copy(void *dst, const void *src, size_t nbytes, void *stream);
  * No upstream counterpart. */
 int rof_device_read(const void *src, size_t nbytes, int repeat, float *sink, void *stream);
 
+/* Nothing but row gathers, as a yardstick for the aggregation launches: every group of `lanes_per_row` lanes (4, 8,
+ * 10, 12, 16, 20, 32 or 64; a row has 16 x lanes_per_row bytes) fetches 2 x iters pseudo-random rows of a table of `rows` rows
+ * (a power of two; 16-byte aligned), two in flight.  *gathered_rows (may be NULL) receives the number of rows the
+ * launch fetches.  Timed over a table that the L2s hold (1-2 MiB), that the Infinity Cache holds (tens of MiB) or
+ * that only HBM holds (GiB), it gives the rates that gathers of that row size can reach on this device.
+ * No upstream counterpart. */
+int rof_device_gather(const void *table, uint32_t rows, int lanes_per_row, int iters, float *sink, void *stream,
+                      uint64_t *gathered_rows);
+
 /* Launch tuning of one layout.  Every field has a "library decides" value, which is what a new layout holds; the
  * settings belong to the layout (no process-wide state) and are read by every aggregation that uses it, so change
  * them only while no other thread launches with the same layout.  No upstream counterpart.
