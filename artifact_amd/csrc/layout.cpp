@@ -842,10 +842,14 @@ int rof_layout_export(const rof_layout *L, rof_bag **out) {
 
 int rof_layout_stats_n(const rof_layout *L, int64_t *stats, int count) {
     if (!L || !stats || count < 0) return ROF_ERR_ARG;
-    int64_t s[20];
+    int64_t s[23];
     int rc = rof_layout_stats(L, s);
     if (rc) return rc;
-    for (int i = 0; i < count; ++i) stats[i] = i < 20 ? s[i] : 0;
+    s[20] = L->hub_split;
+    s[21] = L->segment;
+    s[22] = 0;   // longest task of the destination-row launch
+    for (int32_t t = 0; t < L->b.n_tasks; ++t) s[22] = std::max<int64_t>(s[22], L->b.task_ptr[t + 1] - L->b.task_ptr[t]);
+    for (int i = 0; i < count; ++i) stats[i] = i < 23 ? s[i] : 0;
     return ROF_OK;
 }
 

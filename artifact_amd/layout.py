@@ -18,7 +18,8 @@ NOALLOC_WORKSPACE_BYTES = 64 << 20   # ROF_NOALLOC_WORKSPACE_BYTES of include/ro
 
 STAT_NAMES = ("nodes", "edges", "groups", "materialised_groups", "gathered_rows", "partial_reads", "partial_rows",
               "hub_segments", "tasks_a", "tasks_b", "device_bytes", "part_size", "wave_tasks_a", "wave_tasks_b",
-              "canonical", "gathered_rows_a", "local_groups", "lds_reads", "cluster_workgroups", "lds_rows")
+              "canonical", "gathered_rows_a", "local_groups", "lds_reads", "cluster_workgroups", "lds_rows", "hub_split",
+              "segment", "longest_row_task")
 
 EXPORT_NAMES = ("group_ptr", "group_col", "group_dst_ptr", "group_dst", "res_ptr", "res_col", "canonical", "xcd_run", "long_row_cut",
                 "uniqpart_column_index", "uniqpart_pointers", "part2Node_ptr", "part2Node_col",
@@ -145,12 +146,11 @@ class LayoutFamily:
         ld = -(-feat // mult) * mult
         x = torch.randn((n, ld), device="cuda").to(torch.bfloat16 if bf16 else torch.float32)[:, :feat]
         out = torch.empty((n, feat), dtype=torch.float32, device="cuda")
-        ex = first.export()
-        rule = (ex["hub_split"], ex["segment"])
-        longest = int(np.diff(ex["b_task_ptr"]).max()) if len(ex["b_task_ptr"]) > 1 else 0
-        del ex
+        st = first.stats()
+        rule = (st["hub_split"], st["segment"])
         cands = {rule: first}
-        if first.stats()["hub_segments"] or longest > min(c for c, _ in CUT_CANDIDATES[key[1]]):
+        # other cuts can only matter when some row is long enough to be cut by one of them
+        if st["hub_segments"] or st["longest_row_task"] > min(c for c, _ in CUT_CANDIDATES[key[1]]):
             for cut, seg in CUT_CANDIDATES[key[1]]:
                 if (cut, seg) not in cands:
                     cands[(cut, seg)] = self._make(key, hub_split=cut, segment=seg)
@@ -251,8 +251,8 @@ class Layout:
         return r
 
     def stats(self):
-        s = (C.c_int64 * 20)()
-        check(_lib.lib().rof_layout_stats(self._h, s))
+        s = (C.c_int64 * len(STAT_NAMES))()
+        check(_lib.lib().rof_layout_stats_n(self._h, s, len(STAT_NAMES)))
         return {k: int(s[i]) for i, k in enumerate(STAT_NAMES)}
 
     def set_tuning(self, xcd_run_partial=0, xcd_run_dst=0, wave_cap=-1, lds_pad=0, deep=-1):

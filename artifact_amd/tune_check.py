@@ -71,7 +71,7 @@ def check(name, widths=WIDTHS, log=print):
         out = torch.empty((n, feat), device="cuda")
         rb = feat * eb
         base = Layout.from_csr(ip, ix, lanes_per_row=lpr, elem_bytes=eb, row_bytes=rb)
-        cut = base.export()["hub_split"]
+        cut = base.stats()["hub_split"]
         variants = {"default": (base, {})}
         for cap in (0, 7, 6):
             variants[f"waves {cap or 8}"] = (base, dict(wave_cap=cap))

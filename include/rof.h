@@ -201,7 +201,9 @@ int rof_layout_export(const rof_layout *layout, rof_bag **out);
  * per workgroup that sums it) [17] reads of them [18] workgroups that hold clustered destinations [19] LDS rows the
  * destination-row launch asks for per workgroup. */
 int rof_layout_stats(const rof_layout *layout, int64_t stats[20]);
-/* The first `count` of those counters (fewer than the library knows: the rest is dropped; more: zero-filled). */
+/* The first `count` of the counters the library knows (fewer: the rest is dropped; more: zero-filled): the twenty
+ * above, then [20] the cut of long rows (hub_split) and [21] the segment length as chosen for this layout, [22] the
+ * entries of the longest task of the destination-row launch. */
 int rof_layout_stats_n(const rof_layout *layout, int64_t *stats, int count);
 
 /* Copy the schedule to the current HIP device (idempotent). */

@@ -221,6 +221,9 @@ def test_long_rows_are_cut_by_width_and_their_segments_swept_by_source_id(lanes,
     n = len(ip) - 1
     lay = Layout.from_csr(ip, ix, lanes_per_row=lanes, elem_bytes=elem, row_bytes=row)
     assert (lay.export()["hub_split"], lay.export()["segment"]) == (cut, seg)
+    st0 = lay.stats()                                        # the same through the counters, without an export
+    assert (st0["hub_split"], st0["segment"]) == (cut, seg)
+    assert st0["longest_row_task"] == int(np.diff(lay.export()["b_task_ptr"]).max())
     ex, st = lay.export(), lay.stats()
     deg = np.diff(ip)
     assert st["hub_segments"] == int(np.ceil(deg[deg > cut] / seg).sum())
