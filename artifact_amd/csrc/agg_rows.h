@@ -235,13 +235,12 @@ __device__ __forceinline__ void gather_sum(const char *xb, uint32_t xld, const c
 // Scale the finished sum of task t, apply the layer's epilogue (PHASE 1, 2 and 4) and store this lane's piece of the
 // output row.  `acc` holds the columns cstart .. cstart + VEC - 1; `skip` of them repeat the neighbouring lane's.
 template <typename XT, int VEC, int PHASE>
-__device__ __forceinline__ void finish_row(const AggArgs &a, int32_t t, bool nonempty, const float (&acc)[VEC], const char *xb,
-                                           uint32_t xld, int cstart, int skip) {
+__device__ __forceinline__ void finish_row(const AggArgs &a, int32_t out_row, float scale, bool nonempty, const float (&acc)[VEC],
+                                           const char *xb, uint32_t xld, int cstart, int skip) {
     // an empty task writes zeros whatever its scale is (a node without in-edges keeps the
     // zero-initialised output upstream: reuse_conv_kernel.cu:303)
-    float s = 1.0f;
-    if (a.task_scale && nonempty) s = a.task_scale[t];
-    const int64_t at = (int64_t)a.task_out[t] * a.ldo + cstart;
+    const float s = nonempty ? scale : 1.0f;
+    const int64_t at = (int64_t)out_row * a.ldo + cstart;
     float r[VEC];
 #pragma unroll
     for (int k = 0; k < VEC; ++k) r[k] = acc[k] * s;
@@ -249,7 +248,7 @@ __device__ __forceinline__ void finish_row(const AggArgs &a, int32_t t, bool non
     if (kDst) {   // epilogue of the layer: + own row, + bias, then ReLU (columns cstart .. cstart+VEC-1 exist)
         if (a.self_weight != 0.0f) {
             float own[VEC];
-            RowLoad<XT, VEC>::load(reinterpret_cast<const XT *>(xb + (int64_t)a.task_out[t] * xld), own);
+            RowLoad<XT, VEC>::load(reinterpret_cast<const XT *>(xb + (int64_t)out_row * xld), own);
 #pragma unroll
             for (int k = 0; k < VEC; ++k) r[k] = fmaf(a.self_weight, own[k], r[k]);
         }
@@ -370,10 +369,20 @@ __global__ __launch_bounds__(256) void rof_rows_kernel(AggArgs a) {
         t = a.n_wave + (gw - a.n_wave) * G + sub;
         valid = !idle && t < a.n_tasks;
     }
+    // The output row and its scale are needed last.  The launches that run with more gathers in flight serve small
+    // matrices and are bound by the latency of their longest chain of dependent loads, so they fetch both up front,
+    // with the task's range; everywhere else the two registers would cost an occupancy step, and the loads wait
+    // until the sum is finished.
+    int32_t out_row = 0;
+    float out_scale = 1.0f;
     if (valid) {
         beg = a.task_ptr[t];
         end = a.task_ptr[t + 1];
         mid = beg + a.task_nref[t];
+        if constexpr (kDeep) {
+            out_row = a.task_out[t];
+            if (a.task_scale) out_scale = a.task_scale[t];
+        }
     }
     const uint32_t xld = (uint32_t)(a.ldx * (int64_t)sizeof(XT)), pld = (uint32_t)(a.ldp * 4);
 
@@ -441,8 +450,15 @@ __global__ __launch_bounds__(256) void rof_rows_kernel(AggArgs a) {
             }
         }
 
-        if (valid && act && (!wave_mode || sub == 0))
-            finish_row<XT, VEC, PHASE>(a, t, end > beg, acc, xb, xld, cstart, skip);
+        if (valid && act && (!wave_mode || sub == 0)) {
+            if constexpr (!kDeep) {
+                if (c0 == 0) {
+                    out_row = a.task_out[t];
+                    if (a.task_scale && end > beg) out_scale = a.task_scale[t];
+                }
+            }
+            finish_row<XT, VEC, PHASE>(a, out_row, out_scale, end > beg, acc, xb, xld, cstart, skip);
+        }
     }
 }
 
@@ -537,7 +553,9 @@ __global__ __launch_bounds__(256) void rof_cluster_kernel(AggArgs a) {
                 gather_sum<XT, VEC, LPR, false, false, OFF32, PHASE == 2>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, mid, end, lane,
                                                                          sub, li, act, acc);
             }
-            if (valid && act) finish_row<XT, VEC, PHASE>(a, t, end > first, acc, xb, xld, cstart, skip);
+            if (valid && act)
+                finish_row<XT, VEC, PHASE>(a, a.task_out[t], (a.task_scale && end > first) ? a.task_scale[t] : 1.0f, end > first, acc,
+                                           xb, xld, cstart, skip);
         }
     }
 }
