@@ -50,33 +50,63 @@ const int64_t kWavesToFill = 2 * 8192;   // two rounds of 256 CUs x 32 wavefront
 //     128 / 32 on smaller matrices (1024 / 128 +3 %);
 //   fp32, G = 4 (64 floats): 1024 / 128 (384 / 96 0 ... +6 %, 128 / 32 +1 ... +19 %);
 //   fp32, G >= 5: 640 / 160 (1024 / 256 -2 ... +2 %, 256 / 64 +4 ... +7 %, 5457 +7 % on the 2.4 M-node workload);
+//   fp32, G >= 4, fewer rows than fill the machine twice: 256 / 128 (G = 4: 128 / 64), and any cut steps down where
+//     the longest task under it would outlast the launch (see default_cut);
 //   bf16, G <= 2 (256 columns): 256 / 48 (2^22 nodes: -18 % against 8192; segments of 32 / 40 / 48 / 56 / 64 / 96 /
-//     128 entries 8.53 / 8.49 / 8.46 / 8.57 / 8.57 / 8.92 / 9.17 ms); G = 3: 512 / 128; G >= 4 (128 columns):
+//     128 entries 8.53 / 8.49 / 8.46 / 8.57 / 8.57 / 8.92 / 9.17 ms), 256 / 128 when the caches can hold the matrix,
+//     128 / 32 on launches that cannot fill the machine twice; G = 3: 512 / 128; G >= 4 (128 columns):
 //     1280 / 320 (640 / 160 -1 ... +4 %, 2560 / 640 0 ... +4 %).
 // No rule of sizes gets every graph right (the same width wants 128 / 32 on one graph and 1024 / 128 on another),
 // which is what the timed choice between candidate layouts is for (LayoutFamily(autotune=True)).
 // (Giving long rows a whole workgroup instead -- four wavefronts combined through LDS -- was measured as well:
 // no faster than segments on any workload, so it is not built in.)
 const int64_t kCachedMatrixBytes = 256 << 20;   // the Infinity Cache
-void default_cut(int32_t groups, int32_t elem_bytes, int64_t row_bytes, int64_t matrix_bytes, int32_t &cut, int32_t &segment) {
-    if (elem_bytes == 2) {
-        cut = groups <= 2 ? 256 : groups == 3 ? 512 : 1280;
-        segment = groups <= 2 ? cut * 3 / 16 : cut / 4;
-        return;
-    }
+void default_cut(int32_t groups, int32_t elem_bytes, int64_t row_bytes, int64_t matrix_bytes, int64_t rows, int64_t edges,
+                 int32_t &cut, int32_t &segment) {
     const bool cached = matrix_bytes <= kCachedMatrixBytes;
-    if (groups == 1 && row_bytes >= 1024) {
+    if (elem_bytes == 2 && groups <= 2) {
+        // segments of 48 entries are the optimum of the 2^22-node workload; matrices that the caches hold want
+        // fewer, longer segments (2^16 ... 2^18 nodes x 256 columns: 256 / 128 is 3 ... 23 % faster than 256 / 48),
+        // and the smallest launches the short chains of 128 / 32
+        cut = rows / groups < kWavesToFill ? 128 : 256;
+        segment = rows / groups < kWavesToFill ? 32 : cached ? 128 : 48;
+    } else if (elem_bytes == 2) {
+        cut = groups == 3 ? 512 : 1280;
+        segment = cut / 4;
+    } else if (groups == 1 && row_bytes >= 1024) {
         cut = cached ? 128 : 256;
         segment = 32;
     } else if (groups <= 3) {
         cut = cached ? 128 : 1024;
         segment = cached ? 32 : 128;
+    } else if (rows / groups < kWavesToFill) {
+        // a destination-row launch that cannot fill the machine twice lasts as long as its longest task: a lower cut
+        // shortens that chain of dependent gathers (2^14 nodes x 32 floats: 13.2 us at 640 / 160, 11.0 at 256 / 128,
+        // 11.6 at 128 / 64, 14.3 at 1024 / 256; 2^15 nodes x 64 floats: 25.4 us at 256 / 128, 20.5 at 128 / 64)
+        cut = groups == 4 ? 128 : 256;
+        segment = groups == 4 ? 64 : 128;
     } else if (groups == 4) {
         cut = 1024;
         segment = 128;
     } else {
         cut = 640;
         segment = 160;
+    }
+    // The longest task under the cut is one chain of dependent gathers, measured at (10 + 0.14 x row bytes) ns an
+    // entry while the caches serve them; a launch lasts about 15 us + 60 us per GB it gathers.  Where a chain of
+    // `cut` entries would outlast 3/4 of that, the launch waits for its longest rows (2^17 nodes, average degree 8,
+    // 64 floats: 46.6 us at 1024 / 128, 30.3 at 384 / 96; 2^16 nodes, degree 15: 45.8 against 25.7), so the cut
+    // steps down.
+    const int64_t launch_ns = 15000 + edges * row_bytes * 60 / 1000000;
+    const int64_t entry_ns = 10 + row_bytes * 14 / 100;
+    const int64_t limit = 3 * launch_ns / (4 * entry_ns);
+    static const int32_t kLadder[][2] = {{1024, 128}, {640, 160}, {384, 96}, {256, 128}};
+    for (const auto &step : kLadder) {
+        if (cut <= limit || cut <= 256) break;
+        if (step[0] < cut) {
+            cut = step[0];
+            segment = step[1];
+        }
     }
 }
 // Sharing groups costs one more launch (~4-6 us on MI355X), and on heavy-tailed graphs what it saves is cheap:
@@ -413,7 +443,8 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     const int32_t elem_bytes = (o && o->elem_bytes == 2) ? 2 : 4;
     const int64_t row_bytes = (o && o->row_bytes > 0) ? o->row_bytes : (int64_t)lpr * 16;
     int32_t rule_cut = 0, rule_segment = 0;
-    default_cut(groups, elem_bytes, row_bytes, (int64_t)n * row_bytes, rule_cut, rule_segment);
+    default_cut(groups, elem_bytes, row_bytes, (int64_t)n * row_bytes, n, L->e_orig > 0 ? L->e_orig : total, rule_cut,
+                rule_segment);
     const int32_t hub_split = (o && o->hub_split > 0) ? o->hub_split : rule_cut;
     // (a caller's cut with the library's segment: the rule's share of the rule's cut)
     const int32_t segment = (o && o->segment > 0) ? o->segment
@@ -527,6 +558,11 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     tb.out.reserve(n);
     tb.col.reserve(L->res_col.size() + L->group_dst.size());
     int64_t gathered = (int64_t)tg.col.size() + (int64_t)cl.lg_col.size(), reads = 0, segments = 0, nearby = 0, lds_reads = 0;
+    // "nearby" = within two tiles of ids, and within a sixteenth of the graph: on a graph of a few tiles every source
+    // is within two tiles, which says nothing about locality (R-MAT, 2^14 ... 2^15 nodes: taken for local, whole
+    // tiles per XCD run cost 12 ... 25 % against runs of 4; a block model of sixteen 4096-node blocks still gains
+    // 23 % from them)
+    const int32_t near_ids = (int32_t)std::max<int64_t>(1, std::min<int64_t>(2 * kTileRows, n / 16));
     ivec row;   // one destination's entries: LDS rows first, then references, then feature rows
     ivec local_row(G, -1);
     for (int32_t v = 0; v < n; ++v) {
@@ -558,7 +594,7 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
         if (entry_order == 0) std::sort(row.begin() + nlds + refs, row.end(), std::greater<int32_t>());
         else if (entry_order == 2) std::sort(row.begin() + nlds + refs, row.end());
         const int64_t len = (int64_t)row.size();
-        for (int64_t j = nlds + refs; j < len; ++j) nearby += std::abs(row[j] - v) < 2 * kTileRows;
+        for (int64_t j = nlds + refs; j < len; ++j) nearby += std::abs(row[j] - v) < near_ids;
         gathered += len - refs - nlds;
         reads += refs;
         lds_reads += nlds;

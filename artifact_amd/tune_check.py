@@ -2,7 +2,7 @@
 own choice of wavefront cap, XCD run, row gathers in flight and long-row cut within a few per cent of the best of
 the alternatives?
 
-    python -m artifact_amd.tune_check [--graphs h1,h2,h3,h4] [--out table.md]
+    python -m artifact_amd.tune_check [--graphs h1,...,h7] [--out table.md]
 
 For every (graph, width) one aggregation layer (no reuse plan: `Layout.from_csr`) is timed with the default layout
 and launch settings and then with one setting changed at a time: wavefronts per SIMD of the destination-row launch
@@ -35,6 +35,10 @@ GRAPHS = {
     "h2": ("R-MAT a=.65 b=c=.15, 2^20 nodes, average degree 48", lambda: rmat_csr(1 << 20, 48, 72, a=0.65, b=0.15, c=0.15)),
     "h3": ("uniform degrees (16 random partners per node), 2^21 nodes", lambda: uniform_degree_csr(1 << 21, 16, 73)),
     "h4": ("block model, 2048 blocks of 1024 nodes, degree 16 inside + 4 outside", lambda: sbm_csr(2048, 1024, 16, 4, 74)),
+    # small launches: bound by their longest chain of dependent gathers, not by the memory side
+    "h5": ("R-MAT a=.5 b=c=.2, 2^16 nodes, average degree 24", lambda: rmat_csr(1 << 16, 24, 75, a=0.5, b=0.2, c=0.2)),
+    "h6": ("R-MAT a=.62 b=c=.16, 2^15 nodes, average degree 12", lambda: rmat_csr(1 << 15, 12, 76, a=0.62, b=0.16, c=0.16)),
+    "h7": ("R-MAT a=.55 b=.25 c=.15, 2^17 nodes, average degree 6", lambda: rmat_csr(1 << 17, 6, 77, a=0.55, b=0.25, c=0.15)),
 }
 WIDTHS = ((24, False), (72, False), (160, False), (128, True))
 
@@ -90,7 +94,7 @@ def check(name, widths=WIDTHS, log=print):
                            autotune=True)
         tuned = fam.get(feat, bf16, normalized=False)
         variants["autotuned"] = (tuned, tuned.tuning())
-        res = time_round_robin(variants, x, feat, out)
+        res = time_round_robin(variants, x, feat, out, iters=8 if n >= 1 << 19 else 40)
         picked = next(iter(fam.chosen.values()))
         fam.close()
         for lay in others + [base]:
@@ -127,7 +131,7 @@ def main():
     for g in args.graphs.split(","):
         rows += check(g, log=lambda *a: print(*a, file=sys.stderr, flush=True))
     note = ("ms per aggregation layer (sum aggregation, no reuse plan; the variants of a row are timed in turn, 3 rounds "
-            "of 8 calls each, median of the rounds); one setting changed at a time.")
+            "of 8 calls each -- 40 on graphs under 2^19 nodes --, median of the rounds); one setting changed at a time.")
     text = "\n".join(f"* {k}: {GRAPHS[k][0]}" for k in args.graphs.split(",")) + "\n\n" + note + "\n\n" + table(rows) + "\n"
     print(text)
     if args.out:

@@ -194,8 +194,8 @@ def test_random_graphs_with_shared_neighbour_sets_through_clusters(oracle, seed)
         # only rows that are cut into segments may reference a shared group: the references sit in segment tasks
         # (or in a row that sharing shortened below the cut), never in a row that was short to begin with
         b_ref_rows = ex["b_task_out"][(ex["b_task_nref"] > 0) & (np.diff(ex["b_task_ptr"]) > ex["b_task_nref"])]
-        cut = opts["hub_split"] or {4: 640, 8: 640, 12: 640, 16: 384, 32: 128, 64: 128}[opts["lanes_per_row"]] * (2 if opts["elem_bytes"] == 2 else 1)
-        assert all(np.diff(ip)[v] > min(cut, 640) for v in b_ref_rows), opts
+        cut = st["hub_split"]   # the cut the layout took: the caller's, or the rule's for these sizes
+        assert all(np.diff(ip)[v] > cut for v in b_ref_rows), opts
     x = rng.standard_normal((n, 2))
     w = rng.uniform(0.5, 2.0, n)
     got = emulate_schedule(ex, n, x, lambda c: w[c], lambda v: w[v], st["partial_rows"])
@@ -270,6 +270,35 @@ def test_small_matrices_keep_the_fine_cut():
                              (16, 0, (1024, 128)), (64, 1024, (128, 32)), (64, 2048, (256, 32))):
         ex = Layout.from_csr(ip, ix, lanes_per_row=lanes, row_bytes=row).export()
         assert (ex["hub_split"], ex["segment"]) == want, (lanes, row)
+
+
+def test_small_launches_cut_long_rows_lower():
+    """A launch that cannot fill the machine twice (fewer than 16 384 wavefronts of rows) is bound by its longest
+    chain of dependent gathers: 256 / 128 from five rows per wavefront, 128 / 64 at four, 128 / 32 for wide bf16
+    rows.  Beyond that size the cut still steps down (1024 -> 640 -> 384 -> 256) while a chain of `cut` entries
+    would outlast 3/4 of the launch, priced at (10 + 0.14 x row bytes) ns an entry against 15 us + 60 us per GB
+    gathered.  bf16 rows of 256 columns take segments of 128 entries instead of 48 when the caches hold the matrix."""
+    def cut_of(ip, ix, **kw):
+        st = Layout.from_csr(ip, ix, **kw).stats()
+        return st["hub_split"], st["segment"]
+    ip, ix = make_workload("c1", 0)                          # 2^14 rows
+    assert cut_of(ip, ix, lanes_per_row=8) == (256, 128)
+    assert cut_of(ip, ix, lanes_per_row=12) == (256, 128)
+    assert cut_of(ip, ix, lanes_per_row=16) == (128, 64)
+    assert cut_of(ip, ix, lanes_per_row=32) == (128, 32)     # up to three rows per wavefront: the fine cut anyway
+    assert cut_of(ip, ix, lanes_per_row=32, elem_bytes=2) == (128, 32)
+    assert cut_of(ip, ix, lanes_per_row=16, elem_bytes=2) == (256, 128)     # 1280 / 320 stepped down
+    ip, ix = rmat_csr(1 << 17, 8, seed=24)                   # 1.0 M edges
+    e = len(ix)
+    for lanes, rule in ((16, 1024), (12, 640), (8, 640)):
+        limit = 3 * (15000 + e * lanes * 16 * 60 // 1000000) // (4 * (10 + lanes * 16 * 14 // 100))
+        want = next(c for c in ((rule, 0), (640, 160), (384, 96), (256, 128)) if c[0] <= max(limit, 256) and c[0] <= rule)
+        got = cut_of(ip, ix, lanes_per_row=lanes)
+        assert got[0] == want[0] and got[0] < rule and (want[1] == 0 or got[1] == want[1]), (lanes, got, limit)
+    assert cut_of(ip, ix, lanes_per_row=32, elem_bytes=2) == (256, 128)     # 64 MB of bf16 rows: cached
+    ip, ix = make_workload("c4", 2)                          # 600 000 rows, 15 M edges: no chain outlasts the launch
+    assert cut_of(ip, ix, lanes_per_row=16) == (1024, 128) and cut_of(ip, ix, lanes_per_row=12) == (640, 160)
+    assert cut_of(ip, ix, lanes_per_row=32, elem_bytes=2) == (256, 48)      # 307 MB of bf16 rows
 
 
 def test_xcd_run_follows_the_locality_of_the_graph():
