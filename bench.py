@@ -658,6 +658,34 @@ def main():
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
 
+    # ---- launch-bound workloads only: the same step captured in a HIP graph and replayed, alone and eight to a graph
+    # (a model's forward pass holds several aggregations).  The call only enqueues kernels -- no allocation, no
+    # synchronisation, no memset -- so a replay costs the host one graph launch instead of one launch per kernel.
+    graph_replay = None
+    if wall_ms < 0.1:
+        graph_replay = {"steps_per_graph": [], "ms_per_step": []}
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            reuse.aggregate(x, normalized, out=out, feat_dim=feat, pad_columns=pad)
+        torch.cuda.current_stream().wait_stream(side)
+        for per_graph in (1, 8):
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                for _ in range(per_graph):
+                    reuse.aggregate(x, normalized, out=out, feat_dim=feat, pad_columns=pad)
+            replays = max(1, args.steps // per_graph)
+            for _ in range(max(2, replays // 4)):
+                graph.replay()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(replays):
+                graph.replay()
+            torch.cuda.synchronize()
+            graph_replay["steps_per_graph"].append(per_graph)
+            graph_replay["ms_per_step"].append((time.perf_counter() - t0) * 1e3 / (replays * per_graph))
+            del graph
+
     # ---- HIP-event timings on the launch stream; reuse and reuse-disabled alternate so that drift
     # of clocks or temperature hits both alike
     per = max(5, args.steps // 4)
@@ -925,7 +953,7 @@ def main():
         "traffic_source": traffic.get("source", traffic.get("error")),
         "traffic_counter_scale": {"FETCH_SIZE": traffic.get("fetch_scale"), "WRITE_SIZE": traffic.get("write_scale")},
         "layer": {
-            "event_ms": ev_ms, "event_ms_runs": ev_r, "per_call": spread, "launch1_ms": ms_a, "launch2_ms": ms_b,
+            "event_ms": ev_ms, "event_ms_runs": ev_r, "graph_replay": graph_replay, "per_call": spread, "launch1_ms": ms_a, "launch2_ms": ms_b,
             "traffic": layer_traffic,
             "frac_of_hbm_peak": layer_traffic / (ev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS if layer_traffic else None,
             "b_min": b_min, "traffic_over_b_min": layer_traffic / b_min if layer_traffic else None,
