@@ -468,6 +468,25 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
             for (int32_t j = L->group_dst_ptr[g]; j < L->group_dst_ptr[g + 1]; ++j) ng[at[L->group_dst[j]]++] = (int32_t)g;
     }
 
+    // "nearby" = within two tiles of ids, and within a sixteenth of the graph: on a graph of a few tiles every source
+    // is within two tiles, which says nothing about locality (R-MAT, 2^14 ... 2^15 nodes: taken for local, whole
+    // tiles per XCD run cost 12 ... 25 % against runs of 4; a block model of sixteen 4096-node blocks still gains
+    // 23 % from them)
+    const int32_t near_ids = (int32_t)std::max<int64_t>(1, std::min<int64_t>(2 * kTileRows, n / 16));
+    // Do the rows gather from their own neighbourhood (at least half of the sources nearby, every group expanded)?
+    // Then neighbouring rows share sources through the L2 of the XCD that their tile runs on, and a row that a
+    // cluster takes out of the tile order loses that.
+    auto sources_are_local = [&]() {
+        int64_t near = 0, all = (int64_t)L->res_col.size();
+        for (int32_t v = 0; v < n; ++v)
+            for (int32_t j = L->res_ptr[v]; j < L->res_ptr[v + 1]; ++j) near += std::abs(L->res_col[j] - v) < near_ids;
+        for (int64_t g = 0; g < G; ++g)
+            for (int32_t d = L->group_dst_ptr[g]; d < L->group_dst_ptr[g + 1]; ++d)
+                for (int32_t j = L->group_ptr[g]; j < L->group_ptr[g + 1]; ++j, ++all)
+                    near += std::abs(L->group_col[j] - L->group_dst[d]) < near_ids;
+        return all > 0 && near * 2 >= all;
+    };
+
     // Workgroup-local sharing first (cost-model mode only): consumers that the schedule can bring together in one
     // workgroup take the group's sum from LDS; what is decided below for the partial-sum workspace then concerns
     // the remaining consumers only.
@@ -499,8 +518,12 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
         // still fit the 64 KB a workgroup may request (32 would not)
         const int32_t row_bytes = lpr * 16 * ((o && o->elem_bytes == 2) ? 2 : 1);
         const int32_t max_rows = std::max(4, std::min(31, (16 << 10) / row_bytes));
+        // (the relative gate protects the tile order, which only graphs with local sources profit from: on graphs
+        // without it every cluster that saves kMinClusterSaving gathers pays -- planted sets of 3 anchors x 64 members
+        // + 24 random neighbours, 16 % of the gathers removable: 1.056 ms with reuse disabled, 1.082 with the clusters
+        // that pass the relative gate, 0.960 with all of them)
         build_clusters(L, ng_ptr, ng, full_len, std::min(cut, hub_split), groups, max_rows, local_groups > 0 ? local_groups : kMinClusterSaving,
-                       local_groups == 0, cl);
+                       local_groups == 0 && sources_are_local(), cl);
         for (int32_t v = 0; v < n; ++v)
             if (cl.of_node[v] >= 0)
                 for (int32_t j = cl.ptr[cl.of_node[v]]; j < cl.ptr[cl.of_node[v] + 1]; ++j) served[cl.group[j]]++;
@@ -558,11 +581,7 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     tb.out.reserve(n);
     tb.col.reserve(L->res_col.size() + L->group_dst.size());
     int64_t gathered = (int64_t)tg.col.size() + (int64_t)cl.lg_col.size(), reads = 0, segments = 0, nearby = 0, lds_reads = 0;
-    // "nearby" = within two tiles of ids, and within a sixteenth of the graph: on a graph of a few tiles every source
-    // is within two tiles, which says nothing about locality (R-MAT, 2^14 ... 2^15 nodes: taken for local, whole
-    // tiles per XCD run cost 12 ... 25 % against runs of 4; a block model of sixteen 4096-node blocks still gains
-    // 23 % from them)
-    const int32_t near_ids = (int32_t)std::max<int64_t>(1, std::min<int64_t>(2 * kTileRows, n / 16));
+
     ivec row;   // one destination's entries: LDS rows first, then references, then feature rows
     ivec local_row(G, -1);
     for (int32_t v = 0; v < n; ++v) {
