@@ -137,7 +137,8 @@ typedef struct {
                              /* 0 = by the rows a wavefront gathers at once (G = 64 / lanes_per_row) and the    */
                              /* row bytes: float32 rows 128 / 256 (matrix within / beyond 256 MB) at G = 1 and   */
                              /* >= 1024 bytes; otherwise up to G = 3 128 within and 1024 beyond 256 MB; 1024 at   */
-                             /* G = 4; 640 from 5 on; bfloat16 rows 256 for G <= 2, 512 at 3, 1280 above          */
+                             /* G = 4; 640 from 5 on; bfloat16 rows 256 for G <= 2, 512 at 3, 1280 above; lower     */
+                             /* (down to 128) on launches so small that a row of that length would outlast them    */
     int32_t segment;         /* entries per segment; 0 = an eighth to a quarter of hub_split (see layout.cpp)   */
     int32_t lanes_per_row;   /* lanes one gathered row occupies in the kernel that will use this layout:   */
                              /* smallest of 4,8,10,12,16,20,32,64 >= ceil(feat_dim / 4) (fp32) or / 8      */
@@ -151,7 +152,8 @@ typedef struct {
                              /* the default hub_split.                                                              */
     int32_t local_groups;    /* workgroup-local sharing (min_consumers = 0 only): short destinations that consume the */
                              /* same groups are placed in one workgroup, which sums those groups once into LDS;      */
-                             /* 0 = on: a cluster must save 8 row gathers and an eighth of its rows' gathers, and all  */
+                             /* 0 = on: a cluster must save 8 row gathers (on graphs whose rows gather from their own    */
+                             /* neighbourhood also an eighth of its rows' gathers: it gives up the tile order), and all  */
                              /* clusters together 64 MB of gathers; k > 0 = every cluster that saves k; -1 = off      */
     int32_t share_scope;     /* which consumers read a shared group from the workspace: 0 = every consumer; 1 = only rows   */
                              /* long enough to be cut into segments (more than hub_split entries with every group           */
