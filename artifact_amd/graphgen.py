@@ -122,22 +122,27 @@ def sbm_csr(num_blocks, block_size, deg_in, deg_out, seed, self_loops=False):
     return csr_from_pairs(np.concatenate(us), np.concatenate(vs), n, self_loops)
 
 
-def planted_reuse_csr(num_nodes, set_size=12, members_per_set=64, extra_degree=4, seed=0):
+def planted_reuse_csr(num_nodes, set_size=12, members_per_set=64, extra_degree=4, seed=0, memberships=1):
     """Graph with planted common-neighbour structure: nodes come in clubs of `members_per_set`; every
     member of a club is linked to the same `set_size` anchor nodes (consecutive ids, so the chunks of a
     member's sorted neighbour list coincide with those of its club mates), plus `extra_degree` random
-    neighbours.  Symmetric, duplicate-free.  Not one of the upstream-style workloads: it exists to show
-    what the reuse plan buys when a graph does contain shared neighbour subsets."""
+    neighbours.  With `memberships` > 1 every node also joins that many minus one further clubs, drawn by random
+    permutations of the members: its club mates then differ from set to set, so no ordering of the nodes brings all
+    consumers of every set together.  Symmetric, duplicate-free.  Not one of the upstream-style workloads: it exists
+    to show what the reuse plan buys when a graph does contain shared neighbour subsets."""
     rng = np.random.Generator(np.random.PCG64(seed))
     clubs = max(1, num_nodes // (members_per_set + set_size))
     n_anchor = clubs * set_size
     members = np.arange(n_anchor, num_nodes, dtype=np.int64)
-    club = (members - n_anchor) % clubs
-    u = np.repeat(members, set_size)
-    v = (np.repeat(club * set_size, set_size) + np.tile(np.arange(set_size), len(members)))
+    us, vs = [], []
+    for k in range(max(1, memberships)):
+        order = members - n_anchor if k == 0 else rng.permutation(len(members))
+        club = order % clubs
+        us.append(np.repeat(members, set_size))
+        vs.append(np.repeat(club * set_size, set_size) + np.tile(np.arange(set_size), len(members)))
     ru = rng.integers(n_anchor, num_nodes, size=len(members) * extra_degree // 2)
     rv = rng.integers(n_anchor, num_nodes, size=len(ru))
-    return csr_from_pairs(np.concatenate([u, ru]), np.concatenate([v, rv]), num_nodes, False)
+    return csr_from_pairs(np.concatenate(us + [ru]), np.concatenate(vs + [rv]), num_nodes, False)
 
 
 def features(num_nodes, dim, seed, kind="normal"):

@@ -7,7 +7,8 @@ net saving is under a tenth of all row gathers (or under 256 MB) is folded back 
 clusters of destinations that share groups are kept only if they save an eighth of their rows' gathers.  Those gates
 were set on the five workload graphs and one planted-reuse graph.  This check sweeps graphs with planted shared
 neighbour sets from 80 % down to a few per cent of removable gathers (sets of `set_size` anchors shared by
-`members` nodes each, plus `extra` random neighbours per node) and times the same plan (upstream search, part size 3)
+`members` nodes each, plus `extra` random neighbours per node; also nodes that belong to two or three sets with
+different club mates) and times the same plan (upstream search, part size 3)
 four ways, in turn: as the library would run it by default, with reuse disabled, with every shared group forced
 through LDS clusters, and with every group of two or more consumers forced through workspace rows.  The last column
 is the default's time over the best of the four: 1.00 means the gates chose the fastest.  `--workloads` puts the named
@@ -26,9 +27,10 @@ from .graphgen import WORKLOADS, make_workload, planted_reuse_csr
 from .layout import Layout, lanes_per_row
 from .tune_check import time_round_robin
 
-# (set_size, members per set, extra random neighbours per node)
+# (set_size, members per set, extra random neighbours per node[, sets per node: with more than one a node's club mates
+# differ from set to set, so its sets cannot all be shared inside one workgroup])
 CASES = ((12, 64, 4), (12, 64, 24), (12, 8, 24), (12, 2, 12), (6, 64, 24), (6, 4, 24), (3, 64, 24), (3, 64, 48), (3, 4, 24),
-         (3, 2, 24))
+         (3, 2, 24), (12, 8, 12, 2), (6, 16, 12, 2), (3, 16, 24, 2), (3, 64, 24, 3))
 
 
 def check(case, nodes, feat, part_size=3, log=print):
@@ -43,9 +45,10 @@ def check(case, nodes, feat, part_size=3, log=print):
         feat = WORKLOADS[case]["dims"][-1] if case != "c2" else WORKLOADS[case]["dims"][1]
         label = f"workload {case}, {feat} floats, part size {part_size}"
     else:
-        set_size, members, extra = case
-        ip, ix = planted_reuse_csr(nodes, set_size, members, extra, seed=90 + set_size + members + extra)
-        label = f"{set_size} x {members} + {extra}"
+        set_size, members, extra = case[:3]
+        sets = case[3] if len(case) > 3 else 1
+        ip, ix = planted_reuse_csr(nodes, set_size, members, extra, seed=90 + set_size + members + extra, memberships=sets)
+        label = f"{set_size} x {members} + {extra}" + (f", {sets} sets per node" if sets > 1 else "")
     n, e = len(ip) - 1, len(ix)
     plan = R.build_plan(ip, ix, part_size)
     v2 = (plan["uniqpart_column_index"], plan["uniqpart_pointers"], plan["part2Node_ptr"], plan["part2Node_col"], n, part_size)
