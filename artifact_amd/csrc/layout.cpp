@@ -61,6 +61,14 @@ const int64_t kWavesToFill = 2 * 8192;   // two rounds of 256 CUs x 32 wavefront
 // (Giving long rows a whole workgroup instead -- four wavefronts combined through LDS -- was measured as well:
 // no faster than segments on any workload, so it is not built in.)
 const int64_t kCachedMatrixBytes = 256 << 20;   // the Infinity Cache
+// The longest task of a launch is one chain of dependent gathers, measured at (10 + 0.14 x row bytes) ns an entry
+// while the caches serve them; a launch lasts about 15 us + 60 us per GB it gathers.  Entries a chain may have if it
+// is not to outlast 3/4 of the launch:
+int64_t chain_limit(int64_t edges, int64_t row_bytes) {
+    const int64_t launch_ns = 15000 + edges * row_bytes * 60 / 1000000;
+    const int64_t entry_ns = 10 + row_bytes * 14 / 100;
+    return 3 * launch_ns / (4 * entry_ns);
+}
 void default_cut(int32_t groups, int32_t elem_bytes, int64_t row_bytes, int64_t matrix_bytes, int64_t rows, int64_t edges,
                  int32_t &cut, int32_t &segment) {
     const bool cached = matrix_bytes <= kCachedMatrixBytes;
@@ -92,14 +100,10 @@ void default_cut(int32_t groups, int32_t elem_bytes, int64_t row_bytes, int64_t 
         cut = 640;
         segment = 160;
     }
-    // The longest task under the cut is one chain of dependent gathers, measured at (10 + 0.14 x row bytes) ns an
-    // entry while the caches serve them; a launch lasts about 15 us + 60 us per GB it gathers.  Where a chain of
-    // `cut` entries would outlast 3/4 of that, the launch waits for its longest rows (2^17 nodes, average degree 8,
-    // 64 floats: 46.6 us at 1024 / 128, 30.3 at 384 / 96; 2^16 nodes, degree 15: 45.8 against 25.7), so the cut
-    // steps down.
-    const int64_t launch_ns = 15000 + edges * row_bytes * 60 / 1000000;
-    const int64_t entry_ns = 10 + row_bytes * 14 / 100;
-    const int64_t limit = 3 * launch_ns / (4 * entry_ns);
+    // Where a chain of `cut` entries would outlast the launch (chain_limit), the launch waits for its longest rows
+    // (2^17 nodes, average degree 8, 64 floats: 46.6 us at 1024 / 128, 30.3 at 384 / 96; 2^16 nodes, degree 15: 45.8
+    // against 25.7), so the cut steps down.
+    const int64_t limit = chain_limit(edges, row_bytes);
     static const int32_t kLadder[][2] = {{1024, 128}, {640, 160}, {384, 96}, {256, 128}};
     for (const auto &step : kLadder) {
         if (cut <= limit || cut <= 256) break;
@@ -451,6 +455,9 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
                                                   : std::max<int32_t>(16, (int64_t)hub_split * rule_segment / rule_cut);
     L->hub_split = hub_split;
     L->segment = segment;
+    // partial rows are cold when the row that adds them up reads them (written one launch earlier, each read once):
+    // an entry of that chain costs about twice the cached figure, so half as many are allowed
+    const int64_t max_segments = std::max<int64_t>(64, chain_limit(L->e_orig > 0 ? L->e_orig : total, row_bytes) / 2);
     if (o && (o->share_scope < 0 || o->share_scope > 1)) return ROF_ERR_ARG;
     const bool disable = o && o->disable_reuse;
     const int32_t min_consumers = o ? o->min_consumers : 0;
@@ -622,9 +629,13 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
             // A long row is cut into segments; each becomes a partial-sum task of the middle launch
             // (after the groups it may reference, before the rows), and the row itself just adds them up.
             // (Rows served from LDS are short: nlds is 0 here.)
+            // (a row so long that its segments' partial rows would themselves be the longest chain of the launch
+            // gets longer segments: 2^20 nodes with two rows of 2^20 entries at 64 floats, 8192 segments of 128:
+            // 0.82 ms, of which the two rows' own tasks last 0.78; 2048 segments of 512: 0.40 ms)
+            const int64_t seg_len = std::max<int64_t>(segment, (len + max_segments - 1) / max_segments);
             int32_t nseg = 0;
-            for (int64_t s0 = 0; s0 < len; s0 += segment) {
-                int64_t s1 = std::min<int64_t>(len, s0 + segment);
+            for (int64_t s0 = 0; s0 < len; s0 += seg_len) {
+                int64_t s1 = std::min<int64_t>(len, s0 + seg_len);
                 int32_t slot = (int32_t)slots++;
                 ts.begin_task(slot);
                 ts.col.insert(ts.col.end(), row.begin() + s0, row.begin() + s1);

@@ -7,7 +7,7 @@ from helpers import V2_KEYS, emulate_schedule, toy_csr
 
 from artifact_amd import reuse_search_ext as R
 from artifact_amd._lib import RofError
-from artifact_amd.graphgen import make_workload, planted_reuse_csr, rmat_csr, sbm_csr
+from artifact_amd.graphgen import csr_from_pairs, make_workload, planted_reuse_csr, rmat_csr, sbm_csr
 from artifact_amd.layout import Layout
 
 
@@ -270,6 +270,31 @@ def test_small_matrices_keep_the_fine_cut():
                              (16, 0, (1024, 128)), (64, 1024, (128, 32)), (64, 2048, (256, 32))):
         ex = Layout.from_csr(ip, ix, lanes_per_row=lanes, row_bytes=row).export()
         assert (ex["hub_split"], ex["segment"]) == want, (lanes, row)
+
+
+def test_a_row_of_the_whole_graph_gets_longer_segments():
+    """The row that adds up a long row's partial sums is itself a chain of dependent reads, one per segment; a row
+    so long that this chain would outlast the launch is cut into fewer, longer segments: at most
+    max(64, chain limit / 2) of them (partial rows are read cold, at about twice the cached cost per entry)."""
+    n = 20000
+    rng = np.random.default_rng(4)
+    u, v = rng.integers(1, n, 2 * n), rng.integers(1, n, 2 * n)
+    ip, ix = csr_from_pairs(np.r_[u, np.zeros(n - 1, np.int64)], np.r_[v, np.arange(1, n)], n, False)
+    assert np.diff(ip)[0] == n - 1                           # node 0 is everybody's neighbour
+    lay = Layout.from_csr(ip, ix, lanes_per_row=16)
+    ex, st = lay.export(), lay.stats()
+    limit = 3 * (15000 + len(ix) * 256 * 60 // 1000000) // (4 * (10 + 256 * 14 // 100))
+    most = max(64, limit // 2)
+    assert st["segment"] * most < n - 1                      # the rule's segments would be too many
+    s_len = np.diff(ex["s_task_ptr"])
+    hub = int(np.nonzero(ex["b_task_out"] == 0)[0][0])
+    assert ex["b_task_nref"][hub] == np.diff(ex["b_task_ptr"])[hub] <= most
+    assert s_len.max() == -(-(n - 1) // most) and st["longest_row_task"] <= max(st["hub_split"], most)
+    x = np.random.default_rng(5).standard_normal((n, 2))
+    got = emulate_schedule(ex, n, x, lambda c: 1.0, lambda r: 1.0, st["partial_rows"])
+    want = np.zeros((n, 2))
+    np.add.at(want, np.repeat(np.arange(n), np.diff(ip)), x[ix])
+    assert np.allclose(got, want, rtol=1e-11, atol=1e-11)
 
 
 def test_the_relative_cluster_gate_applies_only_to_graphs_with_local_sources():
