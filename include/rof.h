@@ -139,7 +139,8 @@ typedef struct {
                              /* >= 1024 bytes; otherwise up to G = 3 128 within and 1024 beyond 256 MB; 1024 at   */
                              /* G = 4; 640 from 5 on; bfloat16 rows 256 for G <= 2, 512 at 3, 1280 above; lower     */
                              /* (down to 128) on launches so small that a row of that length would outlast them    */
-    int32_t segment;         /* entries per segment; 0 = an eighth to a quarter of hub_split (see layout.cpp)   */
+    int32_t segment;         /* entries per segment; 0 = an eighth to a quarter of hub_split (see layout.cpp).  A row  */
+                             /* so long that adding up its segments would outlast the launch gets longer ones.    */
     int32_t lanes_per_row;   /* lanes one gathered row occupies in the kernel that will use this layout:   */
                              /* smallest of 4,8,10,12,16,20,32,64 >= ceil(feat_dim / 4) (fp32) or / 8      */
                              /* (bf16); 0 = 16.  Steers the default hub_split and the sharing gate.        */
