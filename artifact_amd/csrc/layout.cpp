@@ -449,6 +449,64 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     int32_t rule_cut = 0, rule_segment = 0;
     default_cut(groups, elem_bytes, row_bytes, (int64_t)n * row_bytes, n, L->e_orig > 0 ? L->e_orig : total, rule_cut,
                 rule_segment);
+    // entries of every destination with every group expanded
+    ivec len_all((size_t)n);
+    {
+        std::vector<int64_t> len((size_t)n);
+        for (int32_t v = 0; v < n; ++v) len[v] = L->res_ptr[v + 1] - L->res_ptr[v];
+        for (int64_t g = 0; g < G; ++g)
+            for (int32_t j = L->group_dst_ptr[g]; j < L->group_dst_ptr[g + 1]; ++j)
+                len[L->group_dst[j]] += L->group_ptr[g + 1] - L->group_ptr[g];
+        for (int32_t v = 0; v < n; ++v) len_all[v] = (int32_t)std::min<int64_t>(len[v], INT32_MAX);
+    }
+    // Dense graphs.  The segments of a row of `len` entries each gather from a band of segment / len of the matrix,
+    // and the swept launch keeps such bands in L2 where a whole row, gathered as one task, ranges over the entire
+    // matrix: rows long enough for bands of a few MB at 64 entries per segment (16 entries per MB of matrix) are
+    // worth cutting even below the rule's cut -- when they hold a quarter of the edges and are half of all rows, on a
+    // matrix several times the size of an L2 (uniform degrees of 600, 2^17 nodes: 24 floats 1.35 ms at 640 / 160 against 0.61 at 128 / 64, 47
+    // floats 2.13 against 0.86, 128 bf16 2.15 against 1.16; sparse graphs lose 4-5 % with the lower cut and do not
+    // meet the condition).
+    const int64_t matrix_mb = (int64_t)n * row_bytes >> 20;
+    const int32_t sweep_cut = (int32_t)std::max<int64_t>(128, 16 * matrix_mb);
+    if (groups >= 4 && matrix_mb >= 8 && sweep_cut < rule_cut) {
+        int64_t between = 0, all = 0, long_rows = 0;
+        for (int32_t v = 0; v < n; ++v) {
+            all += len_all[v];
+            long_rows += len_all[v] > sweep_cut;
+            if (len_all[v] > sweep_cut && len_all[v] <= rule_cut) between += len_all[v];
+        }
+        // (... and when the typical row is that long: where most rows are short and a minority holds the edges,
+        // those rows are also the popular sources, which stay in L2 without a sweep, and coarser segments win:
+        // R-MAT 2^16 nodes, average degree 341, 128 bf16: 0.341 ms at 256 / 64 against 0.303 at 1280 / 320)
+        if (between * 4 >= all && long_rows * 2 >= n) {
+            rule_cut = sweep_cut;
+            rule_segment = 64;
+        }
+    }
+    // Dense graphs with popular sources.  The fine cut of the wide rows (128 / 32 up to three rows per wavefront on a
+    // matrix that the caches hold) was measured on graphs of average degree 14, where a few hub rows are cut and
+    // fine segments balance them.  Where two thirds of all edges lie in rows beyond that cut, the segments are the
+    // launch, and 32 entries are too few for a task that costs a wavefront, a partial row written and read, and
+    // three dependent loads before its first gather (R-MAT 2^18 nodes, average degree 83, 160 floats: 1.15 ms at
+    // 128 / 32, 0.89 at 128 / 64, 0.86 at 128 / 128, 0.79 at 512 / 128, 0.75 at 1024 / 128; 2^16 nodes, degree 341:
+    // 0.87 / 0.72 at 512 / 128; 512 / 128 is at or within 6 % of the best of seven choices on the nine dense graphs
+    // measured at 72, 100 and 160 floats).  Not so when the typical row is long (uniform degrees of 600: 2.95 ms at 128 / 32, 5.08 at 128 / 128):
+    // there no source is popular enough to stay in L2 by itself and the narrow bands of fine segments are what hits.
+    if (elem_bytes == 4 && groups <= 3 && rule_cut == 128 && rule_segment == 32) {
+        int64_t beyond = 0, all = 0, long_rows = 0;
+        for (int32_t v = 0; v < n; ++v) {
+            all += len_all[v];
+            long_rows += len_all[v] > rule_cut;
+            if (len_all[v] > rule_cut) beyond += len_all[v];
+        }
+        if (beyond * 3 >= all * 2 && long_rows * 2 < n) {
+            // (rows of 1 KB: 256 / 64 is within 4 % of the best on the four dense graphs measured at 256 floats,
+            // 1024 / 128 up to 14 % behind and 128 / 32 up to 22 %)
+            const bool wide = groups == 1 && row_bytes >= 1024;
+            rule_cut = wide ? 256 : 512;
+            rule_segment = wide ? 64 : 128;
+        }
+    }
     const int32_t hub_split = (o && o->hub_split > 0) ? o->hub_split : rule_cut;
     // (a caller's cut with the library's segment: the rule's share of the rule's cut)
     const int32_t segment = (o && o->segment > 0) ? o->segment
@@ -502,14 +560,12 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     const int32_t local_groups = o ? o->local_groups : 0;
     const int32_t share_scope = o ? o->share_scope : 0;
     ivec served(G, 0);   // consumers of each group that read it from LDS
-    ivec full_len;       // entries of every destination with every group expanded
+    ivec full_len;       // entries of every destination with every group expanded (only needed where groups exist)
     int64_t over = 0;    // destinations whose task, as cut by hub_split, is a long one
     if (G > 0) {
-        full_len.resize(n);
+        full_len.swap(len_all);
         for (int32_t v = 0; v < n; ++v) {
-            int64_t len = L->res_ptr[v + 1] - L->res_ptr[v];
-            for (int32_t j = ng_ptr[v]; j < ng_ptr[v + 1]; ++j) len += L->group_ptr[ng[j] + 1] - L->group_ptr[ng[j]];
-            full_len[v] = (int32_t)std::min<int64_t>(len, INT32_MAX);
+            const int64_t len = full_len[v];
             const int64_t task_len = len > hub_split ? (len + segment - 1) / segment : len;
             over += task_len > kShortRow;
         }

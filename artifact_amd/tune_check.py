@@ -2,7 +2,7 @@
 own choice of wavefront cap, XCD run, row gathers in flight and long-row cut within a few per cent of the best of
 the alternatives?
 
-    python -m artifact_amd.tune_check [--graphs h1,...,h7] [--out table.md]
+    python -m artifact_amd.tune_check [--graphs h1,...,h9] [--out table.md]
 
 For every (graph, width) one aggregation layer (no reuse plan: `Layout.from_csr`) is timed with the default layout
 and launch settings and then with one setting changed at a time: wavefronts per SIMD of the destination-row launch
@@ -39,6 +39,9 @@ GRAPHS = {
     "h5": ("R-MAT a=.5 b=c=.2, 2^16 nodes, average degree 24", lambda: rmat_csr(1 << 16, 24, 75, a=0.5, b=0.2, c=0.2)),
     "h6": ("R-MAT a=.62 b=c=.16, 2^15 nodes, average degree 12", lambda: rmat_csr(1 << 15, 12, 76, a=0.62, b=0.16, c=0.16)),
     "h7": ("R-MAT a=.55 b=.25 c=.15, 2^17 nodes, average degree 6", lambda: rmat_csr(1 << 17, 6, 77, a=0.55, b=0.25, c=0.15)),
+    # dense graphs: every row is near or beyond the long-row cut
+    "h8": ("uniform degrees (600 random partners per node), 2^17 nodes", lambda: uniform_degree_csr(1 << 17, 600, 78)),
+    "h9": ("R-MAT a=.5 b=c=.2, 2^16 nodes, average degree 400", lambda: rmat_csr(1 << 16, 400, 79, a=0.5, b=0.2, c=0.2)),
 }
 WIDTHS = ((24, False), (72, False), (160, False), (128, True))
 

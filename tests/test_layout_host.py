@@ -209,13 +209,14 @@ def test_random_graphs_with_shared_neighbour_sets_through_clusters(oracle, seed)
 
 
 @pytest.mark.parametrize("lanes,elem,row,cut,seg", [(64, 4, 0, 256, 32), (64, 4, 1024, 256, 32), (64, 4, 640, 1024, 128),
-                                                    (32, 4, 0, 1024, 128), (20, 4, 0, 128, 32), (16, 4, 0, 1024, 128),
+                                                    (32, 4, 0, 1024, 128), (20, 4, 0, 512, 128), (16, 4, 0, 1024, 128),
                                                     (12, 4, 0, 640, 160), (8, 0, 0, 640, 160),
                                                     (32, 2, 0, 256, 48), (20, 2, 0, 512, 128), (16, 2, 0, 1280, 320)])
 def test_long_rows_are_cut_by_width_and_their_segments_swept_by_source_id(lanes, elem, row, cut, seg):
     """Default cut and segment by the rows a wavefront gathers at once, the bytes of a row and whether the caches
     can hold the matrix (the measured table in csrc/layout.cpp; this 600 000-row matrix is beyond them at 32 lanes
-    and more); the segment tasks come in the order of the highest source id they gather (each task lists its sources
+    and more, and at 20 lanes, where they hold it, two thirds of its edges lie in rows beyond the fine cut of 128: the
+    dense rule's 512 / 128); the segment tasks come in the order of the highest source id they gather (each task lists its sources
     by descending id), long tasks before packed ones."""
     ip, ix = make_workload("c4", 2)                          # 600 000 rows: enough segments to fill the machine
     n = len(ip) - 1
@@ -311,6 +312,38 @@ def test_the_relative_cluster_gate_applies_only_to_graphs_with_local_sources():
     assert default == every > 8000
     default, every = clusters(*sbm_csr(64, 4096, 24, 2, 6), 2)
     assert default == 0 and every > 2000
+
+
+def test_dense_graphs_are_cut_by_what_their_rows_look_like():
+    """Two rules for dense graphs.  (1) Up to three rows per wavefront on a matrix that the caches hold: the fine cut
+    128 / 32 suits graphs whose few hub rows it balances; where two thirds of the edges lie beyond it, the segments
+    are the launch and take 512 / 128 (256 / 64 for rows of 1 KB) -- unless the typical row is that long, in which case
+    no source is popular and only the narrow bands of fine segments hit in L2.  (2) From four rows per wavefront, when
+    half of the rows are longer than 16 entries per MB of matrix and those below the rule's cut hold a quarter of the
+    edges, the cut comes down to them (segments of 64), so that they are swept."""
+    def cut_of(ip, ix, **kw):
+        st = Layout.from_csr(ip, ix, **kw).stats()
+        return st["hub_split"], st["segment"]
+    ip, ix = rmat_csr(1 << 16, 100, seed=81)                 # dense and skewed: 80 % of the edges in rows > 128
+    deg = np.diff(ip)
+    assert deg[deg > 128].sum() * 3 >= len(ix) * 2 and (deg > 128).sum() * 2 < len(deg)
+    assert cut_of(ip, ix, lanes_per_row=32) == (512, 128) and cut_of(ip, ix, lanes_per_row=20) == (512, 128)
+    assert cut_of(ip, ix, lanes_per_row=64, row_bytes=640) == (512, 128)
+    assert cut_of(ip, ix, lanes_per_row=64, row_bytes=1024) == (256, 64)
+    ip, ix = make_workload("c2", 2)                          # average degree 14: half of the edges beyond 128
+    assert cut_of(ip, ix, lanes_per_row=32) == (128, 32) and cut_of(ip, ix, lanes_per_row=64, row_bytes=1024) == (128, 32)
+    u = np.repeat(np.arange(1 << 15), 150)                   # uniform degrees around 300: every row beyond 128
+    ip, ix = csr_from_pairs(u, np.random.default_rng(3).integers(0, 1 << 15, len(u)), 1 << 15, False)
+    assert np.diff(ip).min() > 200
+    assert cut_of(ip, ix, lanes_per_row=32) == (128, 32)     # the typical row is long: fine segments
+    assert cut_of(ip, ix, lanes_per_row=8) == (256, 128)     # 4 MB: an L2 holds the matrix, the small-launch cut stays
+    # (2): 2^17 rows x 128 bytes = 16 MB -> rows beyond 256 entries are worth sweeping, and every row has about 300
+    u = np.repeat(np.arange(1 << 17), 150)
+    ip, ix = csr_from_pairs(u, np.random.default_rng(4).integers(0, 1 << 17, len(u)), 1 << 17, False)
+    deg = np.diff(ip)
+    assert (deg > 256).sum() > 0.99 * len(deg) and deg.max() < 640
+    assert cut_of(ip, ix, lanes_per_row=8) == (256, 64)      # the table alone says 640 / 160: no row would be cut
+    assert cut_of(ip, ix, lanes_per_row=8, disable_reuse=True, hub_split=640)[0] == 640   # a caller's cut stands
 
 
 def test_small_launches_cut_long_rows_lower():
