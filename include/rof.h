@@ -138,7 +138,8 @@ typedef struct {
                              /* row bytes: float32 rows 128 / 256 (matrix within / beyond 256 MB) at G = 1 and   */
                              /* >= 1024 bytes; otherwise up to G = 3 128 within and 1024 beyond 256 MB; 1024 at   */
                              /* G = 4; 640 from 5 on; bfloat16 rows 256 for G <= 2, 512 at 3, 1280 above; lower     */
-                             /* (down to 128) on launches so small that a row of that length would outlast them    */
+                             /* (down to 128) on launches so small that a row of that length would outlast them,   */
+                             /* and adjusted on dense graphs by what their rows look like (see layout.cpp)          */
     int32_t segment;         /* entries per segment; 0 = an eighth to a quarter of hub_split (see layout.cpp).  A row  */
                              /* so long that adding up its segments would outlast the launch gets longer ones.    */
     int32_t lanes_per_row;   /* lanes one gathered row occupies in the kernel that will use this layout:   */
