@@ -61,6 +61,7 @@ const int64_t kWavesToFill = 2 * 8192;   // two rounds of 256 CUs x 32 wavefront
 // (Giving long rows a whole workgroup instead -- four wavefronts combined through LDS -- was measured as well:
 // no faster than segments on any workload, so it is not built in.)
 const int64_t kCachedMatrixBytes = 256 << 20;   // the Infinity Cache
+const int64_t kL2Bytes = 4 << 20;               // of one XCD
 // The longest task of a launch is one chain of dependent gathers, measured at (10 + 0.14 x row bytes) ns an entry
 // while the caches serve them; a launch lasts about 15 us + 60 us per GB it gathers.  Entries a chain may have if it
 // is not to outlast 3/4 of the launch:
@@ -537,7 +538,10 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     // is within two tiles, which says nothing about locality (R-MAT, 2^14 ... 2^15 nodes: taken for local, whole
     // tiles per XCD run cost 12 ... 25 % against runs of 4; a block model of sixteen 4096-node blocks still gains
     // 23 % from them)
-    const int32_t near_ids = (int32_t)std::max<int64_t>(1, std::min<int64_t>(2 * kTileRows, n / 16));
+    // (and as far as the rows go that one L2 holds: 16 partners within 32 768 ids on 2^21 nodes at 24 floats, where 4
+    // MB are 43 690 rows, run 43 % faster with whole tiles per XCD run than with runs of 4; at 72 floats 9 %)
+    const int32_t near_ids = (int32_t)std::max<int64_t>(
+        1, std::min<int64_t>(std::max<int64_t>(2 * kTileRows, kL2Bytes / std::max<int64_t>(1, row_bytes)), n / 16));
     // Do the rows gather from their own neighbourhood (at least half of the sources nearby, every group expanded)?
     // Then neighbouring rows share sources through the L2 of the XCD that their tile runs on, and a row that a
     // cluster takes out of the tile order loses that.

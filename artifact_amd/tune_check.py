@@ -2,7 +2,7 @@
 own choice of wavefront cap, XCD run, row gathers in flight and long-row cut within a few per cent of the best of
 the alternatives?
 
-    python -m artifact_amd.tune_check [--graphs h1,...,h9] [--out table.md]
+    python -m artifact_amd.tune_check [--graphs h1,...,h11] [--out table.md]
 
 For every (graph, width) one aggregation layer (no reuse plan: `Layout.from_csr`) is timed with the default layout
 and launch settings and then with one setting changed at a time: wavefronts per SIMD of the destination-row launch
@@ -30,6 +30,22 @@ def uniform_degree_csr(num_nodes, degree, seed):
     return csr_from_pairs(u, v, num_nodes, False)
 
 
+def grid_csr(rows, cols):
+    """4-neighbour grid, ids row-major: every source is 1 or `cols` ids away."""
+    ids = np.arange(rows * cols, dtype=np.int64).reshape(rows, cols)
+    u = np.concatenate([ids[:, :-1].ravel(), ids[:-1, :].ravel()])
+    v = np.concatenate([ids[:, 1:].ravel(), ids[1:, :].ravel()])
+    return csr_from_pairs(u, v, rows * cols, False)
+
+
+def banded_csr(num_nodes, degree, band, seed):
+    """`degree` / 2 random partners per node within `band` ids of it (a nearest-neighbour graph of sorted points)."""
+    rng = np.random.Generator(np.random.PCG64(seed))
+    u = np.repeat(np.arange(num_nodes, dtype=np.int64), degree // 2)
+    v = (u + rng.integers(-band, band + 1, size=len(u))) % num_nodes
+    return csr_from_pairs(u, v, num_nodes, False)
+
+
 GRAPHS = {
     "h1": ("R-MAT a=.45 b=c=.22, 2^21 nodes, average degree 8", lambda: rmat_csr(1 << 21, 8, 71, a=0.45, b=0.22, c=0.22)),
     "h2": ("R-MAT a=.65 b=c=.15, 2^20 nodes, average degree 48", lambda: rmat_csr(1 << 20, 48, 72, a=0.65, b=0.15, c=0.15)),
@@ -42,6 +58,9 @@ GRAPHS = {
     # dense graphs: every row is near or beyond the long-row cut
     "h8": ("uniform degrees (600 random partners per node), 2^17 nodes", lambda: uniform_degree_csr(1 << 17, 600, 78)),
     "h9": ("R-MAT a=.5 b=c=.2, 2^16 nodes, average degree 400", lambda: rmat_csr(1 << 16, 400, 79, a=0.5, b=0.2, c=0.2)),
+    # very sparse graphs with local structure
+    "h10": ("4-neighbour grid 2048 x 2048", lambda: grid_csr(2048, 2048)),
+    "h11": ("16 random partners within 32768 ids, 2^21 nodes", lambda: banded_csr(1 << 21, 16, 1 << 15, 80)),
 }
 WIDTHS = ((24, False), (72, False), (160, False), (128, True))
 
