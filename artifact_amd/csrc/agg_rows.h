@@ -462,6 +462,37 @@ __global__ __launch_bounds__(256) void rof_rows_kernel(AggArgs a) {
     }
 }
 
+// Add the LDS rows of one clustered task (their numbers are the first `nlds` entries of its list) into acc.  The
+// numbers are fetched LPR at a time, one by each lane of the lane group, and handed round: one memory latency per LPR
+// rows instead of one per row.  EARLY: `mine0` holds the first LPR numbers, requested by the caller beforehand.
+template <int VEC, int LPR, bool EARLY>
+__device__ __forceinline__ void add_lds_rows(const float *lds_rows, const int32_t *__restrict__ col, int32_t first, int32_t nlds,
+                                             int32_t mine0, int sub, int li, float (&acc)[VEC]) {
+    constexpr int kLdsRow = LPR * VEC + 4;
+    if constexpr (!EARLY && LPR < 10) {   // (bf16 at 16 and 8 rows per wavefront: the hand-off would cost a wavefront)
+        for (int j = 0; j < nlds; ++j) {
+            const float *row = lds_rows + col[first + j] * kLdsRow + li * VEC;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) acc[k] += row[k];
+        }
+        return;
+    }
+#pragma unroll 1
+    for (int j0 = 0; __any(j0 < nlds); j0 += LPR) {
+        const int32_t mine = (EARLY && j0 == 0) ? mine0 : (j0 + li < nlds) ? col[first + j0 + li] : 0;
+#pragma unroll
+        for (int j = 0; j < LPR; ++j) {
+            if (!__any(j0 + j < nlds)) break;
+            const int32_t r = __builtin_amdgcn_ds_bpermute(lane_addr(sub * LPR * 4, j * 4), mine);
+            if (j0 + j < nlds) {
+                const float *row = lds_rows + r * kLdsRow + li * VEC;
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) acc[k] += row[k];
+            }
+        }
+    }
+}
+
 // The launch of the clustered destinations (PHASE >= 1 only).  Workgroup i holds cluster i: destinations that share
 // reuse groups.  It first sums its local groups lg_ptr[i] .. lg_ptr[i+1] into LDS rows, one lane group per group,
 // then works through its own list of short tasks (lg_task_first[i] .. lg_task_first[i+1], in rounds of 4 * G), and
@@ -522,10 +553,15 @@ __global__ __launch_bounds__(256) void rof_cluster_kernel(AggArgs a) {
         for (int32_t t0 = ct0 + wid * G; t0 < ct1; t0 += kWavesPerBlock * G) {   // one lane group per task
             const int32_t t = t0 + sub;
             const bool valid = !idle && t < ct1;
-            int32_t first = 0, beg = 0, mid = 0, end = 0, nlds = 0;
+            int32_t first = 0, beg = 0, mid = 0, end = 0, nlds = 0, out_row = 0;
+            float out_scale = 1.0f;
             if (valid) {
                 first = a.task_ptr[t];
                 end = a.task_ptr[t + 1];
+                if constexpr (kF32) {   // with the task's range, not after its sum: one latency less before the store
+                    out_row = a.task_out[t];   // (the bf16 instantiations would pay for the two registers with a wavefront)
+                    if (a.task_scale) out_scale = a.task_scale[t];
+                }
                 const uint32_t packed = (uint32_t)a.task_nref[t];   // references in the low 24 bits, LDS rows above
                 nlds = (int32_t)(packed >> 24);
                 beg = first + nlds;
@@ -534,11 +570,11 @@ __global__ __launch_bounds__(256) void rof_cluster_kernel(AggArgs a) {
             float acc[VEC];
 #pragma unroll
             for (int k = 0; k < VEC; ++k) acc[k] = 0.0f;
-            for (int j = 0; j < nlds; ++j) {
-                const float *row = lds_rows + a.col[first + j] * kLdsRow + li * VEC;
-#pragma unroll
-                for (int k = 0; k < VEC; ++k) acc[k] += row[k];
-            }
+            // fp32: the numbers of the first LPR LDS rows are requested before the row gathers what it does not share,
+            // and the rows added after it, by when the numbers have long arrived (the bf16 instantiations would pay for
+            // that order with a wavefront per SIMD and add their LDS rows first)
+            const int32_t mine0 = (kF32 && li < nlds) ? a.col[first + li] : 0;
+            if constexpr (!kF32) add_lds_rows<VEC, LPR, false>(lds_rows, a.col, first, nlds, mine0, sub, li, acc);
             if (kF32) {
                 if (__any(mid > beg))
                     gather_sum<XT, VEC, LPR, false, true, OFF32, PHASE == 2>(xb, xld, pb, pld, a.nsplit, 0, a.col, a.w, beg, end,
@@ -553,9 +589,14 @@ __global__ __launch_bounds__(256) void rof_cluster_kernel(AggArgs a) {
                 gather_sum<XT, VEC, LPR, false, false, OFF32, PHASE == 2>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, mid, end, lane,
                                                                          sub, li, act, acc);
             }
-            if (valid && act)
-                finish_row<XT, VEC, PHASE>(a, a.task_out[t], (a.task_scale && end > first) ? a.task_scale[t] : 1.0f, end > first, acc,
-                                           xb, xld, cstart, skip);
+            if constexpr (kF32) add_lds_rows<VEC, LPR, true>(lds_rows, a.col, first, nlds, mine0, sub, li, acc);
+            if constexpr (!kF32) {
+                if (valid && act) {
+                    out_row = a.task_out[t];
+                    if (a.task_scale && end > first) out_scale = a.task_scale[t];
+                }
+            }
+            if (valid && act) finish_row<XT, VEC, PHASE>(a, out_row, out_scale, end > first, acc, xb, xld, cstart, skip);
         }
     }
 }
