@@ -81,7 +81,7 @@ def _opts(min_consumers=0, disable_reuse=False, hub_split=0, segment=0, lanes_pe
 
 
 # (cut, segment) candidates that an autotuned family times against the rule's choice, by element size
-CUT_CANDIDATES = {4: ((128, 32), (512, 64), (1024, 128)), 2: ((256, 48), (256, 128), (640, 160), (1280, 320))}
+CUT_CANDIDATES = {4: ((128, 32), (512, 64), (1024, 128), (2048, 256)), 2: ((256, 48), (256, 128), (640, 160), (1280, 320))}
 
 
 def autotune_default():

@@ -2,7 +2,7 @@
 own choice of wavefront cap, XCD run, row gathers in flight and long-row cut within a few per cent of the best of
 the alternatives?
 
-    python -m artifact_amd.tune_check [--graphs h1,...,h11] [--out table.md]
+    python -m artifact_amd.tune_check [--graphs h1,...,h12] [--out table.md]
 
 For every (graph, width) one aggregation layer (no reuse plan: `Layout.from_csr`) is timed with the default layout
 and launch settings and then with one setting changed at a time: wavefronts per SIMD of the destination-row launch
@@ -46,6 +46,16 @@ def banded_csr(num_nodes, degree, band, seed):
     return csr_from_pairs(u, v, num_nodes, False)
 
 
+def bipartite_csr(users, items, per_user, seed):
+    """Users (ids 0 .. users-1) each link to `per_user` items (ids users ..), item popularity ~ 1 / rank: two kinds of
+    rows, short user rows that gather from a small popular set and long item rows that gather from everywhere."""
+    rng = np.random.Generator(np.random.PCG64(seed))
+    u = np.repeat(np.arange(users, dtype=np.int64), per_user)
+    p = 1.0 / np.arange(1, items + 1)
+    v = users + rng.choice(items, size=len(u), p=p / p.sum())
+    return csr_from_pairs(u, v, users + items, False)
+
+
 GRAPHS = {
     "h1": ("R-MAT a=.45 b=c=.22, 2^21 nodes, average degree 8", lambda: rmat_csr(1 << 21, 8, 71, a=0.45, b=0.22, c=0.22)),
     "h2": ("R-MAT a=.65 b=c=.15, 2^20 nodes, average degree 48", lambda: rmat_csr(1 << 20, 48, 72, a=0.65, b=0.15, c=0.15)),
@@ -61,6 +71,7 @@ GRAPHS = {
     # very sparse graphs with local structure
     "h10": ("4-neighbour grid 2048 x 2048", lambda: grid_csr(2048, 2048)),
     "h11": ("16 random partners within 32768 ids, 2^21 nodes", lambda: banded_csr(1 << 21, 16, 1 << 15, 80)),
+    "h12": ("bipartite: 2^20 users x 16 of 2^15 items, popularity 1 / rank", lambda: bipartite_csr(1 << 20, 1 << 15, 16, 81)),
 }
 WIDTHS = ((24, False), (72, False), (160, False), (128, True))
 
