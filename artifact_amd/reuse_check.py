@@ -20,8 +20,6 @@ import argparse
 import sys
 import time
 
-import numpy as np
-
 from . import reuse_search_ext as R
 from .graphgen import WORKLOADS, make_workload, planted_reuse_csr
 from .layout import Layout, lanes_per_row
@@ -80,7 +78,7 @@ def check(case, nodes, feat, part_size=3, log=print):
         f"{100 * removable:.1f} %, default runs {how}: " + ", ".join(f"{k} {v:.4f}" for k, v in res.items())
         + f" ms; best {best}; default / best {res['default'] / res[best]:.3f} ({time.time() - t0:.0f} s)")
     return dict(case=case, label=label, n=n, e=e, removable=removable, how=how, res=res, best=best, ratio=res["default"] / res[best],
-                groups=int(len(plan["index_picked"]) if "index_picked" in plan else 0), max_diff=worst,
+                max_diff=worst,
                 lds_reads=d["lds_reads"], materialised=d["materialised_groups"])
 
 
