@@ -12,8 +12,8 @@ pytestmark = pytest.mark.gpu
 torch = pytest.importorskip("torch")
 
 from artifact_amd import reuse_search_ext as R            # noqa: E402
-from artifact_amd.graphgen import features, make_workload  # noqa: E402
-from artifact_amd.layout import Layout                     # noqa: E402
+from artifact_amd.graphgen import csr_from_pairs, features, make_workload  # noqa: E402
+from artifact_amd.layout import Layout, lanes_per_row      # noqa: E402
 from artifact_amd._lib import RofError                     # noqa: E402
 from helpers import close_fp32, strict_excess              # noqa: E402
 
@@ -95,6 +95,39 @@ def test_sum_aggregation_unnormalised(oracle):
     got = lay.aggregate(torch.from_numpy(x).cuda(), normalized=False).cpu().numpy()
     want = oracle.closed_form(indptr, indices, x, normalized=False)
     _close(got, want, oracle.closed_form(indptr, indices, np.abs(x), normalized=False))
+
+
+@pytest.mark.parametrize("kind,feat,bf16", [("dense", 24, False), ("dense", 64, True), ("hub", 64, False), ("hub", 32, False)])
+def test_dense_graphs_and_rows_of_the_whole_graph(oracle, kind, feat, bf16):
+    """The schedules that the degree statistics change: a graph whose typical row is long (every row cut and swept)
+    and a row adjacent to every node (fewer, longer segments), default layouts, normalised, against the float64
+    closed form; bf16 inputs are compared on the values they round to."""
+    rng = np.random.default_rng(11)
+    if kind == "dense":
+        n = 1 << 17
+        u = np.repeat(np.arange(n), 150)
+        indptr, indices = csr_from_pairs(u, rng.integers(0, n, len(u)), n, False)
+    else:
+        n = 300_000
+        u, v = rng.integers(1, n, 2 * n), rng.integers(1, n, 2 * n)
+        indptr, indices = csr_from_pairs(np.r_[u, np.zeros(n - 1, np.int64)], np.r_[v, np.arange(1, n)], n, False)
+    lay = Layout.from_csr(indptr, indices, lanes_per_row=lanes_per_row(feat, bf16), elem_bytes=2 if bf16 else 4,
+                          row_bytes=feat * (2 if bf16 else 4))
+    st = lay.stats()
+    if kind == "dense":
+        assert (np.diff(indptr) > st["hub_split"]).mean() > 0.9 and st["hub_segments"] > n   # nearly every row is cut
+    else:
+        assert st["longest_row_task"] < (n - 1) // st["segment"]                       # longer segments for row 0
+    deg = torch.from_numpy(np.diff(indptr).astype(np.float32)).cuda()
+    lay.set_degrees(deg)
+    x = features(n, feat, seed=12)
+    xt = torch.from_numpy(x).cuda()
+    if bf16:
+        xt = xt.to(torch.bfloat16)
+        x = xt.float().cpu().numpy()
+    got = lay.aggregate(xt, normalized=True).cpu().numpy()
+    want = oracle.closed_form(indptr, indices, x, np.diff(indptr).astype(np.float32))
+    _close(got, want, oracle.closed_form(indptr, indices, np.abs(x), np.diff(indptr).astype(np.float32)))
 
 
 @pytest.mark.parametrize("feat,ld,shift", [(47, 47, 0), (5, 5, 0), (7, 9, 1), (101, 101, 3), (255, 255, 0), (2, 2, 1)])
