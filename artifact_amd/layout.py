@@ -101,13 +101,20 @@ class LayoutFamily:
     GPU builds the rule's layout and the candidates of CUT_CANDIDATES, times one aggregation of random rows of that
     width with each (HIP events, two rounds in turn), keeps the fastest and lets it choose its launch settings by
     timing too (`Layout.calibrate`); `chosen[key]` records what was taken.  That costs a few layout builds and a few
-    dozen aggregations per width class, once."""
+    dozen aggregations per width class, once.  `choices` (what `choices()` of an earlier family returned, e.g. read back
+    from a saved plan) replays recorded decisions instead of timing: the same cut, segment and launch settings, hence
+    the same summation order and the same bits as the run that made them."""
 
-    def __init__(self, build, autotune=None):
+    def __init__(self, build, autotune=None, choices=None):
         self._build = build
         self._by_lpr = {}
         self.autotune = autotune_default() if autotune is None else bool(autotune)
         self.chosen = {}
+        self._replay = {}
+        for k, v in (choices or {}).items():
+            key = tuple(int(p) for p in k.split(",")) if isinstance(k, str) else tuple(k)
+            self._replay[key] = {"cut": int(v["cut"]), "segment": int(v["segment"]),
+                                 "tuning": {n: int(x) for n, x in v.get("tuning", {}).items()}}
         try:
             import inspect
 
@@ -130,11 +137,25 @@ class LayoutFamily:
         key = (lpr, eb, rb)
         lay = self._by_lpr.get(key)
         if lay is None:
-            lay = self._make(key)
-            if self.autotune and self._nargs >= 3 and self._kw:
-                lay = self._autotune(key, lay, int(feat_dim), bool(bf16), bool(normalized))
+            rec = self._replay.get(key)
+            if rec is not None and self._nargs >= 3 and self._kw:
+                lay = self._make(key, hub_split=rec["cut"], segment=rec["segment"])
+                lay.set_tuning(**rec["tuning"])
+                self.chosen[key] = dict(rec, replayed=True)
+            else:
+                lay = self._make(key)
+                if self.autotune and self._nargs >= 3 and self._kw:
+                    lay = self._autotune(key, lay, int(feat_dim), bool(bf16), bool(normalized))
             self._by_lpr[key] = lay
         return lay
+
+    def choices(self):
+        """The decisions taken by timing (or replayed) so far, in a form that JSON can carry: {"lanes,elem bytes,row
+        class": {"cut", "segment", "tuning"}}.  Pass it as `choices=` to a family of the same plan to get the same
+        layouts without timing."""
+        return {",".join(str(p) for p in k): {"cut": int(v["cut"]), "segment": int(v["segment"]),
+                                             "tuning": {n: int(x) for n, x in v["tuning"].items()}}
+                for k, v in self.chosen.items()}
 
     def _autotune(self, key, first, feat, bf16, normalized):
         import torch

@@ -8,6 +8,7 @@ layer the GIN workload needs; upstream has only its kernel (ROF.SAG, reuse_conv_
 """
 from __future__ import annotations
 
+import json
 import math
 
 import numpy as np
@@ -65,13 +66,20 @@ class ROF_inputInfo:
     # ---- on-disk form of the (expensive) plan; upstream caches the whole object with torch.save
     # (ROF_evaluation/cuda/middle-main.py:440-452), which also works; this form is plain numpy
     def save(self, path):
-        """Write every plan tensor plus the two scalars to an .npz file."""
+        """Write every plan tensor plus the two scalars to an .npz file -- and, as a JSON string, what an autotuning
+        layout family has chosen by timing so far (cut of long rows and launch settings per width class), so that a
+        later run takes the same layouts without timing and sums in the same order."""
         arrays = {name: getattr(self, name).detach().cpu().numpy() for name in _TENSOR_FIELDS}
-        np.savez(path, partSize=np.int64(self.partSize), warpPerBlock=np.int64(self.warpPerBlock), **arrays)
+        fam = self.layouts.get("ROF_v2")
+        choices = json.dumps(fam.choices() if fam is not None else {})
+        np.savez(path, partSize=np.int64(self.partSize), warpPerBlock=np.int64(self.warpPerBlock),
+                 layout_choices=np.array(choices), **arrays)
 
     @classmethod
-    def load(cls, path, device="cuda", **layout_opts):
-        """Inverse of save(); rebuilds the device layout from the stored v2 arrays without a plan search."""
+    def load(cls, path, device="cuda", autotune=None, **layout_opts):
+        """Inverse of save(); rebuilds the device layout from the stored v2 arrays without a plan search.  Width
+        classes whose layout was chosen by timing before the save are rebuilt as chosen; `autotune` applies to the
+        others."""
         z = np.load(path if str(path).endswith(".npz") else str(path) + ".npz")
         t = {name: torch.from_numpy(z[name]).to(device) for name in _TENSOR_FIELDS}
         info = cls(t["row_pointers"], t["column_index"], t["degrees"], t["part_pointers"], t["part2Node"],
@@ -82,8 +90,10 @@ class ROF_inputInfo:
             n, ps = len(z["row_pointers"]) - 1, int(z["partSize"])
             v2 = tuple(np.array(z[k]) for k in ("uniqpart_column_index", "uniqpart_pointers", "part2Node_ptr",
                                                  "part2Node_col"))
+            choices = json.loads(str(z["layout_choices"])) if "layout_choices" in z.files else {}
             info.layouts["ROF_v2"] = LayoutFamily(lambda lpr, eb, rb=0, **kw: Layout.from_v2(
-                *v2, n, ps, lanes_per_row=lpr, elem_bytes=eb, row_bytes=rb, **{**layout_opts, **kw}))
+                *v2, n, ps, lanes_per_row=lpr, elem_bytes=eb, row_bytes=rb, **{**layout_opts, **kw}),
+                autotune=autotune, choices=choices)
         return info
 
     def __getstate__(self):

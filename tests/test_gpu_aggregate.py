@@ -619,10 +619,19 @@ def test_calibration_and_autotuning_choose_by_timing_and_change_no_bit(oracle):
                        autotune=True)
     tuned = fam.get(feat, False)
     (key, rec), = fam.chosen.items()
-    assert key == (32, 4, 0) and (rec["cut"], rec["segment"]) in {tuple(rec["rule"]), (128, 32), (512, 64), (1024, 128)}
+    assert key == (32, 4, 0) and (rec["cut"], rec["segment"]) in {tuple(rec["rule"]), (128, 32), (512, 64), (1024, 128), (2048, 256)}
     assert f"{rec['cut']}/{rec['segment']}" in rec["ms"] and len(rec["ms"]) >= 2
     assert fam.get(feat, False) is tuned                          # timed once per width class
     tuned.set_degrees(degt)                                      # (the timing ran on placeholder degrees)
     got = tuned.aggregate(xt, normalized=True).cpu().numpy()
     _close(got, oracle.closed_form(indptr, indices, x, deg), oracle.closed_form(indptr, indices, np.abs(x), deg))
+    # the decisions travel as plain data: a second family replays them without timing and sums in the same order
+    again = LayoutFamily(lambda lpr, eb, rb=0, **kw: Layout.from_v2(*v2, lanes_per_row=lpr, elem_bytes=eb, row_bytes=rb, **kw),
+                         choices=fam.choices())
+    same = again.get(feat, False)
+    assert again.chosen[key]["replayed"] and same.tuning() == tuned.tuning()
+    assert (same.stats()["hub_split"], same.stats()["segment"]) == (rec["cut"], rec["segment"])
+    same.set_degrees(degt)
+    assert np.array_equal(same.aggregate(xt, normalized=True).cpu().numpy(), got)
+    again.close()
     fam.close()

@@ -251,3 +251,24 @@ def test_plan_container_round_trips_through_disk(tmp_path):
     a = ROF_GCNConvFunc.apply(x, w, info, False, "ROF_v2")
     b = ROF_GCNConvFunc.apply(x, w, back, False, "ROF_v2")
     assert torch.equal(a, b)
+
+
+def test_timed_layout_choices_are_saved_with_the_plan(tmp_path):
+    """What an autotuning family chose by timing is written with the plan and replayed after a load: no timing, the
+    same cut and launch settings, the same bits."""
+    from artifact_amd.reuse_conv import ROF_GCNConvFunc
+    ip, ix = make_workload("c4", 6)
+    n = len(ip) - 1
+    info = build_input_info(ip, ix, 3, device=DEV, autotune=True)
+    x = torch.from_numpy(features(n, 20, seed=63)).to(DEV)
+    w = torch.from_numpy(features(20, 47, seed=64)).to(DEV)
+    a = ROF_GCNConvFunc.apply(x, w, info, False, "ROF_v2")
+    chosen = info.layouts["ROF_v2"].choices()
+    assert chosen and all(set(v) == {"cut", "segment", "tuning"} for v in chosen.values())
+    path = str(tmp_path / "plan.npz")
+    info.save(path)
+    back = ROF_inputInfo.load(path, device=DEV)
+    b = ROF_GCNConvFunc.apply(x, w, back, False, "ROF_v2")
+    fam = back.layouts["ROF_v2"]
+    assert fam.choices() == chosen and all(v.get("replayed") for v in fam.chosen.values()) and not fam.autotune
+    assert torch.equal(a, b)
