@@ -381,6 +381,36 @@ def test_aggregation_is_capturable_in_a_hip_graph(oracle, wl, sd, opts):
     assert np.allclose(out.cpu().numpy(), want, rtol=1e-5, atol=1e-5)
 
 
+def test_two_streams_two_layouts_run_side_by_side(oracle):
+    """Calls are re-entrant per stream: two layouts of one plan (each with its own workspace of partial rows), issued
+    in turn on two streams without synchronising in between, give what each gives alone."""
+    indptr, indices, plan = _case("c2", 2, 3)                  # 65 536 nodes: segments, i.e. a workspace, in use
+    n = len(indptr) - 1
+    deg = torch.from_numpy(np.diff(indptr).astype(np.float32)).cuda()
+    lays = [_layout(plan, n, 3, lanes_per_row=16), _layout(plan, n, 3, lanes_per_row=16, min_consumers=2)]
+    xs = [torch.from_numpy(features(n, 64, seed=40 + i)).cuda() for i in range(2)]
+    alone = []
+    for lay, x in zip(lays, xs):
+        assert lay.stats()["partial_rows"] > 0
+        lay.set_degrees(deg)
+        alone.append(lay.aggregate(x, normalized=True).clone())
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    outs = [torch.empty_like(a) for a in alone]
+    for s in streams:
+        s.wait_stream(torch.cuda.current_stream())
+    for _ in range(10):
+        for lay, x, o, s in zip(lays, xs, outs, streams):
+            with torch.cuda.stream(s):
+                lay.aggregate(x, normalized=True, out=o)
+    for s in streams:
+        torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    assert torch.equal(outs[0], alone[0]) and torch.equal(outs[1], alone[1])
+    want = oracle.closed_form(indptr, indices, xs[0].cpu().numpy(), np.diff(indptr).astype(np.float32))
+    assert np.allclose(outs[0].cpu().numpy(), want, rtol=1e-4, atol=1e-5)
+
+
 def test_byte_offsets_between_2_and_4_gib():
     """Regression: with the short address arithmetic (row id x row bytes in 32 bits) a feature matrix or a
     partial-sum workspace between 2 GiB and 4 GiB puts byte offsets above 2^31, which must be taken as unsigned.
