@@ -13,6 +13,8 @@
 
 #include <c10/hip/HIPStream.h>
 
+#include <cstdlib>
+#include <cstring>
 #include <list>
 #include <map>
 #include <memory>
@@ -20,6 +22,7 @@
 #include <vector>
 
 #include "rof.h"
+#include "rof_bench.h"
 
 namespace {
 
@@ -70,33 +73,96 @@ struct Plan {
         // one row per wavefront covers every width from 81 floats up: rows of 1024 bytes and more are a class of
         // their own (they are cut finer), like in the Python layer's LayoutFamily
         const int row_bytes = lpr == 64 ? (feat * 4 >= 1024 ? 1024 : 512) : 0;
-        std::unique_ptr<Layout> &slot = by_lanes[lpr * 2 + (row_bytes == 1024)];
-        if (slot) return *slot;
-        slot.reset(new Layout);
+        const int cls = lpr * 2 + (row_bytes == 1024);
+        auto found = by_lanes.find(cls);
+        if (found != by_lanes.end()) return *found->second;
         rof_layout_opts o;
         memset(&o, 0, sizeof(o));
         o.lanes_per_row = lpr;
         o.elem_bytes = 4;
         o.row_bytes = row_bytes;
+        std::unique_ptr<Layout> lay(new Layout);
+        lay->h = build(o);
+        if (autotune_wanted()) autotune(lay, o, feat);
+        return *(by_lanes[cls] = std::move(lay));
+    }
+
+    // the plan re-laid out with the given options
+    rof_layout *build(rof_layout_opts o) {
         auto p = [this](size_t i) { return host[i].numel() ? host[i].data_ptr<int32_t>() : nullptr; };
+        rof_layout *h = nullptr;
         int rc;
         if (kind == 0) {
             rc = rof_layout_from_parts(p(0), host[1].data_ptr<int32_t>(), p(2), host[2].numel(), (int32_t)nodes, part_size,
-                                       &o, &slot->h);
+                                       &o, &h);
         } else if (kind == 1) {
             o.min_consumers = -1;   // every cache row is materialised, so that workspace row g is upstream's cache row g
             rc = rof_layout_from_v1(p(0), host[1].data_ptr<int32_t>(), p(2), host[2].numel(), p(3),
                                     host[4].data_ptr<int32_t>(), p(5), host[4].numel() - 1, (int32_t)nodes, part_size, &o,
-                                    &slot->h);
+                                    &h);
         } else {
             rc = rof_layout_from_v2(p(0), host[1].data_ptr<int32_t>(), host[2].data_ptr<int32_t>(), p(3),
-                                    host[1].numel() - 1, (int32_t)nodes, part_size, &o, &slot->h);
+                                    host[1].numel() - 1, (int32_t)nodes, part_size, &o, &h);
         }
-        if (rc != ROF_OK) {
-            by_lanes.erase(lpr * 2 + (row_bytes == 1024));
-            rof_check(rc, "re-laying out the plan");
+        rof_check(rc, "re-laying out the plan");
+        return h;
+    }
+
+    // ROF_AUTOTUNE=1 in the environment: how long rows are cut and how the launches are tuned is chosen by timing, as
+    // the Python layer's LayoutFamily(autotune=True) does -- the rule's layout against four other cuts on random rows
+    // of this width (sum aggregation, HIP events), then rof_layout_calibrate for the launch settings of the winner.
+    static bool autotune_wanted() {
+        const char *e = getenv("ROF_AUTOTUNE");
+        return e && *e && strcmp(e, "0") != 0;
+    }
+
+    void autotune(std::unique_ptr<Layout> &lay, const rof_layout_opts &rule_opts, int64_t feat) {
+        if (nodes == 0 || feat < 1) return;
+        static const int kCuts[][2] = {{128, 32}, {512, 64}, {1024, 128}, {2048, 256}};
+        const auto dev = torch::TensorOptions().dtype(torch::kFloat32).device(keep.empty() ? torch::Device(torch::kCUDA) : keep[0].device());
+        const int64_t ld = (feat + 3) / 4 * 4;
+        torch::Tensor x = torch::randn({nodes, ld}, dev), out = torch::empty({nodes, feat}, dev);
+        int64_t st[23];
+        rof_check(rof_layout_stats_n(lay->h, st, 23), "reading the layout's counters");
+        const int64_t rule_cut = st[20], rule_seg = st[21];
+        auto time_of = [&](Layout &l) {
+            rof_check(rof_layout_upload(l.h, current_stream()), "uploading the layout");
+            const size_t need = rof_layout_workspace_bytes(l.h, (int)feat);
+            l.workspace = torch::empty({(int64_t)std::max<size_t>(1, (need + 3) / 4)}, dev);
+            float best = 0.f;
+            for (int round = 0; round < 3; ++round) {   // the first round warms up
+                float ms = 0.f;
+                rof_check(rof_aggregate_timed(l.h, x.data_ptr<float>(), ROF_F32, ld, out.data_ptr<float>(), feat, (int)feat, 0,
+                                              nullptr, l.workspace.data_ptr(), (size_t)l.workspace.numel() * 4,
+                                              current_stream(), 3, &ms),
+                          "timing a candidate layout");
+                if (round == 1 || (round == 2 && ms < best)) best = ms;
+            }
+            return best;
+        };
+        float best_ms = time_of(*lay);
+        const float rule_ms = best_ms;
+        // other cuts can only matter when some row is long enough to be cut by one of them
+        if (st[7] > 0 || st[22] > kCuts[0][0]) {
+            for (const auto &c : kCuts) {
+                if (c[0] == rule_cut && c[1] == rule_seg) continue;
+                rof_layout_opts o = rule_opts;
+                o.hub_split = c[0];
+                o.segment = c[1];
+                std::unique_ptr<Layout> cand(new Layout);
+                cand->h = build(o);
+                const float ms = time_of(*cand);
+                if (ms < 0.99f * rule_ms && ms < best_ms) {   // the rule's choice unless a candidate is measurably faster
+                    best_ms = ms;
+                    lay = std::move(cand);
+                }
+            }
         }
-        return *by_lanes[lpr * 2 + (row_bytes == 1024)];
+        rof_launch_tuning chosen;
+        rof_check(rof_layout_calibrate(lay->h, x.data_ptr<float>(), ROF_F32, ld, out.data_ptr<float>(), feat, (int)feat, 0, nullptr,
+                                       lay->workspace.data_ptr(), (size_t)lay->workspace.numel() * 4, current_stream(), 2, 3,
+                                       &chosen),
+                  "calibrating the launch settings");
     }
 };
 

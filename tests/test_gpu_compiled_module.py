@@ -125,3 +125,32 @@ def test_upstream_layer_runs_on_the_compiled_module(oracle, ROF, monkeypatch):
     gp = oracle.closed_form(ip, ix, np.ones((n, 12)), deg)
     assert np.allclose(xt.grad.cpu().numpy(), gp @ w.astype(np.float64).T, rtol=1e-4, atol=1e-5)
     assert np.allclose(wt.grad.cpu().numpy(), x.astype(np.float64).T @ gp, rtol=1e-4, atol=1e-3)
+
+
+def test_the_compiled_module_chooses_cuts_by_timing_when_asked(oracle, ROF, monkeypatch):
+    """ROF_AUTOTUNE=1: the module times the rule's layout against four other cuts of the long rows and calibrates the
+    launch settings of the winner (rof_aggregate_timed, rof_layout_calibrate from C++).  Whatever it picks, forward
+    and backward give the float64 closed form; with the variable unset the cache holds the rule's layouts again."""
+    ip, ix = make_workload("c4", 5)                                      # 75 000 nodes, rows of up to 10 000 entries
+    n = len(ip) - 1
+    info = build_input_info(ip, ix, part_size=3, device=DEV)
+    x, w = features(n, 20, seed=31), glorot(20, 47, seed=32)
+    xt, wt = torch.from_numpy(x).to(DEV), torch.from_numpy(w).to(DEV)
+    deg = np.diff(ip).astype(np.float32)
+    tmp = x.astype(np.float64) @ w.astype(np.float64)
+    want, mag = oracle.closed_form(ip, ix, tmp, deg), oracle.closed_form(ip, ix, np.abs(tmp), deg)
+    ROF.clear_layout_cache()
+    plain = ROF.reuse_forward_v2(*_call("v2", info, xt, wt))[0].clone()
+    monkeypatch.setenv("ROF_AUTOTUNE", "1")
+    ROF.clear_layout_cache()
+    tuned = ROF.reuse_forward_v2(*_call("v2", info, xt, wt))[0]
+    close_fp32(tuned.cpu().numpy(), want, mag)
+    assert torch.equal(ROF.reuse_forward_v2(*_call("v2", info, xt, wt))[0], tuned)       # timed once, cached
+    d_out = torch.from_numpy(features(n, 47, seed=33)).to(DEV)
+    d_in, d_w = ROF.reuse_backward_v2(*_call("v2", info, d_out, xt, wt))
+    agg = oracle.closed_form(ip, ix, d_out.cpu().numpy().astype(np.float64), deg)
+    assert np.allclose(d_in.cpu().numpy(), agg @ w.astype(np.float64).T, rtol=1e-4, atol=1e-4)
+    assert np.allclose(d_w.cpu().numpy(), x.astype(np.float64).T @ agg, rtol=1e-4, atol=1e-3)
+    monkeypatch.delenv("ROF_AUTOTUNE")
+    ROF.clear_layout_cache()
+    assert torch.equal(ROF.reuse_forward_v2(*_call("v2", info, xt, wt))[0], plain)
