@@ -20,15 +20,28 @@ import argparse
 import sys
 import time
 
+import numpy as np
+
 from . import reuse_search_ext as R
-from .graphgen import WORKLOADS, make_workload, planted_reuse_csr
+from .graphgen import WORKLOADS, csr_from_pairs, make_workload, planted_reuse_csr, rmat_csr
 from .layout import Layout, lanes_per_row
 from .tune_check import time_round_robin
 
 # (set_size, members per set, extra random neighbours per node[, sets per node: with more than one a node's club mates
 # differ from set to set, so its sets cannot all be shared inside one workgroup])
 CASES = ((12, 64, 4), (12, 64, 24), (12, 8, 24), (12, 2, 12), (6, 64, 24), (6, 4, 24), (3, 64, 24), (3, 64, 48), (3, 4, 24),
-         (3, 2, 24), (12, 8, 12, 2), (6, 16, 12, 2), (3, 16, 24, 2), (3, 64, 24, 3))
+         (3, 2, 24), (12, 8, 12, 2), (6, 16, 12, 2), (3, 16, 24, 2), (3, 64, 24, 3), "mixed")
+
+
+def mixed_csr(nodes, seed):
+    """A heavy-tailed R-MAT graph (average degree 16) whose upper half of the ids also carries planted sets (6 anchors
+    x 16 members): rows with hubs and rows with shared neighbour sets in one graph."""
+    a_ptr, a_idx = rmat_csr(nodes, 16, seed)
+    b_ptr, b_idx = planted_reuse_csr(nodes // 2, 6, 16, 0, seed=seed + 1)
+    ua = np.repeat(np.arange(nodes, dtype=np.int64), np.diff(a_ptr))
+    ub = np.repeat(np.arange(nodes // 2, dtype=np.int64), np.diff(b_ptr)) + nodes // 2
+    return csr_from_pairs(np.concatenate([ua, ub]), np.concatenate([a_idx.astype(np.int64), b_idx.astype(np.int64) + nodes // 2]),
+                          nodes, False)
 
 
 def check(case, nodes, feat, part_size=3, log=print):
@@ -36,7 +49,10 @@ def check(case, nodes, feat, part_size=3, log=print):
     import torch
 
     t0 = time.time()
-    if isinstance(case, str):
+    if case == "mixed":
+        ip, ix = mixed_csr(nodes, 95)
+        label = "R-MAT of degree 16 + planted sets 6 x 16 on half of the nodes"
+    elif isinstance(case, str):
         case, _, ps = case.partition(":")              # "c3:2" = workload c3 at part size 2
         part_size = int(ps) if ps else part_size
         ip, ix = make_workload(case)
