@@ -460,52 +460,51 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
                 len[L->group_dst[j]] += L->group_ptr[g + 1] - L->group_ptr[g];
         for (int32_t v = 0; v < n; ++v) len_all[v] = (int32_t)std::min<int64_t>(len[v], INT32_MAX);
     }
-    // Dense graphs.  The segments of a row of `len` entries each gather from a band of segment / len of the matrix,
-    // and the swept launch keeps such bands in L2 where a whole row, gathered as one task, ranges over the entire
-    // matrix: rows long enough for bands of a few MB at 64 entries per segment (16 entries per MB of matrix) are
-    // worth cutting even below the rule's cut -- when they hold a quarter of the edges and are half of all rows, on a
-    // matrix several times the size of an L2 (uniform degrees of 600, 2^17 nodes: 24 floats 1.35 ms at 640 / 160 against 0.61 at 128 / 64, 47
-    // floats 2.13 against 0.86, 128 bf16 2.15 against 1.16; sparse graphs lose 4-5 % with the lower cut and do not
-    // meet the condition).
-    const int64_t matrix_mb = (int64_t)n * row_bytes >> 20;
-    const int32_t sweep_cut = (int32_t)std::max<int64_t>(128, 16 * matrix_mb);
-    if (groups >= 4 && matrix_mb >= 8 && sweep_cut < rule_cut) {
-        int64_t between = 0, all = 0, long_rows = 0;
+    // Dense graphs: two thirds of all edges in rows of more than 128 entries.  What suits them depends on whether a
+    // set of sources that one L2 can hold is popular -- the share of all gathers that goes to the 4 MB / row bytes
+    // most gathered rows (in a symmetric graph: the longest ones).
+    //  * Popular sources (45 % and more; measured 47-64 %) stay in L2 by themselves, and what the segments cost counts:
+    //    the fine cut of the wide rows (128 / 32 up to three rows per wavefront on a matrix that the caches hold) was
+    //    measured at average degree 14, where it balances a few hub rows; where the segments are the launch, 32 entries
+    //    are too few for a task that costs a wavefront, a partial row written and read, and three dependent loads
+    //    before its first gather (R-MAT 2^18 nodes, average degree 83, 160 floats: 1.15 ms at 128 / 32, 0.89 at 128 /
+    //    64, 0.86 at 128 / 128, 0.79 at 512 / 128, 0.75 at 1024 / 128; 2^16 nodes, degree 341: 0.87 / 0.72 at 512 /
+    //    128; 512 / 128 is at or within 6 % of the best of seven choices on the nine such graphs measured at 72, 100
+    //    and 160 floats; rows of 1 KB: 256 / 64 within 4 % of the best on four graphs, 1024 / 128 up to 14 % behind
+    //    and 128 / 32 up to 22 %).
+    //  * No popular sources (uniform degrees of 600: 3-12 %; R-MAT a = .5 on 233 000 nodes, average degree 435: 30-40
+    //    %): a row gathered as one task ranges over the whole matrix and misses, while the segments of a row of `len`
+    //    entries each gather from a band of segment / len of it, which the swept launch keeps in L2.  So the wide
+    //    rows keep their fine cut (uniform degrees, 160 floats: 2.95 ms at 128 / 32, 5.08 at 128 / 128; the R-MAT
+    //    graph, 128 floats: 2.84 at 128 / 32, 3.17 at 512 / 128), and from four rows per wavefront the cut comes down
+    //    to 256 / 64 so that the rows are cut at all (uniform degrees of 600 sit just under 640: 24 floats 1.35 ms at
+    //    640 / 160, 0.61 at 256 / 64; 47 floats 2.13 / 0.85; 128 bf16 at 1280 / 320 2.15 / 1.16; the R-MAT graph at 64
+    //    floats 1.54 at 1024 / 128, 1.40 at 256 / 64).  Only on a matrix of several L2s and a launch that fills the
+    //    machine; sparse graphs lose 4-5 % with the lower cut and do not meet the condition.
+    const bool fine_wide = elem_bytes == 4 && groups <= 3 && rule_cut == 128 && rule_segment == 32;
+    const bool coarse_narrow = groups >= 4 && rule_cut > 256 && (int64_t)n * row_bytes >= 2 * kL2Bytes &&
+                               n / groups >= kWavesToFill;
+    if (fine_wide || coarse_narrow) {
+        int64_t beyond = 0, all = 0;
         for (int32_t v = 0; v < n; ++v) {
             all += len_all[v];
-            long_rows += len_all[v] > sweep_cut;
-            if (len_all[v] > sweep_cut && len_all[v] <= rule_cut) between += len_all[v];
+            if (len_all[v] > 128) beyond += len_all[v];
         }
-        // (... and when the typical row is that long: where most rows are short and a minority holds the edges,
-        // those rows are also the popular sources, which stay in L2 without a sweep, and coarser segments win:
-        // R-MAT 2^16 nodes, average degree 341, 128 bf16: 0.341 ms at 256 / 64 against 0.303 at 1280 / 320)
-        if (between * 4 >= all && long_rows * 2 >= n) {
-            rule_cut = sweep_cut;
-            rule_segment = 64;
-        }
-    }
-    // Dense graphs with popular sources.  The fine cut of the wide rows (128 / 32 up to three rows per wavefront on a
-    // matrix that the caches hold) was measured on graphs of average degree 14, where a few hub rows are cut and
-    // fine segments balance them.  Where two thirds of all edges lie in rows beyond that cut, the segments are the
-    // launch, and 32 entries are too few for a task that costs a wavefront, a partial row written and read, and
-    // three dependent loads before its first gather (R-MAT 2^18 nodes, average degree 83, 160 floats: 1.15 ms at
-    // 128 / 32, 0.89 at 128 / 64, 0.86 at 128 / 128, 0.79 at 512 / 128, 0.75 at 1024 / 128; 2^16 nodes, degree 341:
-    // 0.87 / 0.72 at 512 / 128; 512 / 128 is at or within 6 % of the best of seven choices on the nine dense graphs
-    // measured at 72, 100 and 160 floats).  Not so when the typical row is long (uniform degrees of 600: 2.95 ms at 128 / 32, 5.08 at 128 / 128):
-    // there no source is popular enough to stay in L2 by itself and the narrow bands of fine segments are what hits.
-    if (elem_bytes == 4 && groups <= 3 && rule_cut == 128 && rule_segment == 32) {
-        int64_t beyond = 0, all = 0, long_rows = 0;
-        for (int32_t v = 0; v < n; ++v) {
-            all += len_all[v];
-            long_rows += len_all[v] > rule_cut;
-            if (len_all[v] > rule_cut) beyond += len_all[v];
-        }
-        if (beyond * 3 >= all * 2 && long_rows * 2 < n) {
-            // (rows of 1 KB: 256 / 64 is within 4 % of the best on the four dense graphs measured at 256 floats,
-            // 1024 / 128 up to 14 % behind and 128 / 32 up to 22 %)
-            const bool wide = groups == 1 && row_bytes >= 1024;
-            rule_cut = wide ? 256 : 512;
-            rule_segment = wide ? 64 : 128;
+        if (beyond * 3 >= all * 2) {
+            int64_t hot = 0;
+            const int64_t k = std::min<int64_t>(n, kL2Bytes / std::max<int64_t>(1, row_bytes));
+            ivec sorted(len_all);
+            if (k > 0 && k < n) std::nth_element(sorted.begin(), sorted.begin() + (k - 1), sorted.end(), std::greater<int32_t>());
+            for (int64_t i = 0; i < k; ++i) hot += sorted[i];
+            const bool popular = hot * 20 >= all * 9;
+            if (fine_wide && popular) {
+                const bool wide = groups == 1 && row_bytes >= 1024;
+                rule_cut = wide ? 256 : 512;
+                rule_segment = wide ? 64 : 128;
+            } else if (coarse_narrow && !popular) {
+                rule_cut = 256;
+                rule_segment = 64;
+            }
         }
     }
     const int32_t hub_split = (o && o->hub_split > 0) ? o->hub_split : rule_cut;

@@ -2,7 +2,7 @@
 own choice of wavefront cap, XCD run, row gathers in flight and long-row cut within a few per cent of the best of
 the alternatives?
 
-    python -m artifact_amd.tune_check [--graphs h1,...,h12] [--out table.md]
+    python -m artifact_amd.tune_check [--graphs h1,...,h13] [--out table.md]
 
 For every (graph, width) one aggregation layer (no reuse plan: `Layout.from_csr`) is timed with the default layout
 and launch settings and then with one setting changed at a time: wavefronts per SIMD of the destination-row launch
@@ -72,6 +72,8 @@ GRAPHS = {
     "h10": ("4-neighbour grid 2048 x 2048", lambda: grid_csr(2048, 2048)),
     "h11": ("16 random partners within 32768 ids, 2^21 nodes", lambda: banded_csr(1 << 21, 16, 1 << 15, 80)),
     "h12": ("bipartite: 2^20 users x 16 of 2^15 items, popularity 1 / rank", lambda: bipartite_csr(1 << 20, 1 << 15, 16, 81)),
+    # dense without a popular set of sources that one L2 could hold
+    "h13": ("R-MAT a=.5 b=c=.2, 233 000 nodes, average degree 435", lambda: rmat_csr(233_000, 480, 91, a=0.5, b=0.2, c=0.2)),
 }
 WIDTHS = ((24, False), (72, False), (160, False), (128, True))
 

@@ -315,12 +315,11 @@ def test_the_relative_cluster_gate_applies_only_to_graphs_with_local_sources():
 
 
 def test_dense_graphs_are_cut_by_what_their_rows_look_like():
-    """Two rules for dense graphs.  (1) Up to three rows per wavefront on a matrix that the caches hold: the fine cut
-    128 / 32 suits graphs whose few hub rows it balances; where two thirds of the edges lie beyond it, the segments
-    are the launch and take 512 / 128 (256 / 64 for rows of 1 KB) -- unless the typical row is that long, in which case
-    no source is popular and only the narrow bands of fine segments hit in L2.  (2) From four rows per wavefront, when
-    half of the rows are longer than 16 entries per MB of matrix and those below the rule's cut hold a quarter of the
-    edges, the cut comes down to them (segments of 64), so that they are swept."""
+    """Dense graphs (two thirds of the edges in rows of more than 128 entries) are cut by whether a set of sources
+    that one L2 can hold is popular (45 % of all gathers go to the 4 MB / row bytes longest rows).  Popular: the
+    segments' cost counts, and wide rows on a cached matrix take 512 / 128 (256 / 64 for rows of 1 KB) instead of the
+    fine 128 / 32.  Not popular: only the narrow bands of fine segments hit in L2; wide rows keep 128 / 32, and from
+    four rows per wavefront the cut comes down to 256 / 64 so that the rows are swept at all."""
     def cut_of(ip, ix, **kw):
         st = Layout.from_csr(ip, ix, **kw).stats()
         return st["hub_split"], st["segment"]
@@ -335,9 +334,9 @@ def test_dense_graphs_are_cut_by_what_their_rows_look_like():
     u = np.repeat(np.arange(1 << 15), 150)                   # uniform degrees around 300: every row beyond 128
     ip, ix = csr_from_pairs(u, np.random.default_rng(3).integers(0, 1 << 15, len(u)), 1 << 15, False)
     assert np.diff(ip).min() > 200
-    assert cut_of(ip, ix, lanes_per_row=32) == (128, 32)     # the typical row is long: fine segments
+    assert cut_of(ip, ix, lanes_per_row=32) == (128, 32)     # no popular sources: fine segments
     assert cut_of(ip, ix, lanes_per_row=8) == (256, 128)     # 4 MB: an L2 holds the matrix, the small-launch cut stays
-    # (2): 2^17 rows x 128 bytes = 16 MB -> rows beyond 256 entries are worth sweeping, and every row has about 300
+    # 2^17 rows x 128 bytes = 16 MB, every row about 300 entries and none popular: cut below them
     u = np.repeat(np.arange(1 << 17), 150)
     ip, ix = csr_from_pairs(u, np.random.default_rng(4).integers(0, 1 << 17, len(u)), 1 << 17, False)
     deg = np.diff(ip)
