@@ -476,8 +476,8 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     //    %): a row gathered as one task ranges over the whole matrix and misses, while the segments of a row of `len`
     //    entries each gather from a band of segment / len of it, which the swept launch keeps in L2.  So the wide
     //    rows keep their fine cut (uniform degrees, 160 floats: 2.95 ms at 128 / 32, 5.08 at 128 / 128; the R-MAT
-    //    graph, 128 floats: 2.84 at 128 / 32, 3.17 at 512 / 128), and from four rows per wavefront the cut comes down
-    //    to 256 / 64 so that the rows are cut at all (uniform degrees of 600 sit just under 640: 24 floats 1.35 ms at
+    //    graph, 128 floats: 2.84 at 128 / 32, 3.17 at 512 / 128), and from four rows per wavefront, where half of the
+    //    rows are that long, the cut comes down to 256 / 64 so that the rows are cut at all (uniform degrees of 600 sit just under 640: 24 floats 1.35 ms at
     //    640 / 160, 0.61 at 256 / 64; 47 floats 2.13 / 0.85; 128 bf16 at 1280 / 320 2.15 / 1.16; the R-MAT graph at 64
     //    floats 1.54 at 1024 / 128, 1.40 at 256 / 64).  Only on a matrix of several L2s and a launch that fills the
     //    machine; sparse graphs lose 4-5 % with the lower cut and do not meet the condition.
@@ -485,10 +485,13 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     const bool coarse_narrow = groups >= 4 && rule_cut > 256 && (int64_t)n * row_bytes >= 2 * kL2Bytes &&
                                n / groups >= kWavesToFill;
     if (fine_wide || coarse_narrow) {
-        int64_t beyond = 0, all = 0;
+        int64_t beyond = 0, all = 0, long_rows = 0;
         for (int32_t v = 0; v < n; ++v) {
             all += len_all[v];
-            if (len_all[v] > 128) beyond += len_all[v];
+            if (len_all[v] > 128) {
+                beyond += len_all[v];
+                ++long_rows;
+            }
         }
         if (beyond * 3 >= all * 2) {
             int64_t hot = 0;
@@ -501,7 +504,9 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
                 const bool wide = groups == 1 && row_bytes >= 1024;
                 rule_cut = wide ? 256 : 512;
                 rule_segment = wide ? 64 : 128;
-            } else if (coarse_narrow && !popular) {
+            } else if (coarse_narrow && !popular && long_rows * 2 >= n) {
+                // (only where the typical row is that long: on heavy-tailed graphs, whose median row has a few entries,
+                // a lower cut costs 4-7 %)
                 rule_cut = 256;
                 rule_segment = 64;
             }

@@ -319,7 +319,8 @@ def test_dense_graphs_are_cut_by_what_their_rows_look_like():
     that one L2 can hold is popular (45 % of all gathers go to the 4 MB / row bytes longest rows).  Popular: the
     segments' cost counts, and wide rows on a cached matrix take 512 / 128 (256 / 64 for rows of 1 KB) instead of the
     fine 128 / 32.  Not popular: only the narrow bands of fine segments hit in L2; wide rows keep 128 / 32, and from
-    four rows per wavefront the cut comes down to 256 / 64 so that the rows are swept at all."""
+    four rows per wavefront, where half of the rows are that long, the cut comes down to 256 / 64 so that the rows are
+    swept at all."""
     def cut_of(ip, ix, **kw):
         st = Layout.from_csr(ip, ix, **kw).stats()
         return st["hub_split"], st["segment"]
