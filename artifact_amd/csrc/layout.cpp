@@ -462,7 +462,7 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     }
     // Dense graphs: two thirds of all edges in rows of more than 128 entries.  What suits them depends on whether a
     // set of sources that one L2 can hold is popular -- the share of all gathers that goes to the 4 MB / row bytes
-    // most gathered rows (in a symmetric graph: the longest ones).
+    // most gathered rows.
     //  * Popular sources (45 % and more; measured 47-64 %) stay in L2 by themselves, and what the segments cost counts:
     //    the fine cut of the wide rows (128 / 32 up to three rows per wavefront on a matrix that the caches hold) was
     //    measured at average degree 14, where it balances a few hub rows; where the segments are the launch, 32 entries
@@ -494,9 +494,15 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
             }
         }
         if (beyond * 3 >= all * 2) {
+            // how often every row is gathered (every group expanded), then the k most gathered
             int64_t hot = 0;
             const int64_t k = std::min<int64_t>(n, kL2Bytes / std::max<int64_t>(1, row_bytes));
-            ivec sorted(len_all);
+            ivec sorted((size_t)n, 0);
+            for (int32_t c : L->res_col) sorted[c]++;
+            for (int64_t g = 0; g < G; ++g) {
+                const int32_t uses = L->group_dst_ptr[g + 1] - L->group_dst_ptr[g];
+                for (int32_t j = L->group_ptr[g]; j < L->group_ptr[g + 1]; ++j) sorted[L->group_col[j]] += uses;
+            }
             if (k > 0 && k < n) std::nth_element(sorted.begin(), sorted.begin() + (k - 1), sorted.end(), std::greater<int32_t>());
             for (int64_t i = 0; i < k; ++i) hot += sorted[i];
             const bool popular = hot * 20 >= all * 9;
