@@ -452,3 +452,23 @@ def test_algorithmic_bytes_formula():
     assert a + b == lay.algorithmic_bytes(f) and a == 6 * (4 + 4 * f) + 2 * 4 * f + 4 * 3
     plain = _v2(plan, 10, 3, disable_reuse=True)
     assert plain.algorithmic_bytes(f) == 28 * (4 + 4 * f) + 10 * (4 * f + 8) + 4
+
+
+def test_recorded_layout_choices_are_replayed_without_a_gpu():
+    """`LayoutFamily(choices=...)` rebuilds the width classes it has a record for with the recorded cut, segment and
+    launch settings (plain data, as `choices()` returns it and `ROF_inputInfo.save` stores it); other classes follow
+    the rules."""
+    from artifact_amd.layout import LayoutFamily
+    ip, ix = make_workload("c4", 4)
+    rec = {"12,4,0": {"cut": 512, "segment": 64, "tuning": {"xcd_run_partial": 0, "xcd_run_dst": 16, "wave_cap": 6,
+                                                            "lds_pad": 0, "deep": 1}}}
+    fam = LayoutFamily(lambda lpr, eb, rb=0, **kw: Layout.from_csr(ip, ix, lanes_per_row=lpr, elem_bytes=eb, row_bytes=rb, **kw),
+                       autotune=False, choices=rec)
+    lay = fam.get(47)
+    st = lay.stats()
+    assert (st["hub_split"], st["segment"]) == (512, 64) and lay.tuning() == rec["12,4,0"]["tuning"]
+    assert fam.choices() == rec and fam.chosen[(12, 4, 0)]["replayed"]
+    other = fam.get(32)                                       # no record for 8 lanes: the rule's cut, default settings
+    assert (other.stats()["hub_split"], other.stats()["segment"]) == (640, 160) and other.tuning()["wave_cap"] == -1
+    assert fam.choices() == rec
+    fam.close()
