@@ -1,6 +1,6 @@
 """The boundary as a compiler sees it: include/rof.h and include/rof_bench.h are valid C11 and C++17 on their own,
 the struct sizes that the ctypes binding assumes are the compiler's, and the C++ operator module that binds the C
-ABI (artifact_amd/csrc/rof_torch.cpp, the text INTEGRATION.md shows) is built and loads.  No GPU."""
+ABI (artifact_amd/csrc/rof_torch.cpp, the text that the integration guide shows) is built and loads.  No GPU."""
 import os
 import shutil
 import subprocess
@@ -79,7 +79,7 @@ def test_compiled_operator_module_is_built_and_exports_the_upstream_functions():
 
 
 def test_integration_doc_shows_the_compiled_source():
-    """INTEGRATION.md's C++ binding is quoted from csrc/rof_torch.cpp, not written beside it."""
+    """The C++ binding that the integration guide shows is quoted from csrc/rof_torch.cpp, not written beside it."""
     doc = open(os.path.join(ROOT, "INTEGRATION.md")).read()
     src = open(os.path.join(ROOT, "artifact_amd", "csrc", "rof_torch.cpp")).read()
     start = doc.index("```cpp", doc.index("### 3.2")) + len("```cpp\n")
@@ -87,4 +87,4 @@ def test_integration_doc_shows_the_compiled_source():
     blocks = [b for b in quoted.split("// ...\n") if b.strip()]
     assert blocks, "no quoted source"
     for b in blocks:
-        assert b in src, "INTEGRATION.md quotes text that is not in csrc/rof_torch.cpp:\n" + b[:200]
+        assert b in src, "the integration guide quotes text that is not in csrc/rof_torch.cpp:\n" + b[:200]
