@@ -524,9 +524,18 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
                                                   : std::max<int32_t>(16, (int64_t)hub_split * rule_segment / rule_cut);
     L->hub_split = hub_split;
     L->segment = segment;
-    // partial rows are cold when the row that adds them up reads them (written one launch earlier, each read once):
-    // an entry of that chain costs about twice the cached figure, so half as many are allowed
-    const int64_t max_segments = std::max<int64_t>(64, chain_limit(L->e_orig > 0 ? L->e_orig : total, row_bytes) / 2);
+    // Partial rows are cold when the row that adds them up reads them (written one launch earlier, each read once): an
+    // entry of that chain costs about twice the cached figure -- and never less than a memory latency (700 ns) shared by
+    // the two reads that each of the wavefront's `groups` lane groups keeps in flight, which is what counts at wide
+    // rows (bipartite graph, 160 floats, one row of 821 000 entries: 4550 segments made the destination-row launch 1.69
+    // ms, 1.6 of it that row's task at 350 ns a segment; 1.19 ms with half as many).
+    int64_t max_segments;
+    {
+        const int64_t edges = L->e_orig > 0 ? L->e_orig : total;
+        const int64_t launch_ns = 15000 + edges * row_bytes * 60 / 1000000;
+        const int64_t ref_ns = std::max<int64_t>(2 * (10 + row_bytes * 14 / 100), 700 / (2 * groups));
+        max_segments = std::max<int64_t>(64, 3 * launch_ns / (4 * ref_ns));
+    }
     if (o && (o->share_scope < 0 || o->share_scope > 1)) return ROF_ERR_ARG;
     const bool disable = o && o->disable_reuse;
     const int32_t min_consumers = o ? o->min_consumers : 0;
