@@ -276,7 +276,8 @@ def test_small_matrices_keep_the_fine_cut():
 def test_a_row_of_the_whole_graph_gets_longer_segments():
     """The row that adds up a long row's partial sums is itself a chain of dependent reads, one per segment; a row
     so long that this chain would outlast the launch is cut into fewer, longer segments: at most
-    max(64, chain limit / 2) of them (partial rows are read cold, at about twice the cached cost per entry)."""
+    max(64, chain limit / 2) of them at these four rows per wavefront (partial rows are read cold, at about twice the
+    cached cost per entry; at wider rows a read costs no less than a memory latency shared by the reads in flight)."""
     n = 20000
     rng = np.random.default_rng(4)
     u, v = rng.integers(1, n, 2 * n), rng.integers(1, n, 2 * n)
