@@ -297,6 +297,13 @@ def test_a_row_of_the_whole_graph_gets_longer_segments():
     want = np.zeros((n, 2))
     np.add.at(want, np.repeat(np.arange(n), np.diff(ip)), x[ix])
     assert np.allclose(got, want, rtol=1e-11, atol=1e-11)
+    # one row per wavefront, rows of 640 bytes: a read costs 350 ns (700 ns of latency, two reads in flight)
+    wide = Layout.from_csr(ip, ix, lanes_per_row=64, row_bytes=640)
+    launch_ns = 15000 + len(ix) * 640 * 60 // 1000000
+    most_wide = max(64, 3 * launch_ns // (4 * 350))
+    exw = wide.export()
+    hub = int(np.nonzero(exw["b_task_out"] == 0)[0][0])
+    assert np.diff(exw["b_task_ptr"])[hub] == -(-(n - 1) // -(-(n - 1) // most_wide)) <= most_wide
 
 
 def test_the_relative_cluster_gate_applies_only_to_graphs_with_local_sources():
