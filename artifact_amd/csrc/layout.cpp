@@ -561,7 +561,8 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     // MB are 43 690 rows, run 43 % faster with whole tiles per XCD run than with runs of 4; at 72 floats 9 %)
     const int32_t near_ids = (int32_t)std::max<int64_t>(
         1, std::min<int64_t>(std::max<int64_t>(2 * kTileRows, kL2Bytes / std::max<int64_t>(1, row_bytes)), n / 16));
-    // Do the rows gather from their own neighbourhood (at least half of the sources nearby, every group expanded)?
+    // Do the rows gather from their own neighbourhood (35 % of the sources nearby, every group expanded: R-MAT graphs
+    // of 2^14 ... 2.4 M nodes measure 6-26 %, a band of 32 768 ids at 288-byte rows 44 %, block models 80-93 %)?
     // Then neighbouring rows share sources through the L2 of the XCD that their tile runs on, and a row that a
     // cluster takes out of the tile order loses that.
     auto sources_are_local = [&]() {
@@ -572,7 +573,7 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
             for (int32_t d = L->group_dst_ptr[g]; d < L->group_dst_ptr[g + 1]; ++d)
                 for (int32_t j = L->group_ptr[g]; j < L->group_ptr[g + 1]; ++j, ++all)
                     near += std::abs(L->group_col[j] - L->group_dst[d]) < near_ids;
-        return all > 0 && near * 2 >= all;
+        return all > 0 && near * 20 >= all * 7;
     };
 
     // Workgroup-local sharing first (cost-model mode only): consumers that the schedule can bring together in one
@@ -739,7 +740,7 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     // faster than 16 at every width from 16 to 100 floats on two devices and equal on a third, 1 and 2 are 0.9 %
     // slower than 4, 64 is 1-6 % slower; smaller graphs measure alike from 2 to 16).
     const int64_t tile_run = std::max<int64_t>(16, std::min<int64_t>(1024, tile_rows / (4 * groups)));
-    L->local_sources = gathered > 0 && nearby * 2 >= gathered;
+    L->local_sources = gathered > 0 && nearby * 20 >= gathered * 7;
     L->xcd_run = L->local_sources ? (int32_t)tile_run : 4;
     L->n_slots = slots;
     L->n_segments = segments;

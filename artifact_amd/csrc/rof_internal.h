@@ -61,7 +61,7 @@ struct rof_layout {
     int32_t xcd_run = 4;      // consecutive workgroups of the destination-row launch kept on one XCD
     // launch tuning of the benchmark interface (rof_layout_set_tuning): 0 / -1 = the library's own choice
     int32_t tune_xcd_run_partial = 0, tune_xcd_run_dst = 0, tune_wave_cap = -1, tune_lds_pad = 0, tune_deep = -1;
-    bool local_sources = false;   // at least half of the gathered rows lie within min(max(8192, rows of 4 MB), n / 16) ids of their destination
+    bool local_sources = false;   // 35 % of the gathered rows lie within min(max(8192, rows of 4 MB), n / 16) ids of their destination
     int64_t n_slots = 0;      // rows of the partial-sum workspace
     int64_t n_materialised = 0, n_segments = 0, gathered_rows = 0, partial_reads = 0, gathered_before_rows = 0;
     int64_t n_local_groups = 0, lds_reads = 0;   // workgroup-local groups (summed into LDS) and the reads of them
