@@ -739,7 +739,9 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     // graphs without that locality short runs balance the XCDs better (R-MAT, 2.4 M nodes: runs of 4 were 0-2 %
     // faster than 16 at every width from 16 to 100 floats on two devices and equal on a third, 1 and 2 are 0.9 %
     // slower than 4, 64 is 1-6 % slower; smaller graphs measure alike from 2 to 16).
-    const int64_t tile_run = std::max<int64_t>(16, std::min<int64_t>(1024, tile_rows / (4 * groups)));
+    // (at least 256 workgroups: at five rows per wavefront and more a tile is fewer, and runs of 256 measure the same
+    // on block models and 6 % faster on a graph whose sources lie in a band around the row)
+    const int64_t tile_run = std::max<int64_t>(256, std::min<int64_t>(1024, tile_rows / (4 * groups)));
     L->local_sources = gathered > 0 && nearby * 20 >= gathered * 7;
     L->xcd_run = L->local_sources ? (int32_t)tile_run : 4;
     L->n_slots = slots;
