@@ -52,8 +52,9 @@ int rof_device_gather(const void *table, uint32_t rows, int lanes_per_row, int i
  *   xcd_run_partial / xcd_run_dst: how many consecutive workgroups of the partial-sum launches / of the
  *     destination-row launch stay on one XCD (each XCD has its own L2, so runs of neighbouring destination rows
  *     share gathered rows there).  0 = the library's choice: 1 for the partial-sum launches; for the destination
- *     rows one tile of destinations per run when 35 % of the neighbours or more lie within min(max(8192, the rows
- *     that fill 4 MB), n / 16) ids of their row (block-structured and banded graphs), 4 workgroups otherwise.
+ *     rows one tile of destinations (256 workgroups at least) per run when 35 % of the neighbours or more lie
+ *     within min(max(8192, the rows that fill 4 MB), n / 16) ids of their row (block-structured and banded graphs),
+ *     4 workgroups otherwise.
  *   wave_cap: wavefronts per SIMD of the destination-row launch, 2..7; 0 = as many as fit; -1 = the library's
  *     choice from the size of the feature matrix, the row bytes and the row stride.
  *   deep: see below.
