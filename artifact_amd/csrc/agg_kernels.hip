@@ -75,6 +75,7 @@ constexpr int64_t kStreamPartialBytes = 64 << 20;
 // partial-sum launches, and graphs without hub rows (uniform degrees, 2^20 nodes x 64 floats: 689 / 700 us).  The
 // layout knows the latter by having no segmented rows.
 constexpr int64_t kServedMatrixBytes = 96 << 20;
+constexpr int64_t kLatencyBoundGatherBytes = (int64_t)8 << 30;
 constexpr int64_t kColdMatrixBytes = 128 << 20;   // 4x the L2 of the eight XCDs; the 42 MB matrix above is served, the 154 MB one (16 floats) is not
 int dst_wave_cap(const rof_layout *L, int64_t matrix_bytes, int64_t row_bytes, int64_t stride_bytes) {
     if (L->local_sources || L->n_segments == 0 || matrix_bytes < kColdMatrixBytes) return 0;
@@ -561,7 +562,14 @@ static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64
     int rc;
     // a feature matrix that the caches serve: more row gathers in flight in every launch (fp32 rows).  2^18-node
     // R-MAT graph against two in flight: 42 MB -8 %, 67 MB -7 %, 84 MB -2.8 %, 105 MB 0, 126 MB +1.9 %.
-    const bool deep = x_dtype == ROF_F32 && (L->tune_deep >= 0 ? L->tune_deep == 1 : (int64_t)L->n * ldx * esz < kServedMatrixBytes);
+    // That is a gain of launches bound by latency; a dense graph on a small matrix keeps the caches busy instead, and
+    // two in flight are as good or better from 8 GB gathered per launch (R-MAT, 233 000 nodes x 72 floats, average
+    // degree 435, 29 GB: 2.02 ms with four, 1.85 with two; 2^16 nodes x 160 floats, degree 341, 14 GB: 0.712 / 0.689;
+    // uniform degrees of 600: equal; below 8 GB four win by 1-20 %).
+    const bool deep = x_dtype == ROF_F32 &&
+                      (L->tune_deep >= 0 ? L->tune_deep == 1
+                                         : (int64_t)L->n * ldx * esz < kServedMatrixBytes &&
+                                               L->gathered_rows * (int64_t)feat * esz < kLatencyBoundGatherBytes);
     // launches 1 and 2: partial-sum rows (shared groups, then segments of long rows)
     const rof_phase_dev *partial[2] = {&L->dg, &L->ds};
     for (int i = 0; i < 2 && (launches & 1); ++i) {
