@@ -66,8 +66,9 @@ typedef struct {
     int32_t wave_cap;
     int32_t lds_pad;
     int32_t deep;          /* row gathers in flight per lane group: -1 = the library's choice (more of them when the */
-                           /* caches serve the whole fp32 feature matrix), 0 = two, 1 = four (five at 10 lanes per   */
-                           /* row) wherever such an instantiation exists (fp32 rows, 32-bit offsets)                 */
+                           /* caches serve the whole fp32 feature matrix and the launch gathers under 8 GB), 0 = two, */
+                           /* 1 = four (five at 10 lanes per row) wherever such an instantiation exists (fp32 rows,  */
+                           /* 32-bit offsets)                                                                        */
     int32_t reserved[3];
 } rof_launch_tuning;
 
