@@ -570,6 +570,8 @@ def main():
     # HIP runtime PyTorch brings; importing it does not initialise the device.)
     import torch
 
+    if torch.cuda.device_count() == 0:   # (counting devices does not initialise one)
+        sys.exit("bench.py needs a GPU: no HIP device is visible")
     d, t_gen, t_plan = load_or_build(name, ps, args.cache_dir)
     traffic = {"error": "switched off (--no-traffic / --quick) or non-default options"}
     if not args.no_traffic and default_opts:
