@@ -509,6 +509,7 @@ static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64
     if (x_dtype != ROF_F32 && x_dtype != ROF_BF16) return ROF_ERR_UNSUPPORTED;
     if (out_dtype != ROF_F32 && out_dtype != ROF_BF16) return ROF_ERR_UNSUPPORTED;
     if (((uintptr_t)out) % (out_dtype == ROF_F32 ? 4 : 2)) return ROF_ERR_ARG;
+    if (((uintptr_t)x) % (x_dtype == ROF_F32 ? 4 : 2) || ((uintptr_t)bias) % 4) return ROF_ERR_ARG;   // whole elements
     if (!L->uploaded || (normalized && !L->weights_set)) return ROF_ERR_STATE;
     if ((int64_t)L->n * ldx >= ((int64_t)1 << 40) || (int64_t)L->n * ldo >= ((int64_t)1 << 40)) return ROF_ERR_UNSUPPORTED;
     if (ldx >= ((int64_t)1 << 28) || feat >= (1 << 24)) return ROF_ERR_UNSUPPORTED;   // the kernel keeps row bytes in 32 bits

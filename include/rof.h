@@ -229,6 +229,7 @@ void rof_layout_free(rof_layout *layout);
  * w = s = 1 otherwise (sum aggregation: reuse_conv_kernel.cu:123-196), evaluated through the
  * layout's reuse groups.  x: [n, feat_dim] with row stride ldx (elements), out: float32
  * [n, feat_dim] with row stride ldo; every row of out is overwritten (no zero-fill needed).
+ * x, out and a bias start on a boundary of their element type (ROF_ERR_ARG otherwise), the workspace on 16 bytes.
  * The same call serves the backward pass on d_output because upstream runs the un-transposed
  * plan there (reuse_conv_kernel.cu:1021-1041).
  * ---------------------------------------------------------------------------------------- */

@@ -82,6 +82,32 @@ def test_error_codes_and_messages():
         _lib.check(-1)
 
 
+def test_operands_that_do_not_start_on_an_element_are_refused_before_any_launch():
+    """x, out and the bias must start on a boundary of their element type; the check comes before the layout's state
+    is looked at, so a layout that was never uploaded shows it (no HIP call is made)."""
+    import numpy as np
+    L = _lib.lib()
+    ip = np.arange(0, 9, 2, dtype=np.int32)                       # 4 nodes x 2 neighbours
+    ix = np.array([1, 2, 0, 3, 0, 3, 1, 2], dtype=np.int32)
+    pn = np.arange(4, dtype=np.int32)
+    p = lambda a: a.ctypes.data_as(C.c_void_p)
+    h = C.c_void_p()
+    assert L.rof_layout_from_parts(p(ix), p(ip), p(pn), 4, 4, 2, None, C.byref(h)) == 0
+    try:
+        buf = (C.c_float * 64)()
+        base = C.addressof(buf)
+        agg = lambda x, dt, out: L.rof_aggregate(h, C.c_void_p(x), dt, 4, C.c_void_p(out), 4, 4, 0, None, 0, None)
+        assert agg(base, 0, base + 64) == -5                      # aligned operands: only the upload is missing
+        assert agg(base + 2, 0, base + 64) == -1                  # fp32 rows from a 2-byte boundary
+        assert agg(base + 1, 1, base + 64) == -1                  # bf16 rows from an odd address
+        assert agg(base + 2, 1, base + 64) == -5                  # bf16 rows from a 2-byte boundary are fine
+        assert agg(base, 0, base + 66) == -1
+        ep = _lib.Epilogue(C.c_void_p(base + 130), 0, 0, 0.0)
+        assert L.rof_aggregate_epilogue(h, C.c_void_p(base), 0, 4, C.c_void_p(base + 64), 4, 4, 0, C.byref(ep), None, 0, None) == -1
+    finally:
+        L.rof_layout_free(h)
+
+
 def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(_lib, "_lib", None)
     monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/librof.so")
