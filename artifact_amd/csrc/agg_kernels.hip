@@ -11,6 +11,9 @@
 // (which may read group rows) -> partial-sum rows; every destination row -> out; and, for destinations that the
 // schedule has clustered around groups they share, one workgroup per cluster that sums those groups once into LDS
 // before it gathers the cluster's rows (rof_cluster_kernel).  There are no atomics: each output row has one writer.
+// On a small graph the layout keeps long rows whole instead of cutting them into segments, and the destination-row
+// launch is rof_coop_kernel: workgroups of sixteen wavefronts, one per long row (its wavefronts' sums meet in LDS),
+// the others running the remaining tasks as below -- one launch where segments would need two.
 //
 // Mapping to the machine:
 //   * the feature dimension runs across lanes, VEC consecutive elements per lane (one 16-byte
@@ -618,7 +621,14 @@ static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64
         a.n_tasks = L->db.n_regular;   // the clustered destinations at the end of the list have a launch of their own
         a.wave_cap = L->tune_wave_cap >= 0 ? L->tune_wave_cap
                                            : dst_wave_cap(L, (int64_t)L->n * ldx * esz, (int64_t)feat * esz, ldx * esz);
-        if ((rc = rofk::launch_rows(x_dtype != ROF_F32, a, phase, vec, off32, 0, st))) return rc;
+        // a small graph whose layout keeps long rows whole: one launch in which a workgroup of 16 wavefronts sums each
+        // of them (the kernel exists for fp32 rows gathered as 16-byte vectors; any other call runs the ordinary kernel,
+        // which sums such a row with one wavefront)
+        if (L->coop_tasks > 0 && x_dtype == ROF_F32 && vec == 4 && off32 && phase != 2)
+            rc = rofk::launch_rows_f32_coop(a, phase == 4, L->coop_tasks, st);
+        else
+            rc = rofk::launch_rows(x_dtype != ROF_F32, a, phase, vec, off32, 0, st);
+        if (rc) return rc;
         a.wave_cap = 0;
         if (L->db.lg_blocks > 0) {
             a.n_tasks = L->db.n_tasks;

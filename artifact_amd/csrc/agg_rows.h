@@ -601,6 +601,161 @@ __global__ __launch_bounds__(256) void rof_cluster_kernel(AggArgs a) {
     }
 }
 
+// The destination-row launch of a small graph (fp32 rows, short offsets).  A launch that cannot fill the machine lasts
+// as long as its longest chain of dependent gathers, and cutting long rows into segments shortens that chain only at
+// the price of a second, dependent launch (a quarter to a half of the whole on graphs of 2^14 ... 2^16 nodes).  Here
+// the workgroups are 16 wavefronts wide and the first n_coop of them take one long row each (the layout puts the
+// longest tasks first): every wavefront sums a sixteenth of the row's entries, the sixteen sums meet in LDS, and the
+// first wavefront adds them up and stores the row -- the chain of a segment, no partial row through memory and no
+// second launch.  The other workgroups run the remaining tasks exactly like rof_rows_kernel, sixteen wavefronts each.
+// DEEP: four row gathers in flight per lane group (five at 10 lanes per row) instead of two.
+constexpr int kCoopWaves = 16;
+
+template <int VEC, int LPR, bool DEEP>
+__global__ __launch_bounds__(64 * kCoopWaves) void rof_coop_kernel(AggArgs a, int32_t n_coop) {
+    typedef float XT;
+    constexpr int G = 64 / LPR;
+    constexpr int kU = DEEP ? (LPR % 4 == 0 ? 4 : LPR % 5 == 0 ? 5 : kGathersInFlight) : kGathersInFlight;
+    constexpr int PHASE = 1;
+    __shared__ float red[kCoopWaves][LPR * VEC];
+    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+    const int sub = lane / LPR, li = lane % LPR;
+    const bool idle = (G * LPR < 64) && lane >= G * LPR;   // lanes left over when LPR does not divide 64
+    const uint32_t xld = (uint32_t)(a.ldx * (int64_t)sizeof(XT)), pld = (uint32_t)(a.ldp * 4);
+    const int hw = blockIdx.x;
+
+    if (hw < n_coop) {   // one long row, summed by the whole workgroup (no thread leaves before the last barrier)
+        const int32_t t = hw;
+        const int32_t beg = a.task_ptr[t], end = a.task_ptr[t + 1];
+        const int32_t mid = beg + a.task_nref[t];
+        const int32_t out_row = a.task_out[t];
+        const float out_scale = a.task_scale ? a.task_scale[t] : 1.0f;
+        const int32_t share = (end - beg + kCoopWaves - 1) / kCoopWaves;
+        const int32_t wb = min(end, beg + wid * share), we = min(end, wb + share);
+        for (int c0 = 0; c0 < a.feat; c0 += LPR * VEC) {
+            const int cbase = c0 + li * VEC;
+            const bool act = !idle && cbase < a.feat;
+            const int cstart = (VEC > 1 && cbase + VEC > a.feat) ? a.feat - VEC : cbase;   // see rof_rows_kernel
+            const int skip = cbase - cstart;
+            const char *xb = reinterpret_cast<const char *>(a.x) + (size_t)cstart * sizeof(XT);
+            const char *pb = reinterpret_cast<const char *>(a.part) + (size_t)cstart * 4;
+            float acc[VEC];
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) acc[k] = 0.0f;
+            if (mid > beg)   // the row references partial rows of shared groups
+                gather_sum<XT, VEC, LPR, true, true, true, false, kU>(xb, xld, pb, pld, a.nsplit, 0, a.col, a.w, wb, we, lane, sub,
+                                                                     li, act, acc);
+            else
+                gather_sum<XT, VEC, LPR, true, false, true, false, kU>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, wb, we, lane, sub,
+                                                                      li, act, acc);
+            if ((G & (G - 1)) == 0) {
+#pragma unroll
+                for (int off = LPR; off < 64; off <<= 1) {
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) acc[k] += __shfl_xor(acc[k], off);
+                }
+            } else {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) {
+                    float tot = acc[k];
+#pragma unroll
+                    for (int g = 1; g < G; ++g)
+                        tot += __int_as_float(__builtin_amdgcn_ds_bpermute(lane_addr(li * 4, g * LPR * 4), __float_as_int(acc[k])));
+                    acc[k] = tot;
+                }
+            }
+            if (c0 > 0) __syncthreads();   // the previous chunk's sums have been read
+            if (act && sub == 0) {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) red[wid][li * VEC + k] = acc[k];
+            }
+            __syncthreads();
+            if (wid == 0 && act && sub == 0) {
+                float tot[VEC];
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) tot[k] = red[0][li * VEC + k];
+#pragma unroll
+                for (int w = 1; w < kCoopWaves; ++w) {
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) tot[k] += red[w][li * VEC + k];
+                }
+                finish_row<XT, VEC, PHASE>(a, out_row, out_scale, end > beg, tot, xb, xld, cstart, skip);
+            }
+        }
+        return;
+    }
+
+    // the remaining tasks: a wavefront each while they are long, a lane group each after that
+    const int hb = hw - n_coop;
+    const int xcd = hb % kXcds, nth = hb / kXcds;
+    const int run = a.xcd_run;
+    const int logical = ((nth / run) * kXcds + xcd) * run + (nth % run);
+    if (logical >= a.n_blocks) return;
+    const int gw = n_coop + logical * kCoopWaves + wid;
+    int32_t t, beg = 0, end = 0, mid = 0, out_row = 0;
+    float out_scale = 1.0f;
+    bool valid;
+    const bool wave_mode = gw < a.n_wave;
+    if (wave_mode) {
+        t = gw;
+        valid = true;
+    } else {
+        t = a.n_wave + (gw - a.n_wave) * G + sub;
+        valid = !idle && t < a.n_tasks;
+    }
+    if (valid) {
+        beg = a.task_ptr[t];
+        end = a.task_ptr[t + 1];
+        mid = beg + a.task_nref[t];
+        out_row = a.task_out[t];
+        if (a.task_scale) out_scale = a.task_scale[t];
+    }
+    for (int c0 = 0; c0 < a.feat; c0 += LPR * VEC) {
+        const int cbase = c0 + li * VEC;
+        const bool act = !idle && cbase < a.feat;
+        const int cstart = (VEC > 1 && cbase + VEC > a.feat) ? a.feat - VEC : cbase;
+        const int skip = cbase - cstart;
+        const char *xb = reinterpret_cast<const char *>(a.x) + (size_t)cstart * sizeof(XT);
+        const char *pb = reinterpret_cast<const char *>(a.part) + (size_t)cstart * 4;
+        float acc[VEC];
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) acc[k] = 0.0f;
+        if (wave_mode) {
+            if (mid > beg)
+                gather_sum<XT, VEC, LPR, true, true, true, false, kU>(xb, xld, pb, pld, a.nsplit, 0, a.col, a.w, beg, end, lane, sub,
+                                                                     li, act, acc);
+            else
+                gather_sum<XT, VEC, LPR, true, false, true, false, kU>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, beg, end, lane, sub,
+                                                                      li, act, acc);
+            if ((G & (G - 1)) == 0) {
+#pragma unroll
+                for (int off = LPR; off < 64; off <<= 1) {
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) acc[k] += __shfl_xor(acc[k], off);
+                }
+            } else {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) {
+                    float tot = acc[k];
+#pragma unroll
+                    for (int g = 1; g < G; ++g)
+                        tot += __int_as_float(__builtin_amdgcn_ds_bpermute(lane_addr(li * 4, g * LPR * 4), __float_as_int(acc[k])));
+                    acc[k] = tot;
+                }
+            }
+        } else {
+            if (__any(mid > beg))
+                gather_sum<XT, VEC, LPR, false, true, true, false, kU>(xb, xld, pb, pld, a.nsplit, 0, a.col, a.w, beg, end, lane, sub,
+                                                                      li, act, acc);
+            else
+                gather_sum<XT, VEC, LPR, false, false, true, false, kU>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, beg, end, lane, sub,
+                                                                       li, act, acc);
+        }
+        if (valid && act && (!wave_mode || sub == 0))
+            finish_row<XT, VEC, PHASE>(a, out_row, out_scale, end > beg, acc, xb, xld, cstart, skip);
+    }
+}
+
 // Lanes one gathered row occupies: the smallest supported count that covers ceil(feat / vec).  Counts
 // that do not divide 64 (10, 12, 20) leave 4 lanes idle but fit 6, 5 or 3 rows into one load instruction
 // where the next power of two would fit 4, 4 or 2.
@@ -673,14 +828,46 @@ int launch_lpr(const AggArgs &a0, int lpr, int lds_rows, hipStream_t st) {
     return ROF_OK;
 }
 
+template <bool DEEP>
+int launch_coop(const AggArgs &a0, int lpr, int32_t n_coop, hipStream_t st) {
+    AggArgs a = a0;
+    const int g = 64 / lpr;
+    if (n_coop < 0 || n_coop > a.n_wave || a.n_wave > a.n_tasks) return ROF_ERR_ARG;
+    const int64_t waves = (int64_t)(a.n_wave - n_coop) + ((int64_t)a.n_tasks - a.n_wave + g - 1) / g;
+    a.n_blocks = (int32_t)((waves + kCoopWaves - 1) / kCoopWaves);
+    a.xcd_run = std::max(1, a.xcd_run / (kCoopWaves / kWavesPerBlock));   // runs counted in workgroups four times as wide
+    const int64_t span = (int64_t)kXcds * a.xcd_run;
+    const int64_t grid = n_coop + (a.n_blocks + span - 1) / span * span;
+    if (grid == 0) return ROF_OK;
+    dim3 gr((unsigned)grid), bl(64 * kCoopWaves);
+#define ROF_LAUNCH(LPR) hipLaunchKernelGGL((rof_coop_kernel<4, LPR, DEEP>), gr, bl, 0, st, a, n_coop)
+    switch (lpr) {
+        case 4: ROF_LAUNCH(4); break;
+        case 8: ROF_LAUNCH(8); break;
+        case 10: ROF_LAUNCH(10); break;
+        case 12: ROF_LAUNCH(12); break;
+        case 16: ROF_LAUNCH(16); break;
+        case 20: ROF_LAUNCH(20); break;
+        case 32: ROF_LAUNCH(32); break;
+        default: ROF_LAUNCH(64); break;
+    }
+#undef ROF_LAUNCH
+    HIP_TRY(hipGetLastError());
+    return ROF_OK;
+}
+
 // Instantiated in agg_rows_{f32,bf16}_partial.hip (partial-sum launches; phase 0, 3 or 5 / stream: phase 3), agg_rows_{f32,bf16}_dst.hip (destination
-// rows; phase 1, or 2 = streaming stores) and agg_cluster_{f32,bf16}.hip (the clustered destination rows: a.n_blocks
-// clusters whose workgroups need lds_rows LDS rows), one translation unit each so that the build runs them side by side.
+// rows; phase 1, or 2 = streaming stores), agg_cluster_{f32,bf16}.hip (the clustered destination rows: a.n_blocks
+// clusters whose workgroups need lds_rows LDS rows) and agg_coop_f32.hip (the destination rows of a small graph), one
+// translation unit each so that the build runs them side by side.
 // off32: every byte offset into the feature matrix and into the partial-sum workspace fits 32 bits and
 // every row id fits 24 bits, so the kernels may use the short address arithmetic.
 int launch_rows_f32_partial(const AggArgs &a, int phase, int vec, bool off32, hipStream_t st);
 int launch_rows_f32_dst(const AggArgs &a, int phase, int vec, bool off32, hipStream_t st);
 int launch_rows_f32_cluster(const AggArgs &a, int phase, int vec, bool off32, int lds_rows, hipStream_t st);
+// agg_coop_f32.hip: the destination-row launch of a small graph whose first n_coop tasks get a workgroup each
+// (rof_coop_kernel; fp32 rows gathered as 16-byte vectors with short offsets); a.n_tasks: the tasks of this launch
+int launch_rows_f32_coop(const AggArgs &a, bool deep, int32_t n_coop, hipStream_t st);
 int launch_rows_bf16_partial(const AggArgs &a, bool stream, int vec, bool off32, hipStream_t st);
 int launch_rows_bf16_dst(const AggArgs &a, int phase, int vec, bool off32, hipStream_t st);
 int launch_rows_bf16_cluster(const AggArgs &a, int phase, int vec, bool off32, int lds_rows, hipStream_t st);

@@ -32,6 +32,12 @@ typedef std::vector<int32_t> ivec;
 // by its longest task instead and keeps the lower cut (16 384 rows: 18 us against 26).
 const int32_t kShortRow = 64, kShortRowSmall = 32;
 const int64_t kWavesToFill = 2 * 8192;   // two rounds of 256 CUs x 32 wavefronts
+// Rows that a whole workgroup sums on small launches: more entries than kCoopRow, at most kCoopMaxRows of them (each
+// takes the 16 wavefronts of a workgroup, kCoopWaves in agg_rows.h: 2^14 nodes x 32 floats, 106 rows beyond 256 entries
+// 6.4 us, 468 beyond 128 entries 9.4, two launches with segments 10.7; 2^16 nodes, 697 rows beyond 256 entries: 26.4 us
+// against 22.5 with segments), the longest of at most kCoopChain entries per lane group (2486 entries at two rows per
+// wavefront, 78 per lane group: 15.7 us against 18.9).
+const int32_t kCoopRow = 256, kCoopWaves = 16, kCoopChain = 96, kCoopMaxRows = 256;
 // Long rows.  Rows longer than a cut are gathered in segments that fill partial rows one launch earlier, and
 // the segment tasks of all rows run in the order of the highest source id they gather (entries inside a task are
 // listed by descending id): every wavefront in flight then works in the same narrow band of the feature matrix
@@ -524,6 +530,22 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
                                                   : std::max<int32_t>(16, (int64_t)hub_split * rule_segment / rule_cut);
     L->hub_split = hub_split;
     L->segment = segment;
+    // Small launches (fp32 rows, the library's own cut): no row is cut.  The destination-row launch runs workgroups of
+    // 16 wavefronts and gives every row of more than kCoopRow entries a whole workgroup, whose wavefronts each sum a
+    // sixteenth of it and combine in LDS: the chain of dependent gathers of a segment without the second launch that
+    // segments need (2^14 nodes x 32 floats: two launches of 5-6 us each).  Only while the longest row leaves a lane
+    // group at most kCoopChain entries; a longer one is better off spread over the machine in segments.
+    bool coop = false;
+    if (!(o && (o->hub_split > 0 || o->segment > 0 || o->share_scope == 1)) && elem_bytes == 4 && n / groups < kWavesToFill) {
+        int32_t longest = 0;
+        int64_t long_rows = 0;
+        for (int32_t v = 0; v < n; ++v) {
+            longest = std::max(longest, len_all[v]);
+            long_rows += len_all[v] > kCoopRow;
+        }
+        coop = long_rows > 0 && long_rows <= kCoopMaxRows && longest <= (int64_t)kCoopWaves * groups * kCoopChain;
+    }
+    const int32_t cut_rows = coop ? INT32_MAX : hub_split;   // rows beyond this are cut into segments
     // Partial rows are cold when the row that adds them up reads them (written one launch earlier, each read once): an
     // entry of that chain costs about twice the cached figure -- and never less than a memory latency (700 ns) shared by
     // the two reads that each of the wavefront's `groups` lane groups keeps in flight, which is what counts at wide
@@ -590,12 +612,12 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
         full_len.swap(len_all);
         for (int32_t v = 0; v < n; ++v) {
             const int64_t len = full_len[v];
-            const int64_t task_len = len > hub_split ? (len + segment - 1) / segment : len;
+            const int64_t task_len = len > cut_rows ? (len + segment - 1) / segment : len;
             over += task_len > kShortRow;
         }
     }
     // share_scope 1: only rows that will be cut into segments read shared groups from the workspace
-    auto in_scope = [&](int32_t v) { return share_scope != 1 || full_len[v] > hub_split; };
+    auto in_scope = [&](int32_t v) { return share_scope != 1 || full_len[v] > cut_rows; };
     if (!disable && min_consumers == 0 && local_groups >= 0 && G > 0) {
         // sharing only shortens rows, so a row that is short now stays short, and rows above the segment cut are
         // no candidates
@@ -609,7 +631,7 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
         // without it every cluster that saves kMinClusterSaving gathers pays -- planted sets of 3 anchors x 64 members
         // + 24 random neighbours, 16 % of the gathers removable: 1.056 ms with reuse disabled, 1.082 with the clusters
         // that pass the relative gate, 0.960 with all of them)
-        build_clusters(L, ng_ptr, ng, full_len, std::min(cut, hub_split), groups, max_rows, local_groups > 0 ? local_groups : kMinClusterSaving,
+        build_clusters(L, ng_ptr, ng, full_len, std::min(cut, cut_rows), groups, max_rows, local_groups > 0 ? local_groups : kMinClusterSaving,
                        local_groups == 0 && sources_are_local(), cl);
         for (int32_t v = 0; v < n; ++v)
             if (cl.of_node[v] >= 0)
@@ -705,7 +727,7 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
         reads += refs;
         lds_reads += nlds;
         tb.begin_task(v);
-        if (len > hub_split) {
+        if (len > cut_rows) {
             // A long row is cut into segments; each becomes a partial-sum task of the middle launch
             // (after the groups it may reference, before the rows), and the row itself just adds them up.
             // (Rows served from LDS are short: nlds is 0 here.)
@@ -751,6 +773,10 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     finalize_phase(tg, 1 << 30, groups, false, L->g);
     finalize_phase(ts, 1 << 30, groups, entry_order == 0, L->s);   // the sweep needs the descending lists
     finalize_phase(tb, tile_rows, groups, false, L->b, &cl);
+    L->coop_tasks = 0;
+    if (coop)   // the long tasks come first, longest first
+        while (L->coop_tasks < L->b.n_wave && L->b.task_ptr[L->coop_tasks + 1] - L->b.task_ptr[L->coop_tasks] > kCoopRow)
+            ++L->coop_tasks;
     L->n_local_groups = (int64_t)cl.lg_task_ptr.size() - 1;
     L->lds_reads = lds_reads;
     L->gathered_before_rows = (int64_t)tg.col.size();
@@ -990,14 +1016,15 @@ int rof_layout_export(const rof_layout *L, rof_bag **out) {
 
 int rof_layout_stats_n(const rof_layout *L, int64_t *stats, int count) {
     if (!L || !stats || count < 0) return ROF_ERR_ARG;
-    int64_t s[23];
+    int64_t s[24];
     int rc = rof_layout_stats(L, s);
     if (rc) return rc;
     s[20] = L->hub_split;
     s[21] = L->segment;
     s[22] = 0;   // longest task of the destination-row launch
     for (int32_t t = 0; t < L->b.n_tasks; ++t) s[22] = std::max<int64_t>(s[22], L->b.task_ptr[t + 1] - L->b.task_ptr[t]);
-    for (int i = 0; i < count; ++i) stats[i] = i < 23 ? s[i] : 0;
+    s[23] = L->coop_tasks;
+    for (int i = 0; i < count; ++i) stats[i] = i < 24 ? s[i] : 0;
     return ROF_OK;
 }
 

@@ -19,7 +19,7 @@ NOALLOC_WORKSPACE_BYTES = 64 << 20   # ROF_NOALLOC_WORKSPACE_BYTES of include/ro
 STAT_NAMES = ("nodes", "edges", "groups", "materialised_groups", "gathered_rows", "partial_reads", "partial_rows",
               "hub_segments", "tasks_a", "tasks_b", "device_bytes", "part_size", "wave_tasks_a", "wave_tasks_b",
               "canonical", "gathered_rows_a", "local_groups", "lds_reads", "cluster_workgroups", "lds_rows", "hub_split",
-              "segment", "longest_row_task")
+              "segment", "longest_row_task", "workgroup_rows")
 
 EXPORT_NAMES = ("group_ptr", "group_col", "group_dst_ptr", "group_dst", "res_ptr", "res_col", "canonical", "xcd_run", "long_row_cut",
                 "uniqpart_column_index", "uniqpart_pointers", "part2Node_ptr", "part2Node_col",

@@ -311,7 +311,8 @@ def read_counter_csv(path):
     """One rocprofv3 counter_collection.csv of a counter run -> ({(counter, phase): value per aggregation},
     {counter: value of the calibration copy}).  Phase 0 = the partial-sum launches (shared groups, segments of long
     rows; template argument PHASE of the kernel name <XT, VEC, LPR, PHASE, OFF32> is 0, 3 with streamed partial
-    rows or 5 with more gathers in flight), phase 1 = the destination rows and their clusters (PHASE 1, 2 or 4).  A phase may consist of two launches, so the dispatches of one phase are summed and divided
+    rows or 5 with more gathers in flight), phase 1 = the destination rows and their clusters (PHASE 1, 2 or 4, or
+    rof_coop_kernel on small graphs).  A phase may consist of two launches, so the dispatches of one phase are summed and divided
     by the number of aggregations the run executes."""
     acc, copy = collections.defaultdict(float), {}
     with open(path) as f:
@@ -319,6 +320,8 @@ def read_counter_csv(path):
             k = row["Kernel_Name"]
             if "rof_copy_kernel" in k:
                 copy[row["Counter_Name"]] = float(row["Counter_Value"])
+            elif "rof_coop_kernel" in k:   # the destination-row launch of a small graph (long rows: a workgroup each)
+                acc[(row["Counter_Name"], 1)] += float(row["Counter_Value"])
             elif "rof_rows_kernel" in k or "rof_cluster_kernel" in k:
                 phase = int(k.split("<")[1].split(">")[0].split(",")[3])
                 if phase not in (0, 1, 2, 3, 4, 5):
@@ -948,7 +951,8 @@ def main():
         "config": {"workload": DESCR[name], "nodes": n, "edges": e, "feat": feat, "row_stride": ld, "out_row_stride": ldo,
                    "output": "padded rows (pad_columns)" if pad else "packed [N, feat], as the operator API returns it",
                    "part_size": ps, "normalized": normalized, "search": args.search},
-        "roofline": roof(1, "rof_rows_kernel (destination-row launch)", bytes_b, ms_b),
+        "roofline": roof(1, ("rof_coop_kernel (destination-row launch of a small graph: long rows get a workgroup each)"
+                             if st.get("workgroup_rows") else "rof_rows_kernel (destination-row launch)"), bytes_b, ms_b),
         # the launch before it (segments of long rows, swept in the order of their source ids): same kernel
         # template, second in duration
         "roofline_partial_launch": roof(0, "rof_rows_kernel (partial-sum launch)", bytes_a, ms_a),

@@ -139,7 +139,11 @@ typedef struct {
                              /* >= 1024 bytes; otherwise up to G = 3 128 within and 1024 beyond 256 MB; 1024 at   */
                              /* G = 4; 640 from 5 on; bfloat16 rows 256 for G <= 2, 512 at 3, 1280 above; lower     */
                              /* (down to 128) on launches so small that a row of that length would outlast them,   */
-                             /* and adjusted on dense graphs by what their rows look like (see layout.cpp)          */
+                             /* and adjusted on dense graphs by what their rows look like (see layout.cpp).  With    */
+                             /* 0 here and in `segment`, a small graph of float32 rows (fewer than 16 384 wavefronts */
+                             /* of rows, at most 256 rows beyond 256 entries, none beyond 1536 per row that a        */
+                             /* wavefront gathers at once) keeps its long rows whole: the destination-row launch then */
+                             /* sums each of them with a workgroup of 16 wavefronts, and there is no earlier launch  */
     int32_t segment;         /* entries per segment; 0 = an eighth to a quarter of hub_split (see layout.cpp).  A row  */
                              /* so long that adding up its segments would outlast the launch gets longer ones.    */
     int32_t lanes_per_row;   /* lanes one gathered row occupies in the kernel that will use this layout:   */
@@ -207,7 +211,8 @@ int rof_layout_export(const rof_layout *layout, rof_bag **out);
 int rof_layout_stats(const rof_layout *layout, int64_t stats[20]);
 /* The first `count` of the counters the library knows (fewer: the rest is dropped; more: zero-filled): the twenty
  * above, then [20] the cut of long rows (hub_split) and [21] the segment length as chosen for this layout, [22] the
- * entries of the longest task of the destination-row launch. */
+ * entries of the longest task of the destination-row launch, [23] the rows that the destination-row launch of a small
+ * graph sums with a whole workgroup each (0: long rows are cut into segments as [20] and [21] say). */
 int rof_layout_stats_n(const rof_layout *layout, int64_t *stats, int count);
 
 /* Copy the schedule to the current HIP device (idempotent). */

@@ -130,6 +130,57 @@ def test_dense_graphs_and_rows_of_the_whole_graph(oracle, kind, feat, bf16):
     _close(got, want, oracle.closed_form(indptr, indices, np.abs(x), np.diff(indptr).astype(np.float32)))
 
 
+@pytest.mark.parametrize("scale_down,feat,opts", [(0, 3, {}), (0, 16, {}), (0, 32, {}), (0, 40, {}), (0, 47, {}), (0, 64, {}), (0, 72, {}),
+                                                  (0, 128, {}), (2, 256, {}), (2, 300, {}), (0, 32, dict(min_consumers=2)),
+                                                  (0, 47, dict(disable_reuse=True))])
+def test_long_rows_of_small_graphs_are_summed_by_a_workgroup_each(oracle, scale_down, feat, opts):
+    """On a launch that cannot fill the machine the layout keeps long rows whole and the destination-row launch gives
+    each of them a workgroup of sixteen wavefronts (one launch instead of two): every lane count, rows of more than one
+    chunk of columns, rows that reference partial rows of shared groups, the layer's epilogue, and the same rows through
+    the ordinary kernels (the layout with an explicit cut; rows of three floats, which only scalar loads can read and
+    the ordinary kernel therefore sums uncut)."""
+    indptr, indices, plan = _case("c1", scale_down, 3)
+    n = len(indptr) - 1
+    deg = np.diff(indptr).astype(np.float32)
+    x = features(n, feat, seed=21)
+    ld = -(-feat // 4) * 4
+    xt = torch.zeros((n, ld), device="cuda")[:, :feat]
+    xt.copy_(torch.from_numpy(x))
+    lay = _layout(plan, n, 3, lanes_per_row=lanes_per_row(feat), row_bytes=ld * 4, **opts)
+    st = lay.stats()
+    assert st["workgroup_rows"] > 0 and st["hub_segments"] == 0, st
+    assert st["longest_row_task"] > st["hub_split"]                           # a row that the rule would have cut
+    cut = _layout(plan, n, 3, lanes_per_row=lanes_per_row(feat), row_bytes=ld * 4, hub_split=st["hub_split"],
+                  segment=st["segment"], **opts)
+    assert cut.stats()["workgroup_rows"] == 0 and cut.stats()["hub_segments"] > 0
+    d = torch.from_numpy(deg).cuda()
+    lay.set_degrees(d)
+    cut.set_degrees(d)
+    want = oracle.closed_form(indptr, indices, x, deg)
+    mag = oracle.closed_form(indptr, indices, np.abs(x), deg)
+    got = lay.aggregate(xt, normalized=True, feat_dim=feat)
+    _close(got.cpu().numpy(), want, mag)
+    _close(cut.aggregate(xt, normalized=True, feat_dim=feat).cpu().numpy(), want, mag)
+    assert torch.equal(got, lay.aggregate(xt, normalized=True, feat_dim=feat))           # run to run
+    # two gathers in flight instead of four: the other instantiation, the same sums
+    lay.set_tuning(deep=0)
+    _close(lay.aggregate(xt, normalized=True, feat_dim=feat).cpu().numpy(), want, mag)
+    lay.set_tuning()
+    # epilogue on the workgroup's store: own row, bias, ReLU, bf16
+    bias = torch.from_numpy(features(1, feat, seed=22)[0]).cuda()
+    full = lay.aggregate(xt, normalized=True, feat_dim=feat, bias=bias, relu=True, self_weight=0.5)
+    sep = torch.relu(got + 0.5 * xt + bias)
+    assert torch.allclose(full, sep, rtol=1e-5, atol=1e-5)
+    half = lay.aggregate(xt, normalized=True, feat_dim=feat, out_dtype=torch.bfloat16)
+    assert torch.equal(half, got.to(torch.bfloat16))
+    # sum aggregation
+    plain = lay.aggregate(xt, normalized=False, feat_dim=feat).cpu().numpy()
+    _close(plain, oracle.closed_form(indptr, indices, x, None, normalized=False),
+           oracle.closed_form(indptr, indices, np.abs(x), None, normalized=False))
+    lay.close()
+    cut.close()
+
+
 @pytest.mark.parametrize("feat,ld,shift", [(47, 47, 0), (5, 5, 0), (7, 9, 1), (101, 101, 3), (255, 255, 0), (2, 2, 1)])
 def test_packed_and_misaligned_rows(oracle, feat, ld, shift):
     """Rows that start on arbitrary 4-byte boundaries (packed widths, odd strides, an offset base pointer):

@@ -383,6 +383,42 @@ def test_small_launches_cut_long_rows_lower():
     assert cut_of(ip, ix, lanes_per_row=32, elem_bytes=2) == (256, 48)      # 307 MB of bf16 rows
 
 
+def test_small_graphs_keep_long_rows_whole_for_a_workgroup_each():
+    """A small launch (fp32 rows, the library's own cut) with at most 256 rows of more than 256 entries, the longest of
+    at most 16 x 96 entries per lane group, keeps those rows whole: they lead the task list (longest first) and the
+    launch gives each a workgroup of sixteen wavefronts.  No segment, no partial row, no second launch; the cut the
+    rule would have used is still reported."""
+    ip, ix = make_workload("c1", 0)                          # 2^14 rows, 106 of them beyond 256 entries, the longest 2486
+    deg = np.diff(ip)
+    lay = Layout.from_csr(ip, ix, lanes_per_row=8)
+    st, ex = lay.stats(), lay.export()
+    assert st["workgroup_rows"] == int((deg > 256).sum()) == 106 and st["hub_segments"] == 0 and st["partial_rows"] == 0
+    assert (st["hub_split"], st["segment"]) == (256, 128) and st["longest_row_task"] == deg.max()
+    lens = np.diff(ex["b_task_ptr"])
+    assert (lens[:106] > 256).all() and (lens[106:] <= 256).all() and (np.diff(lens[:106].astype(np.int64)) <= 0).all()
+    assert sorted(ex["b_task_out"][:106].tolist()) == sorted(np.nonzero(deg > 256)[0].tolist())
+    # every entry of every row is still there
+    assert len(ex["b_col"]) == len(ix) and st["gathered_rows"] == len(ix)
+    # a caller's cut, bf16 rows, or a scope that needs segments: the segments stay
+    for kw in (dict(hub_split=256), dict(segment=64), dict(elem_bytes=2), dict(share_scope="long_rows")):
+        st = Layout.from_csr(ip, ix, lanes_per_row=8, **kw).stats()
+        assert st["workgroup_rows"] == 0 and st["hub_segments"] > 0, kw
+    # one row per wavefront: 2^14 rows are no small launch, and 2486 entries would be 155 per lane group
+    assert Layout.from_csr(ip, ix, lanes_per_row=64).stats()["workgroup_rows"] == 0
+    # too many long rows for a workgroup each (697 beyond 256 entries): segments
+    ip, ix = rmat_csr(1 << 16, 24, seed=91, a=0.5, b=0.2, c=0.2)
+    st = Layout.from_csr(ip, ix, lanes_per_row=8).stats()
+    assert int((np.diff(ip) > 256).sum()) > 256 and st["workgroup_rows"] == 0 and st["hub_segments"] > 0
+    # a row too long for one workgroup: 2^13 nodes, one of which every node is a neighbour of
+    n = 1 << 13
+    u = np.concatenate([np.arange(n), np.zeros(n, np.int64), np.arange(n)])
+    v = np.concatenate([(np.arange(n) + 1) % n, np.arange(n), np.zeros(n, np.int64)])
+    ip, ix = csr_from_pairs(u, v, n, False)
+    st = Layout.from_csr(ip, ix, lanes_per_row=32).stats()   # two rows per wavefront: at most 3072 entries
+    assert st["workgroup_rows"] == 0 and st["hub_segments"] > 0
+    assert Layout.from_csr(ip, ix, lanes_per_row=8).stats()["workgroup_rows"] == 1      # 12 288 at eight
+
+
 def test_xcd_run_follows_the_locality_of_the_graph():
     """Block-structured graphs (rows gather from their own neighbourhood) keep a whole tile of destinations on
     one XCD; graphs without that locality use short runs."""
