@@ -213,6 +213,8 @@ class Layout:
         self.num_nodes = int(num_nodes)
         self._deg_key = None
         self._workspace = None
+        self._uploaded = False               # the library's upload is idempotent; this saves the call on every launch
+        self._ws_bytes = {}                  # feat_dim -> bytes of partial-sum rows (fixed once the layout is built)
 
     # ---- construction -------------------------------------------------------------------
     @classmethod
@@ -299,7 +301,9 @@ class Layout:
 
     # ---- device side ---------------------------------------------------------------------
     def upload(self, stream=0):
-        check(_lib.lib().rof_layout_upload(self._h, C.c_void_p(stream)))
+        if not self._uploaded:
+            check(_lib.lib().rof_layout_upload(self._h, C.c_void_p(stream)))
+            self._uploaded = True
         return self
 
     def set_degrees(self, degrees, stream=None):
@@ -321,7 +325,11 @@ class Layout:
         return self
 
     def workspace_bytes(self, feat_dim):
-        return int(_lib.lib().rof_layout_workspace_bytes(self._h, int(feat_dim)))
+        f = int(feat_dim)
+        need = self._ws_bytes.get(f)
+        if need is None:
+            need = self._ws_bytes[f] = int(_lib.lib().rof_layout_workspace_bytes(self._h, f))
+        return need
 
     def _args(self, x, out, feat_dim, workspace, out_dtype=None):
         import torch
