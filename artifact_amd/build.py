@@ -20,7 +20,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "librof.so")
 
 HOST_SOURCES = ["plan_builder.cpp", "hub_patterns.cpp", "dynamic_greedy.cpp", "layout.cpp"]
-HIP_SOURCES = ["agg_kernels.hip", "agg_rows_f32_partial.hip", "agg_rows_f32_dst.hip", "agg_cluster_f32.hip", "agg_coop_f32.hip",
+HIP_SOURCES = ["agg_kernels.hip", "agg_rows_f32_partial.hip", "agg_rows_f32_dst.hip", "agg_cluster_f32.hip", "agg_coop_f32.hip", "agg_coop_bf16.hip",
                "agg_rows_bf16_partial.hip", "agg_rows_bf16_dst.hip", "agg_cluster_bf16.hip"]
 
 # packed fp32 instructions stay off: the compiler must not form v_pk_{add,mul,fma}_f32

@@ -622,10 +622,11 @@ static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64
         a.wave_cap = L->tune_wave_cap >= 0 ? L->tune_wave_cap
                                            : dst_wave_cap(L, (int64_t)L->n * ldx * esz, (int64_t)feat * esz, ldx * esz);
         // a small graph whose layout keeps long rows whole: one launch in which a workgroup of 16 wavefronts sums each
-        // of them (the kernel exists for fp32 rows gathered as 16-byte vectors; any other call runs the ordinary kernel,
-        // which sums such a row with one wavefront)
-        if (L->coop_tasks > 0 && x_dtype == ROF_F32 && vec == 4 && off32 && phase != 2)
-            rc = rofk::launch_rows_f32_coop(a, phase == 4, L->coop_tasks, st);
+        // of them (the kernel exists for rows gathered as 16-byte vectors with short offsets; any other call runs the
+        // ordinary kernel, which sums such a row with one wavefront)
+        if (L->coop_tasks > 0 && vec == wide && off32 && phase != 2)
+            rc = x_dtype == ROF_F32 ? rofk::launch_rows_f32_coop(a, phase == 4, L->coop_tasks, st)
+                                    : rofk::launch_rows_bf16_coop(a, L->coop_tasks, st);
         else
             rc = rofk::launch_rows(x_dtype != ROF_F32, a, phase, vec, off32, 0, st);
         if (rc) return rc;

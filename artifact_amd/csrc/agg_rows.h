@@ -608,13 +608,13 @@ __global__ __launch_bounds__(256) void rof_cluster_kernel(AggArgs a) {
 // longest tasks first): every wavefront sums a sixteenth of the row's entries, the sixteen sums meet in LDS, and the
 // first wavefront adds them up and stores the row -- the chain of a segment, no partial row through memory and no
 // second launch.  The other workgroups run the remaining tasks exactly like rof_rows_kernel, sixteen wavefronts each.
-// DEEP: four row gathers in flight per lane group (five at 10 lanes per row) instead of two.
+// DEEP: four row gathers in flight per lane group (five at 10 lanes per row) instead of two (fp32 rows).
 constexpr int kCoopWaves = 16;
 
-template <int VEC, int LPR, bool DEEP>
+template <typename XT, int VEC, int LPR, bool DEEP>
 __global__ __launch_bounds__(64 * kCoopWaves) void rof_coop_kernel(AggArgs a, int32_t n_coop) {
-    typedef float XT;
     constexpr int G = 64 / LPR;
+    constexpr bool kF32 = sizeof(XT) == 4;   // fp32 features: partial rows have the same element type
     constexpr int kU = DEEP ? (LPR % 4 == 0 ? 4 : LPR % 5 == 0 ? 5 : kGathersInFlight) : kGathersInFlight;
     constexpr int PHASE = 1;
     __shared__ float red[kCoopWaves][LPR * VEC];
@@ -642,12 +642,20 @@ __global__ __launch_bounds__(64 * kCoopWaves) void rof_coop_kernel(AggArgs a, in
             float acc[VEC];
 #pragma unroll
             for (int k = 0; k < VEC; ++k) acc[k] = 0.0f;
-            if (mid > beg)   // the row references partial rows of shared groups
-                gather_sum<XT, VEC, LPR, true, true, true, false, kU>(xb, xld, pb, pld, a.nsplit, 0, a.col, a.w, wb, we, lane, sub,
-                                                                     li, act, acc);
-            else
-                gather_sum<XT, VEC, LPR, true, false, true, false, kU>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, wb, we, lane, sub,
-                                                                      li, act, acc);
+            if (kF32) {
+                if (mid > beg)   // the row references partial rows of shared groups
+                    gather_sum<XT, VEC, LPR, true, true, true, false, kU>(xb, xld, pb, pld, a.nsplit, 0, a.col, a.w, wb, we, lane,
+                                                                         sub, li, act, acc);
+                else
+                    gather_sum<XT, VEC, LPR, true, false, true, false, kU>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, wb, we, lane,
+                                                                          sub, li, act, acc);
+            } else {   // bf16 features: the references (fp32 partial rows) come first in the row's list
+                if (mid > wb)
+                    gather_sum<float, VEC, LPR, true, false, true, false, kU>(pb, pld, nullptr, 0, 0, a.nsplit, a.col, a.w, wb,
+                                                                             min(we, mid), lane, sub, li, act, acc);
+                gather_sum<XT, VEC, LPR, true, false, true, false, kU>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, max(wb, mid), we, lane,
+                                                                      sub, li, act, acc);
+            }
             if ((G & (G - 1)) == 0) {
 #pragma unroll
                 for (int off = LPR; off < 64; off <<= 1) {
@@ -721,12 +729,20 @@ __global__ __launch_bounds__(64 * kCoopWaves) void rof_coop_kernel(AggArgs a, in
 #pragma unroll
         for (int k = 0; k < VEC; ++k) acc[k] = 0.0f;
         if (wave_mode) {
-            if (mid > beg)
-                gather_sum<XT, VEC, LPR, true, true, true, false, kU>(xb, xld, pb, pld, a.nsplit, 0, a.col, a.w, beg, end, lane, sub,
-                                                                     li, act, acc);
-            else
-                gather_sum<XT, VEC, LPR, true, false, true, false, kU>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, beg, end, lane, sub,
+            if (kF32) {
+                if (mid > beg)
+                    gather_sum<XT, VEC, LPR, true, true, true, false, kU>(xb, xld, pb, pld, a.nsplit, 0, a.col, a.w, beg, end, lane,
+                                                                         sub, li, act, acc);
+                else
+                    gather_sum<XT, VEC, LPR, true, false, true, false, kU>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, beg, end, lane,
+                                                                          sub, li, act, acc);
+            } else {
+                if (mid > beg)
+                    gather_sum<float, VEC, LPR, true, false, true, false, kU>(pb, pld, nullptr, 0, 0, a.nsplit, a.col, a.w, beg,
+                                                                             mid, lane, sub, li, act, acc);
+                gather_sum<XT, VEC, LPR, true, false, true, false, kU>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, mid, end, lane, sub,
                                                                       li, act, acc);
+            }
             if ((G & (G - 1)) == 0) {
 #pragma unroll
                 for (int off = LPR; off < 64; off <<= 1) {
@@ -743,13 +759,19 @@ __global__ __launch_bounds__(64 * kCoopWaves) void rof_coop_kernel(AggArgs a, in
                     acc[k] = tot;
                 }
             }
-        } else {
+        } else if (kF32) {
             if (__any(mid > beg))
                 gather_sum<XT, VEC, LPR, false, true, true, false, kU>(xb, xld, pb, pld, a.nsplit, 0, a.col, a.w, beg, end, lane, sub,
                                                                       li, act, acc);
             else
                 gather_sum<XT, VEC, LPR, false, false, true, false, kU>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, beg, end, lane, sub,
                                                                        li, act, acc);
+        } else {
+            if (__any(mid > beg))
+                gather_sum<float, VEC, LPR, false, false, true, false, kU>(pb, pld, nullptr, 0, 0, a.nsplit, a.col, a.w, beg, mid,
+                                                                          lane, sub, li, act, acc);
+            gather_sum<XT, VEC, LPR, false, false, true, false, kU>(xb, xld, nullptr, 0, 0, 0, a.col, a.w, mid, end, lane, sub, li,
+                                                                   act, acc);
         }
         if (valid && act && (!wave_mode || sub == 0))
             finish_row<XT, VEC, PHASE>(a, out_row, out_scale, end > beg, acc, xb, xld, cstart, skip);
@@ -828,7 +850,7 @@ int launch_lpr(const AggArgs &a0, int lpr, int lds_rows, hipStream_t st) {
     return ROF_OK;
 }
 
-template <bool DEEP>
+template <typename XT, int VEC, bool DEEP>
 int launch_coop(const AggArgs &a0, int lpr, int32_t n_coop, hipStream_t st) {
     AggArgs a = a0;
     const int g = 64 / lpr;
@@ -840,7 +862,7 @@ int launch_coop(const AggArgs &a0, int lpr, int32_t n_coop, hipStream_t st) {
     const int64_t grid = n_coop + (a.n_blocks + span - 1) / span * span;
     if (grid == 0) return ROF_OK;
     dim3 gr((unsigned)grid), bl(64 * kCoopWaves);
-#define ROF_LAUNCH(LPR) hipLaunchKernelGGL((rof_coop_kernel<4, LPR, DEEP>), gr, bl, 0, st, a, n_coop)
+#define ROF_LAUNCH(LPR) hipLaunchKernelGGL((rof_coop_kernel<XT, VEC, LPR, DEEP>), gr, bl, 0, st, a, n_coop)
     switch (lpr) {
         case 4: ROF_LAUNCH(4); break;
         case 8: ROF_LAUNCH(8); break;
@@ -858,16 +880,17 @@ int launch_coop(const AggArgs &a0, int lpr, int32_t n_coop, hipStream_t st) {
 
 // Instantiated in agg_rows_{f32,bf16}_partial.hip (partial-sum launches; phase 0, 3 or 5 / stream: phase 3), agg_rows_{f32,bf16}_dst.hip (destination
 // rows; phase 1, or 2 = streaming stores), agg_cluster_{f32,bf16}.hip (the clustered destination rows: a.n_blocks
-// clusters whose workgroups need lds_rows LDS rows) and agg_coop_f32.hip (the destination rows of a small graph), one
+// clusters whose workgroups need lds_rows LDS rows) and agg_coop_{f32,bf16}.hip (the destination rows of a small graph), one
 // translation unit each so that the build runs them side by side.
 // off32: every byte offset into the feature matrix and into the partial-sum workspace fits 32 bits and
 // every row id fits 24 bits, so the kernels may use the short address arithmetic.
 int launch_rows_f32_partial(const AggArgs &a, int phase, int vec, bool off32, hipStream_t st);
 int launch_rows_f32_dst(const AggArgs &a, int phase, int vec, bool off32, hipStream_t st);
 int launch_rows_f32_cluster(const AggArgs &a, int phase, int vec, bool off32, int lds_rows, hipStream_t st);
-// agg_coop_f32.hip: the destination-row launch of a small graph whose first n_coop tasks get a workgroup each
-// (rof_coop_kernel; fp32 rows gathered as 16-byte vectors with short offsets); a.n_tasks: the tasks of this launch
+// agg_coop_{f32,bf16}.hip: the destination-row launch of a small graph whose first n_coop tasks get a workgroup each
+// (rof_coop_kernel; rows gathered as 16-byte vectors with short offsets); a.n_tasks: the tasks of this launch
 int launch_rows_f32_coop(const AggArgs &a, bool deep, int32_t n_coop, hipStream_t st);
+int launch_rows_bf16_coop(const AggArgs &a, int32_t n_coop, hipStream_t st);
 int launch_rows_bf16_partial(const AggArgs &a, bool stream, int vec, bool off32, hipStream_t st);
 int launch_rows_bf16_dst(const AggArgs &a, int phase, int vec, bool off32, hipStream_t st);
 int launch_rows_bf16_cluster(const AggArgs &a, int phase, int vec, bool off32, int lds_rows, hipStream_t st);

@@ -530,13 +530,13 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
                                                   : std::max<int32_t>(16, (int64_t)hub_split * rule_segment / rule_cut);
     L->hub_split = hub_split;
     L->segment = segment;
-    // Small launches (fp32 rows, the library's own cut): no row is cut.  The destination-row launch runs workgroups of
+    // Small launches (the library's own cut): no row is cut.  The destination-row launch runs workgroups of
     // 16 wavefronts and gives every row of more than kCoopRow entries a whole workgroup, whose wavefronts each sum a
     // sixteenth of it and combine in LDS: the chain of dependent gathers of a segment without the second launch that
     // segments need (2^14 nodes x 32 floats: two launches of 5-6 us each).  Only while the longest row leaves a lane
     // group at most kCoopChain entries; a longer one is better off spread over the machine in segments.
     bool coop = false;
-    if (!(o && (o->hub_split > 0 || o->segment > 0 || o->share_scope == 1)) && elem_bytes == 4 && n / groups < kWavesToFill) {
+    if (!(o && (o->hub_split > 0 || o->segment > 0 || o->share_scope == 1)) && n / groups < kWavesToFill) {
         int32_t longest = 0;
         int64_t long_rows = 0;
         for (int32_t v = 0; v < n; ++v) {

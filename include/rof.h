@@ -140,7 +140,7 @@ typedef struct {
                              /* G = 4; 640 from 5 on; bfloat16 rows 256 for G <= 2, 512 at 3, 1280 above; lower     */
                              /* (down to 128) on launches so small that a row of that length would outlast them,   */
                              /* and adjusted on dense graphs by what their rows look like (see layout.cpp).  With    */
-                             /* 0 here and in `segment`, a small graph of float32 rows (fewer than 16 384 wavefronts */
+                             /* 0 here and in `segment`, a small graph (fewer than 16 384 wavefronts                 */
                              /* of rows, at most 256 rows beyond 256 entries, none beyond 1536 per row that a        */
                              /* wavefront gathers at once) keeps its long rows whole: the destination-row launch then */
                              /* sums each of them with a workgroup of 16 wavefronts, and there is no earlier launch  */

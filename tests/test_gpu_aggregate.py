@@ -181,6 +181,35 @@ def test_long_rows_of_small_graphs_are_summed_by_a_workgroup_each(oracle, scale_
     cut.close()
 
 
+@pytest.mark.parametrize("feat,opts", [(32, {}), (128, {}), (256, {}), (72, {}), (41, {}), (64, dict(min_consumers=2))])
+def test_long_rows_of_small_graphs_with_bf16_features(oracle, feat, opts):
+    """The same launch for bf16 rows (8 values per lane, fp32 sums); 41 columns are rows of 82 bytes, which only scalar
+    loads can read: the ordinary kernel then sums the uncut rows."""
+    indptr, indices, plan = _case("c1", 0, 3)
+    n = len(indptr) - 1
+    deg = np.diff(indptr).astype(np.float32)
+    xb = torch.from_numpy(features(n, feat, seed=23, kind="uniform")).to(torch.bfloat16)
+    x = xb.to(torch.float32).numpy()                         # the oracle sees the bf16-rounded values
+    lay = _layout(plan, n, 3, lanes_per_row=lanes_per_row(feat, True), elem_bytes=2, **opts)
+    st = lay.stats()
+    assert st["workgroup_rows"] > 0 and st["hub_segments"] == 0, st
+    cut = _layout(plan, n, 3, lanes_per_row=lanes_per_row(feat, True), elem_bytes=2, hub_split=st["hub_split"],
+                  segment=st["segment"], **opts)
+    assert cut.stats()["workgroup_rows"] == 0 and cut.stats()["hub_segments"] > 0
+    d = torch.from_numpy(deg).cuda()
+    lay.set_degrees(d)
+    cut.set_degrees(d)
+    want = oracle.closed_form(indptr, indices, x, deg)
+    mag = oracle.closed_form(indptr, indices, np.abs(x), deg)
+    got = lay.aggregate(xb.cuda(), normalized=True)
+    _close(got.cpu().numpy(), want, mag)                      # the fp32 bar: the products of the rounded inputs are exact
+    _close(cut.aggregate(xb.cuda(), normalized=True).cpu().numpy(), want, mag)
+    half = lay.aggregate(xb.cuda(), normalized=True, out_dtype=torch.bfloat16, relu=True)
+    assert torch.equal(half, torch.relu(got).to(torch.bfloat16))
+    lay.close()
+    cut.close()
+
+
 @pytest.mark.parametrize("feat,ld,shift", [(47, 47, 0), (5, 5, 0), (7, 9, 1), (101, 101, 3), (255, 255, 0), (2, 2, 1)])
 def test_packed_and_misaligned_rows(oracle, feat, ld, shift):
     """Rows that start on arbitrary 4-byte boundaries (packed widths, odd strides, an offset base pointer):

@@ -384,7 +384,7 @@ def test_small_launches_cut_long_rows_lower():
 
 
 def test_small_graphs_keep_long_rows_whole_for_a_workgroup_each():
-    """A small launch (fp32 rows, the library's own cut) with at most 256 rows of more than 256 entries, the longest of
+    """A small launch (the library's own cut) with at most 256 rows of more than 256 entries, the longest of
     at most 16 x 96 entries per lane group, keeps those rows whole: they lead the task list (longest first) and the
     launch gives each a workgroup of sixteen wavefronts.  No segment, no partial row, no second launch; the cut the
     rule would have used is still reported."""
@@ -399,8 +399,9 @@ def test_small_graphs_keep_long_rows_whole_for_a_workgroup_each():
     assert sorted(ex["b_task_out"][:106].tolist()) == sorted(np.nonzero(deg > 256)[0].tolist())
     # every entry of every row is still there
     assert len(ex["b_col"]) == len(ix) and st["gathered_rows"] == len(ix)
-    # a caller's cut, bf16 rows, or a scope that needs segments: the segments stay
-    for kw in (dict(hub_split=256), dict(segment=64), dict(elem_bytes=2), dict(share_scope="long_rows")):
+    assert Layout.from_csr(ip, ix, lanes_per_row=8, elem_bytes=2).stats()["workgroup_rows"] == 106     # bf16 rows alike
+    # a caller's cut or a scope that needs segments: the segments stay
+    for kw in (dict(hub_split=256), dict(segment=64), dict(share_scope="long_rows")):
         st = Layout.from_csr(ip, ix, lanes_per_row=8, **kw).stats()
         assert st["workgroup_rows"] == 0 and st["hub_segments"] > 0, kw
     # one row per wavefront: 2^14 rows are no small launch, and 2486 entries would be 155 per lane group
