@@ -4,8 +4,8 @@
 
 namespace rofk {
 
-int launch_rows_bf16_coop(const AggArgs &a, int32_t n_coop, hipStream_t st) {
-    return launch_coop<uint16_t, 8, false>(a, rof_lanes_per_row(a.feat, 8), n_coop, st);
+int launch_rows_bf16_coop(const AggArgs &a, const CoopSplit &cs, hipStream_t st) {
+    return launch_coop<uint16_t, 8, false>(a, rof_lanes_per_row(a.feat, 8), cs, st);
 }
 
 }  // namespace rofk

@@ -4,9 +4,9 @@
 
 namespace rofk {
 
-int launch_rows_f32_coop(const AggArgs &a, bool deep, int32_t n_coop, hipStream_t st) {
+int launch_rows_f32_coop(const AggArgs &a, bool deep, const CoopSplit &cs, hipStream_t st) {
     const int lpr = rof_lanes_per_row(a.feat, 4);
-    return deep ? launch_coop<float, 4, true>(a, lpr, n_coop, st) : launch_coop<float, 4, false>(a, lpr, n_coop, st);
+    return deep ? launch_coop<float, 4, true>(a, lpr, cs, st) : launch_coop<float, 4, false>(a, lpr, cs, st);
 }
 
 }  // namespace rofk

@@ -624,11 +624,13 @@ static int aggregate_impl(const rof_layout *L, const void *x, int x_dtype, int64
         // a small graph whose layout keeps long rows whole: one launch in which a workgroup of 16 wavefronts sums each
         // of them (the kernel exists for rows gathered as 16-byte vectors with short offsets; any other call runs the
         // ordinary kernel, which sums such a row with one wavefront)
-        if (L->coop_tasks > 0 && vec == wide && off32 && phase != 2)
-            rc = x_dtype == ROF_F32 ? rofk::launch_rows_f32_coop(a, phase == 4, L->coop_tasks, st)
-                                    : rofk::launch_rows_bf16_coop(a, L->coop_tasks, st);
-        else
+        if (L->coop_tasks > 0 && vec == wide && off32 && phase != 2) {
+            const rofk::CoopSplit cs = {L->coop16, L->coop8, L->coop_tasks - L->coop16 - L->coop8};
+            rc = x_dtype == ROF_F32 ? rofk::launch_rows_f32_coop(a, phase == 4, cs, st) : rofk::launch_rows_bf16_coop(a, cs, st);
+        } else
+        {
             rc = rofk::launch_rows(x_dtype != ROF_F32, a, phase, vec, off32, 0, st);
+        }
         if (rc) return rc;
         a.wave_cap = 0;
         if (L->db.lg_blocks > 0) {

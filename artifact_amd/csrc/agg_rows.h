@@ -604,15 +604,21 @@ __global__ __launch_bounds__(256) void rof_cluster_kernel(AggArgs a) {
 // The destination-row launch of a small graph (fp32 rows, short offsets).  A launch that cannot fill the machine lasts
 // as long as its longest chain of dependent gathers, and cutting long rows into segments shortens that chain only at
 // the price of a second, dependent launch (a quarter to a half of the whole on graphs of 2^14 ... 2^16 nodes).  Here
-// the workgroups are 16 wavefronts wide and the first n_coop of them take one long row each (the layout puts the
-// longest tasks first): every wavefront sums a sixteenth of the row's entries, the sixteen sums meet in LDS, and the
-// first wavefront adds them up and stores the row -- the chain of a segment, no partial row through memory and no
-// second launch.  The other workgroups run the remaining tasks exactly like rof_rows_kernel, sixteen wavefronts each.
+// the workgroups are 16 wavefronts wide and the first of them take the long rows (the layout puts the longest tasks
+// first): the n16 longest get a workgroup each, the next n8 share one between two (8 wavefronts a row), the next n4
+// between four.  Every wavefront sums its share of the row's entries, the sums meet in LDS, and the row's first
+// wavefront adds them up and stores the row -- the chain of a segment, no partial row through memory and no second
+// launch.  The other workgroups run the remaining tasks exactly like rof_rows_kernel, sixteen wavefronts each.
 // DEEP: four row gathers in flight per lane group (five at 10 lanes per row) instead of two (fp32 rows).
 constexpr int kCoopWaves = 16;
+struct CoopSplit {
+    int32_t n16, n8, n4;   // leading tasks that get 16, 8 and 4 wavefronts each
+    __host__ __device__ int32_t tasks() const { return n16 + n8 + n4; }
+    __host__ __device__ int32_t blocks() const { return n16 + (n8 + 1) / 2 + (n4 + 3) / 4; }
+};
 
 template <typename XT, int VEC, int LPR, bool DEEP>
-__global__ __launch_bounds__(64 * kCoopWaves) void rof_coop_kernel(AggArgs a, int32_t n_coop) {
+__global__ __launch_bounds__(64 * kCoopWaves) void rof_coop_kernel(AggArgs a, CoopSplit cs) {
     constexpr int G = 64 / LPR;
     constexpr bool kF32 = sizeof(XT) == 4;   // fp32 features: partial rows have the same element type
     constexpr int kU = DEEP ? (LPR % 4 == 0 ? 4 : LPR % 5 == 0 ? 5 : kGathersInFlight) : kGathersInFlight;
@@ -624,14 +630,30 @@ __global__ __launch_bounds__(64 * kCoopWaves) void rof_coop_kernel(AggArgs a, in
     const uint32_t xld = (uint32_t)(a.ldx * (int64_t)sizeof(XT)), pld = (uint32_t)(a.ldp * 4);
     const int hw = blockIdx.x;
 
-    if (hw < n_coop) {   // one long row, summed by the whole workgroup (no thread leaves before the last barrier)
-        const int32_t t = hw;
-        const int32_t beg = a.task_ptr[t], end = a.task_ptr[t + 1];
-        const int32_t mid = beg + a.task_nref[t];
-        const int32_t out_row = a.task_out[t];
-        const float out_scale = a.task_scale ? a.task_scale[t] : 1.0f;
-        const int32_t share = (end - beg + kCoopWaves - 1) / kCoopWaves;
-        const int32_t wb = min(end, beg + wid * share), we = min(end, wb + share);
+    const int32_t n_coop = cs.tasks(), coop_blocks = cs.blocks();
+    if (hw < coop_blocks) {   // long rows, summed by 16, 8 or 4 wavefronts each (no thread leaves before the last barrier)
+        int per, first, limit;   // wavefronts per row, the workgroup's first task, end of its class of tasks
+        if (hw < cs.n16) {
+            per = 16, first = hw, limit = cs.n16;
+        } else if (hw < cs.n16 + (cs.n8 + 1) / 2) {
+            per = 8, first = cs.n16 + (hw - cs.n16) * 2, limit = cs.n16 + cs.n8;
+        } else {
+            per = 4, first = cs.n16 + cs.n8 + (hw - cs.n16 - (cs.n8 + 1) / 2) * 4, limit = n_coop;
+        }
+        const int32_t t = first + wid / per;   // this wavefront's row
+        const int wsh = wid % per;             // and its share of it
+        const bool have = t < limit;
+        int32_t beg = 0, end = 0, mid = 0, out_row = 0;
+        float out_scale = 1.0f;
+        if (have) {
+            beg = a.task_ptr[t];
+            end = a.task_ptr[t + 1];
+            mid = beg + a.task_nref[t];
+            out_row = a.task_out[t];
+            if (a.task_scale) out_scale = a.task_scale[t];
+        }
+        const int32_t share = (end - beg + per - 1) / per;
+        const int32_t wb = min(end, beg + wsh * share), we = min(end, wb + share);
         for (int c0 = 0; c0 < a.feat; c0 += LPR * VEC) {
             const int cbase = c0 + li * VEC;
             const bool act = !idle && cbase < a.feat;
@@ -678,14 +700,13 @@ __global__ __launch_bounds__(64 * kCoopWaves) void rof_coop_kernel(AggArgs a, in
                 for (int k = 0; k < VEC; ++k) red[wid][li * VEC + k] = acc[k];
             }
             __syncthreads();
-            if (wid == 0 && act && sub == 0) {
+            if (wsh == 0 && have && act && sub == 0) {
                 float tot[VEC];
 #pragma unroll
-                for (int k = 0; k < VEC; ++k) tot[k] = red[0][li * VEC + k];
+                for (int k = 0; k < VEC; ++k) tot[k] = red[wid][li * VEC + k];
+                for (int w = 1; w < per; ++w) {
 #pragma unroll
-                for (int w = 1; w < kCoopWaves; ++w) {
-#pragma unroll
-                    for (int k = 0; k < VEC; ++k) tot[k] += red[w][li * VEC + k];
+                    for (int k = 0; k < VEC; ++k) tot[k] += red[wid + w][li * VEC + k];
                 }
                 finish_row<XT, VEC, PHASE>(a, out_row, out_scale, end > beg, tot, xb, xld, cstart, skip);
             }
@@ -694,7 +715,7 @@ __global__ __launch_bounds__(64 * kCoopWaves) void rof_coop_kernel(AggArgs a, in
     }
 
     // the remaining tasks: a wavefront each while they are long, a lane group each after that
-    const int hb = hw - n_coop;
+    const int hb = hw - coop_blocks;
     const int xcd = hb % kXcds, nth = hb / kXcds;
     const int run = a.xcd_run;
     const int logical = ((nth / run) * kXcds + xcd) * run + (nth % run);
@@ -851,18 +872,19 @@ int launch_lpr(const AggArgs &a0, int lpr, int lds_rows, hipStream_t st) {
 }
 
 template <typename XT, int VEC, bool DEEP>
-int launch_coop(const AggArgs &a0, int lpr, int32_t n_coop, hipStream_t st) {
+int launch_coop(const AggArgs &a0, int lpr, const CoopSplit &cs, hipStream_t st) {
     AggArgs a = a0;
     const int g = 64 / lpr;
-    if (n_coop < 0 || n_coop > a.n_wave || a.n_wave > a.n_tasks) return ROF_ERR_ARG;
+    const int32_t n_coop = cs.tasks();
+    if (cs.n16 < 0 || cs.n8 < 0 || cs.n4 < 0 || n_coop > a.n_wave || a.n_wave > a.n_tasks) return ROF_ERR_ARG;
     const int64_t waves = (int64_t)(a.n_wave - n_coop) + ((int64_t)a.n_tasks - a.n_wave + g - 1) / g;
     a.n_blocks = (int32_t)((waves + kCoopWaves - 1) / kCoopWaves);
     a.xcd_run = std::max(1, a.xcd_run / (kCoopWaves / kWavesPerBlock));   // runs counted in workgroups four times as wide
     const int64_t span = (int64_t)kXcds * a.xcd_run;
-    const int64_t grid = n_coop + (a.n_blocks + span - 1) / span * span;
+    const int64_t grid = cs.blocks() + (a.n_blocks + span - 1) / span * span;
     if (grid == 0) return ROF_OK;
     dim3 gr((unsigned)grid), bl(64 * kCoopWaves);
-#define ROF_LAUNCH(LPR) hipLaunchKernelGGL((rof_coop_kernel<XT, VEC, LPR, DEEP>), gr, bl, 0, st, a, n_coop)
+#define ROF_LAUNCH(LPR) hipLaunchKernelGGL((rof_coop_kernel<XT, VEC, LPR, DEEP>), gr, bl, 0, st, a, cs)
     switch (lpr) {
         case 4: ROF_LAUNCH(4); break;
         case 8: ROF_LAUNCH(8); break;
@@ -887,10 +909,11 @@ int launch_coop(const AggArgs &a0, int lpr, int32_t n_coop, hipStream_t st) {
 int launch_rows_f32_partial(const AggArgs &a, int phase, int vec, bool off32, hipStream_t st);
 int launch_rows_f32_dst(const AggArgs &a, int phase, int vec, bool off32, hipStream_t st);
 int launch_rows_f32_cluster(const AggArgs &a, int phase, int vec, bool off32, int lds_rows, hipStream_t st);
-// agg_coop_{f32,bf16}.hip: the destination-row launch of a small graph whose first n_coop tasks get a workgroup each
-// (rof_coop_kernel; rows gathered as 16-byte vectors with short offsets); a.n_tasks: the tasks of this launch
-int launch_rows_f32_coop(const AggArgs &a, bool deep, int32_t n_coop, hipStream_t st);
-int launch_rows_bf16_coop(const AggArgs &a, int32_t n_coop, hipStream_t st);
+// agg_coop_{f32,bf16}.hip: the destination-row launch of a small graph whose first cs.tasks() tasks are summed by 16, 8
+// or 4 wavefronts each (rof_coop_kernel; rows gathered as 16-byte vectors with short offsets); a.n_tasks: the tasks
+// of this launch
+int launch_rows_f32_coop(const AggArgs &a, bool deep, const CoopSplit &cs, hipStream_t st);
+int launch_rows_bf16_coop(const AggArgs &a, const CoopSplit &cs, hipStream_t st);
 int launch_rows_bf16_partial(const AggArgs &a, bool stream, int vec, bool off32, hipStream_t st);
 int launch_rows_bf16_dst(const AggArgs &a, int phase, int vec, bool off32, hipStream_t st);
 int launch_rows_bf16_cluster(const AggArgs &a, int phase, int vec, bool off32, int lds_rows, hipStream_t st);

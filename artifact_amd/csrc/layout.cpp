@@ -32,12 +32,16 @@ typedef std::vector<int32_t> ivec;
 // by its longest task instead and keeps the lower cut (16 384 rows: 18 us against 26).
 const int32_t kShortRow = 64, kShortRowSmall = 32;
 const int64_t kWavesToFill = 2 * 8192;   // two rounds of 256 CUs x 32 wavefronts
-// Rows that a whole workgroup sums on small launches: more entries than kCoopRow, at most kCoopMaxRows of them (each
-// takes the 16 wavefronts of a workgroup, kCoopWaves in agg_rows.h: 2^14 nodes x 32 floats, 106 rows beyond 256 entries
+// Rows that several wavefronts of one workgroup sum on small launches: more entries than kCoopRow, at most kCoopMaxRows
+// of them (measured with the 16 wavefronts of a workgroup for every row, kCoopWaves in agg_rows.h: 2^14 nodes x 32 floats, 106 rows beyond 256 entries
 // 6.4 us, 468 beyond 128 entries 9.4, two launches with segments 10.7; 2^16 nodes, 697 rows beyond 256 entries: 26.4 us
 // against 22.5 with segments), the longest of at most kCoopChain entries per lane group (2486 entries at two rows per
 // wavefront, 78 per lane group: 15.7 us against 18.9).
 const int32_t kCoopRow = 256, kCoopWaves = 16, kCoopChain = 96, kCoopMaxRows = 256;
+// Wavefronts per such row: 16 (a whole workgroup) beyond kCoopRow16 entries, 8 beyond kCoopRow8, 4 below (2^15 nodes,
+// 121 long rows, 16 / 32 / 47 floats: 8.2 / 9.1 / 11.2 us with 16 wavefronts for every row, 7.4 / 8.5 / 11.0 with the
+// steps at 1024 and 512 entries, 6.5 / 7.9 / 10.1 at 2048 and 1024; 2^14 nodes: 6.5 / 6.2 / 6.2 at 32 floats).
+const int32_t kCoopRow16 = 2048, kCoopRow8 = 1024;
 // Long rows.  Rows longer than a cut are gathered in segments that fill partial rows one launch earlier, and
 // the segment tasks of all rows run in the order of the highest source id they gather (entries inside a task are
 // listed by descending id): every wavefront in flight then works in the same narrow band of the feature matrix
@@ -531,8 +535,8 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     L->hub_split = hub_split;
     L->segment = segment;
     // Small launches (the library's own cut): no row is cut.  The destination-row launch runs workgroups of
-    // 16 wavefronts and gives every row of more than kCoopRow entries a whole workgroup, whose wavefronts each sum a
-    // sixteenth of it and combine in LDS: the chain of dependent gathers of a segment without the second launch that
+    // 16 wavefronts and gives every row of more than kCoopRow entries 4, 8 or 16 of them, which each sum their share
+    // of it and combine in LDS: the chain of dependent gathers of a segment without the second launch that
     // segments need (2^14 nodes x 32 floats: two launches of 5-6 us each).  Only while the longest row leaves a lane
     // group at most kCoopChain entries; a longer one is better off spread over the machine in segments.
     bool coop = false;
@@ -773,10 +777,14 @@ int build_schedule(rof_layout *L, const rof_layout_opts *o) {
     finalize_phase(tg, 1 << 30, groups, false, L->g);
     finalize_phase(ts, 1 << 30, groups, entry_order == 0, L->s);   // the sweep needs the descending lists
     finalize_phase(tb, tile_rows, groups, false, L->b, &cl);
-    L->coop_tasks = 0;
+    L->coop_tasks = L->coop16 = L->coop8 = 0;
     if (coop)   // the long tasks come first, longest first
-        while (L->coop_tasks < L->b.n_wave && L->b.task_ptr[L->coop_tasks + 1] - L->b.task_ptr[L->coop_tasks] > kCoopRow)
+        while (L->coop_tasks < L->b.n_wave && L->b.task_ptr[L->coop_tasks + 1] - L->b.task_ptr[L->coop_tasks] > kCoopRow) {
+            const int32_t len = L->b.task_ptr[L->coop_tasks + 1] - L->b.task_ptr[L->coop_tasks];
+            L->coop16 += len > kCoopRow16;
+            L->coop8 += len > kCoopRow8 && len <= kCoopRow16;
             ++L->coop_tasks;
+        }
     L->n_local_groups = (int64_t)cl.lg_task_ptr.size() - 1;
     L->lds_reads = lds_reads;
     L->gathered_before_rows = (int64_t)tg.col.size();

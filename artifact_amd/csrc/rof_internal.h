@@ -59,7 +59,8 @@ struct rof_layout {
     rof_phase_host g, s, b;   // g: shared groups; s: segments of long rows (may read g's rows); b: destination rows
     int32_t hub_split = 0, segment = 0;
     int32_t xcd_run = 4;      // consecutive workgroups of the destination-row launch kept on one XCD
-    int32_t coop_tasks = 0;   // small launches: the first this many destination tasks get a workgroup of 16 wavefronts each
+    int32_t coop_tasks = 0;   // small launches: the first this many destination tasks are summed by several wavefronts each,
+    int32_t coop16 = 0, coop8 = 0;   // the first coop16 of them by 16 (a whole workgroup), the next coop8 by 8, the rest by 4
     // launch tuning of the benchmark interface (rof_layout_set_tuning): 0 / -1 = the library's own choice
     int32_t tune_xcd_run_partial = 0, tune_xcd_run_dst = 0, tune_wave_cap = -1, tune_lds_pad = 0, tune_deep = -1;
     bool local_sources = false;   // 35 % of the gathered rows lie within min(max(8192, rows of 4 MB), n / 16) ids of their destination

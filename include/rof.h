@@ -143,7 +143,7 @@ typedef struct {
                              /* 0 here and in `segment`, a small graph (fewer than 16 384 wavefronts                 */
                              /* of rows, at most 256 rows beyond 256 entries, none beyond 1536 per row that a        */
                              /* wavefront gathers at once) keeps its long rows whole: the destination-row launch then */
-                             /* sums each of them with a workgroup of 16 wavefronts, and there is no earlier launch  */
+                             /* sums each with 4, 8 or 16 wavefronts of one workgroup; there is no earlier launch    */
     int32_t segment;         /* entries per segment; 0 = an eighth to a quarter of hub_split (see layout.cpp).  A row  */
                              /* so long that adding up its segments would outlast the launch gets longer ones.    */
     int32_t lanes_per_row;   /* lanes one gathered row occupies in the kernel that will use this layout:   */
@@ -212,7 +212,7 @@ int rof_layout_stats(const rof_layout *layout, int64_t stats[20]);
 /* The first `count` of the counters the library knows (fewer: the rest is dropped; more: zero-filled): the twenty
  * above, then [20] the cut of long rows (hub_split) and [21] the segment length as chosen for this layout, [22] the
  * entries of the longest task of the destination-row launch, [23] the rows that the destination-row launch of a small
- * graph sums with a whole workgroup each (0: long rows are cut into segments as [20] and [21] say). */
+ * graph sums with several wavefronts of one workgroup each (0: long rows are cut into segments as [20] and [21] say). */
 int rof_layout_stats_n(const rof_layout *layout, int64_t *stats, int count);
 
 /* Copy the schedule to the current HIP device (idempotent). */
