@@ -12,7 +12,8 @@
 // schedule has clustered around groups they share, one workgroup per cluster that sums those groups once into LDS
 // before it gathers the cluster's rows (rof_cluster_kernel).  There are no atomics: each output row has one writer.
 // On a small graph the layout keeps long rows whole instead of cutting them into segments, and the destination-row
-// launch is rof_coop_kernel: workgroups of sixteen wavefronts, one per long row (its wavefronts' sums meet in LDS),
+// launch is rof_coop_kernel: workgroups of sixteen wavefronts, the first of which sum one, two or four long rows
+// each (the sums of a row's wavefronts meet in LDS),
 // the others running the remaining tasks as below -- one launch where segments would need two.
 //
 // Mapping to the machine:

@@ -951,7 +951,7 @@ def main():
         "config": {"workload": DESCR[name], "nodes": n, "edges": e, "feat": feat, "row_stride": ld, "out_row_stride": ldo,
                    "output": "padded rows (pad_columns)" if pad else "packed [N, feat], as the operator API returns it",
                    "part_size": ps, "normalized": normalized, "search": args.search},
-        "roofline": roof(1, ("rof_coop_kernel (destination-row launch of a small graph: long rows get a workgroup each)"
+        "roofline": roof(1, ("rof_coop_kernel (destination-row launch of a small graph: long rows get several wavefronts of a workgroup each)"
                              if st.get("workgroup_rows") else "rof_rows_kernel (destination-row launch)"), bytes_b, ms_b),
         # the launch before it (segments of long rows, swept in the order of their source ids): same kernel
         # template, second in duration

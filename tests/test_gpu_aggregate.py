@@ -135,7 +135,7 @@ def test_dense_graphs_and_rows_of_the_whole_graph(oracle, kind, feat, bf16):
                                                   (0, 47, dict(disable_reuse=True))])
 def test_long_rows_of_small_graphs_are_summed_by_a_workgroup_each(oracle, scale_down, feat, opts):
     """On a launch that cannot fill the machine the layout keeps long rows whole and the destination-row launch gives
-    each of them a workgroup of sixteen wavefronts (one launch instead of two): every lane count, rows of more than one
+    each of them sixteen, eight or four wavefronts of one workgroup (one launch instead of two): every lane count, rows of more than one
     chunk of columns, rows that reference partial rows of shared groups, the layer's epilogue, and the same rows through
     the ordinary kernels (the layout with an explicit cut; rows of three floats, which only scalar loads can read and
     the ordinary kernel therefore sums uncut)."""

@@ -386,7 +386,7 @@ def test_small_launches_cut_long_rows_lower():
 def test_small_graphs_keep_long_rows_whole_for_a_workgroup_each():
     """A small launch (the library's own cut) with at most 256 rows of more than 256 entries, the longest of
     at most 16 x 96 entries per lane group, keeps those rows whole: they lead the task list (longest first) and the
-    launch gives each a workgroup of sixteen wavefronts.  No segment, no partial row, no second launch; the cut the
+    launch gives each 16, 8 or 4 wavefronts of one workgroup.  No segment, no partial row, no second launch; the cut the
     rule would have used is still reported."""
     ip, ix = make_workload("c1", 0)                          # 2^14 rows, 106 of them beyond 256 entries, the longest 2486
     deg = np.diff(ip)
