@@ -392,11 +392,15 @@ class Layout:
             if (bias.dtype != torch.float32 or bias.device != x.device or bias.dim() != 1
                     or bias.numel() != (pad or f) or not bias.is_contiguous()):
                 raise ValueError("bias must be a contiguous float32 vector of feat_dim elements on the device of x")
-        ep = _lib.Epilogue(bias.data_ptr() if bias is not None else None, int(bool(relu)),
-                           ROF_BF16 if out.dtype == torch.bfloat16 else ROF_F32, float(self_weight), int(bool(pad)))
+        if bias is None and not relu and out.dtype == torch.float32 and not self_weight and not pad:
+            ep = None                        # the plain aggregation: no epilogue struct to build
+        else:
+            ep = C.byref(_lib.Epilogue(bias.data_ptr() if bias is not None else None, int(bool(relu)),
+                                       ROF_BF16 if out.dtype == torch.bfloat16 else ROF_F32, float(self_weight),
+                                       int(bool(pad))))
         check(_lib.lib().rof_aggregate_epilogue(
             self._h, C.c_void_p(x.data_ptr()), dt, x.stride(0), C.c_void_p(out.data_ptr()), out.stride(0), f,
-            int(bool(normalized)), C.byref(ep), C.c_void_p(workspace.data_ptr()),
+            int(bool(normalized)), ep, C.c_void_p(workspace.data_ptr()),
             workspace.numel() * workspace.element_size(), C.c_void_p(st)))
         return out
 
